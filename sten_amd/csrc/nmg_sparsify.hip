@@ -1,0 +1,524 @@
+// Dense -> grouped n:m compressor (bit-exact with the reference CPU sparsifier), plus the
+// element-wise companions: to_dense scatter, same-pattern gather and the rowpack re-ordering.
+//
+// Reference algorithm (grouped_nm_tensor.py:255-297), per tile of c*g columns x m values:
+//   score[o][p] = sum_j |d[o][order[p][j]]|  (left to right, in the input precision)
+//   sort all (score, o, p) descending (ties: larger o, then larger p)
+//   walk the sorted list; accept (o, p) if column o is free and pattern p has < g members;
+//   the k-th column accepted by pattern p lands in slot p*g + k.
+//
+// GPU formulation (same result, no global sort): the sorted walk always accepts next the
+// largest key among {(o, p): o free, p not full}.  Every free column keeps its "head" = its best
+// key over the patterns that still have room; one step = arg-max of the heads over the free
+// columns, accept it, and if that filled the pattern, recompute the heads that pointed to it.
+// A step is a wavefront (or workgroup) max-reduction; a tile needs c*g steps.
+//
+// Work split: a "team" of TW wavefronts owns one tile; a workgroup holds NT teams that work on
+// NT consecutive tiles, which are adjacent in memory along the sparse dim when that dim is the
+// contiguous one, so the cooperative tile load is coalesced across them.
+#include "nmg_common.h"
+
+namespace nmg {
+
+template <typename T> struct ScoreOf { using type = float; using bits = uint32_t; };
+template <> struct ScoreOf<double> { using type = double; using bits = uint64_t; };
+
+__device__ __forceinline__ uint32_t score_bits(float s) { return __float_as_uint(s); }
+__device__ __forceinline__ uint64_t score_bits(double s) { return (uint64_t)__double_as_longlong(s); }
+
+__device__ __forceinline__ float score_of(float x) { return fabsf(x); }
+__device__ __forceinline__ double score_of(double x) { return fabs(x); }
+__device__ __forceinline__ float score_of(__half x) { return fabsf(__half2float(x)); }
+__device__ __forceinline__ float score_of(__hip_bfloat16 x) { return fabsf(__bfloat162float(x)); }
+
+// Key = (score bits, (o << 16 | p) + 1); the all-zero key means "nothing".
+template <typename SB> struct Key {
+    SB s;
+    uint32_t op;
+};
+template <typename SB> __device__ __forceinline__ bool key_gt(const Key<SB> &a, const Key<SB> &b)
+{
+    return a.s > b.s || (a.s == b.s && a.op > b.op);
+}
+
+__device__ __forceinline__ uint32_t shfl_xor_bits(uint32_t v, int mask)
+{
+    return (uint32_t)__shfl_xor((int)v, mask, 64);
+}
+__device__ __forceinline__ uint64_t shfl_xor_bits(uint64_t v, int mask)
+{
+    uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)v, mask, 64);
+    uint32_t hi = (uint32_t)__shfl_xor((int)(uint32_t)(v >> 32), mask, 64);
+    return ((uint64_t)hi << 32) | lo;
+}
+
+template <typename SB> __device__ __forceinline__ Key<SB> wave_max(Key<SB> k)
+{
+#pragma unroll
+    for (int mask = 32; mask >= 1; mask >>= 1) {
+        Key<SB> o;
+        o.s = shfl_xor_bits(k.s, mask);
+        o.op = shfl_xor_bits(k.op, mask);
+        if (key_gt(o, k)) k = o;
+    }
+    return k;
+}
+
+struct SparsifyParams {
+    const void *dense;
+    void *val;
+    int16_t *idx;
+    const int8_t *order;  // device table [c][n]
+    ViewDev view;
+    int64_t outer;
+    int n, m, g, c, cols;
+    int team_bytes;  // LDS bytes of one team's region
+    int off_hs, off_hp, off_cnt, off_oval, off_oidx, off_wbest;  // offsets inside a team region
+};
+
+template <int TW> __device__ __forceinline__ void team_sync()
+{
+    if (TW == 1) {
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    } else {
+        __syncthreads();
+    }
+}
+
+template <typename T, int TW, int NT>
+__global__ __launch_bounds__(64 * TW * NT) void sparsify_kernel(SparsifyParams P)
+{
+    using CT = typename ScoreOf<T>::type;
+    using SB = typename ScoreOf<T>::bits;
+    constexpr int TS = 64 * TW;  // threads per team
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int n = P.n, m = P.m, g = P.g, c = P.c, cols = P.cols;
+    const int tid = threadIdx.x;
+    const int team = tid / TS, tt = tid % TS;
+    const int wave_in_team = tt / 64;
+
+    // LDS: [order table][team 0 region][team 1 region]...
+    int8_t *s_order = (int8_t *)smem;
+    const int order_bytes = (c * n + 15) & ~15;
+    unsigned char *region = smem + order_bytes + (size_t)team * P.team_bytes;
+    T *s_d = (T *)region;
+    SB *s_hs = (SB *)(region + P.off_hs);
+    uint16_t *s_hp = (uint16_t *)(region + P.off_hp);
+    int16_t *s_cnt = (int16_t *)(region + P.off_cnt);
+    T *s_oval = (T *)(region + P.off_oval);
+    int16_t *s_oidx = (int16_t *)(region + P.off_oidx);
+    Key<SB> *s_wbest = (Key<SB> *)(region + P.off_wbest);
+
+    for (int i = tid; i < c * n; i += 64 * TW * NT) s_order[i] = P.order[i];
+
+    // ---- cooperative load of the NT tiles of this workgroup (zero beyond G / S) ----
+    const int64_t tile0 = (int64_t)blockIdx.x * NT;
+    const T *dense = (const T *)P.dense;
+    const int per_tile = cols * m;
+    for (int e = tid; e < NT * per_tile; e += 64 * TW * NT) {
+        int r = e % m;
+        int rest = e / m;
+        int tm = rest % NT;
+        int o = rest / NT;
+        int64_t t = tile0 + tm;
+        T v = Zero<T>::v();
+        if (t < P.outer) {
+            int64_t tiles_per_b = P.view.num_chunks * P.view.num_blocks;
+            int64_t b = t / tiles_per_b;
+            int64_t rem = t - b * tiles_per_b;
+            int64_t kc = rem / P.view.num_blocks;
+            int64_t mb = rem - kc * P.view.num_blocks;
+            int64_t gi = kc * cols + o, si = mb * m + r;
+            if (gi < P.view.G && si < P.view.S)
+                v = dense[b * P.view.stride_b + gi * P.view.stride_g + si * P.view.stride_s];
+        }
+        T *dst = (T *)(smem + order_bytes + (size_t)tm * P.team_bytes);
+        dst[o * m + r] = v;
+    }
+    for (int p = tt; p < c; p += TS) s_cnt[p] = 0;
+    __syncthreads();
+
+    // Best key of column o over the patterns that still have room (skip_p = pattern that just
+    // filled up and whose counter may not be visible yet).
+    auto head_of = [&](int o, int skip_p, SB &best_s, int &best_p) {
+        best_p = -1;
+        best_s = 0;
+        const T *col = s_d + o * m;
+        for (int p = 0; p < c; p++) {
+            if (p == skip_p || s_cnt[p] >= g) continue;
+            CT acc = 0;
+            for (int j = 0; j < n; j++) acc += score_of(col[s_order[p * n + j]]);
+            SB sb = score_bits(acc);
+            if (best_p < 0 || sb >= best_s) {  // ties: larger p wins
+                best_s = sb;
+                best_p = p;
+            }
+        }
+    };
+    auto local_best = [&]() {
+        Key<SB> lb;
+        lb.s = 0;
+        lb.op = 0;
+        for (int o = tt; o < cols; o += TS) {
+            uint16_t hp = s_hp[o];
+            if (hp == 0xFFFF) continue;
+            Key<SB> k;
+            k.s = s_hs[o];
+            k.op = (((uint32_t)o << 16) | hp) + 1u;
+            if (key_gt(k, lb)) lb = k;
+        }
+        return lb;
+    };
+
+    for (int o = tt; o < cols; o += TS) {
+        SB bs;
+        int bp;
+        head_of(o, -1, bs, bp);
+        s_hs[o] = bs;
+        s_hp[o] = (uint16_t)bp;
+    }
+    Key<SB> lb = local_best();
+
+    for (int step = 0; step < cols; step++) {
+        Key<SB> b = wave_max(lb);
+        if (TW > 1) {
+            if ((tt & 63) == 0) s_wbest[wave_in_team] = b;
+            __syncthreads();
+            b = s_wbest[0];
+#pragma unroll
+            for (int w = 1; w < TW; w++) {
+                Key<SB> o = s_wbest[w];
+                if (key_gt(o, b)) b = o;
+            }
+        }
+        const uint32_t op = b.op - 1u;
+        const int o_star = (int)(op >> 16), p_star = (int)(op & 0xFFFFu);
+        const int oldcnt = s_cnt[p_star];
+        team_sync<TW>();
+        bool dirty = false;
+        if (o_star % TS == tt) {
+            const int slot = p_star * g + oldcnt;
+            s_cnt[p_star] = (int16_t)(oldcnt + 1);
+            s_hp[o_star] = 0xFFFF;
+            s_oidx[slot] = (int16_t)o_star;
+            for (int j = 0; j < n; j++) s_oval[slot * n + j] = s_d[o_star * m + s_order[p_star * n + j]];
+            dirty = true;
+        }
+        if (oldcnt + 1 == g) {
+            for (int o = tt; o < cols; o += TS) {
+                if (s_hp[o] != (uint16_t)p_star) continue;
+                SB bs;
+                int bp;
+                head_of(o, p_star, bs, bp);
+                s_hs[o] = bs;
+                s_hp[o] = (uint16_t)bp;
+                dirty = true;
+            }
+        }
+        if (dirty) lb = local_best();
+        team_sync<TW>();
+    }
+
+    // ---- coalesced store of the team's tile ----
+    __syncthreads();
+    const int64_t t = tile0 + team;
+    if (t < P.outer) {
+        T *val = (T *)P.val + t * (int64_t)cols * n;
+        int16_t *idx = P.idx + t * (int64_t)cols;
+        for (int i = tt; i < cols * n; i += TS) val[i] = s_oval[i];
+        for (int i = tt; i < cols; i += TS) idx[i] = s_oidx[i];
+    }
+}
+
+static inline int align_up(int x, int a) { return (x + a - 1) / a * a; }
+
+template <typename T, int TW, int NT>
+static int launch_sparsify(SparsifyParams &P, hipStream_t stream)
+{
+    using SB = typename ScoreOf<T>::bits;
+    const int cols = P.cols, n = P.n, m = P.m, c = P.c;
+    int off = align_up(cols * m * (int)sizeof(T), 16);
+    P.off_hs = off;
+    off = align_up(off + cols * (int)sizeof(SB), 16);
+    P.off_hp = off;
+    off = align_up(off + cols * 2, 16);
+    P.off_cnt = off;
+    off = align_up(off + c * 2, 16);
+    P.off_oval = off;
+    off = align_up(off + cols * (n > 0 ? n : 1) * (int)sizeof(T), 16);
+    P.off_oidx = off;
+    off = align_up(off + cols * 2, 16);
+    P.off_wbest = off;
+    off = align_up(off + TW * (int)sizeof(Key<SB>), 16);
+    P.team_bytes = off;
+    const size_t lds = (size_t)align_up(c * n, 16) + (size_t)NT * P.team_bytes;
+    NMG_REQUIRE(lds <= 160 * 1024, NMG_ERR_UNSUPPORTED,
+                "sparsify tile (c*g=%d columns, m=%d) needs %zu bytes of LDS, limit 163840", cols,
+                m, lds);
+    auto kern = sparsify_kernel<T, TW, NT>;
+    if (lds > 64 * 1024)
+        NMG_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)lds));
+    const int64_t grid = (P.outer + NT - 1) / NT;
+    NMG_REQUIRE(grid <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "too many tiles (%lld)", (long long)grid);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(64 * TW * NT), lds, stream, P);
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
+template <typename T> static int dispatch_sparsify(SparsifyParams &P, hipStream_t stream)
+{
+    if (P.cols <= 128) return launch_sparsify<T, 1, 4>(P, stream);
+    if (P.cols <= 512) return launch_sparsify<T, 4, 1>(P, stream);
+    return launch_sparsify<T, 16, 1>(P, stream);
+}
+
+static int check_common(const nmg_view *view, int n, int m, int g, int dtype, TileGeom *tg)
+{
+    NMG_REQUIRE(view != nullptr, NMG_ERR_ARG, "null view");
+    NMG_REQUIRE(m >= 1 && m <= 64 && n >= 0 && n <= m && g >= 1, NMG_ERR_ARG,
+                "invalid n:m:g = %d:%d:%d", n, m, g);
+    NMG_REQUIRE(dtype_size(dtype) != 0, NMG_ERR_ARG, "invalid dtype code %d", dtype);
+    NMG_REQUIRE(view->batch >= 0 && view->G >= 0 && view->S >= 0, NMG_ERR_ARG, "negative extent");
+    int64_t c = binom(m, n);
+    NMG_REQUIRE(c * g < 32768, NMG_ERR_ARG,
+                "chunk_size * group_size = %lld must be < 2^15 (int16 indices)", (long long)(c * g));
+    *tg = tile_geom(*view, n, m, g);
+    return NMG_OK;
+}
+
+static ViewDev view_dev(const nmg_view &v, const TileGeom &tg)
+{
+    ViewDev d;
+    d.G = v.G;
+    d.S = v.S;
+    d.stride_b = v.stride_b;
+    d.stride_g = v.stride_g;
+    d.stride_s = v.stride_s;
+    d.num_chunks = tg.num_chunks;
+    d.num_blocks = tg.num_blocks;
+    return d;
+}
+
+// ------------------------------------------------------------------ element-wise companions
+
+struct ScatterParams {
+    const void *val;
+    const int16_t *idx;
+    void *dense;
+    const int8_t *order;
+    ViewDev view;
+    int64_t outer;
+    int n, m, g, c, cols;
+};
+
+// One thread per slot: writes the m values of its column (kept ones + zeros), so every element
+// of the view is written exactly once (idx is a permutation of the tile's columns).
+template <typename T> __global__ void to_dense_kernel(ScatterParams P)
+{
+    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= P.outer * P.cols) return;
+    const int64_t t = gid / P.cols;
+    const int slot = (int)(gid - t * P.cols);
+    const int p = slot / P.g;
+    const int o = P.idx[gid];
+    if (o < 0 || o >= P.cols) return;
+    const int64_t tiles_per_b = P.view.num_chunks * P.view.num_blocks;
+    const int64_t b = t / tiles_per_b;
+    const int64_t rem = t - b * tiles_per_b;
+    const int64_t kc = rem / P.view.num_blocks, mb = rem - kc * P.view.num_blocks;
+    const int64_t gi = kc * P.cols + o;
+    if (gi >= P.view.G) return;
+    const T *v = (const T *)P.val + gid * P.n;
+    T *base = (T *)P.dense + b * P.view.stride_b + gi * P.view.stride_g;
+    int j = 0;
+    for (int r = 0; r < P.m; r++) {
+        T x = Zero<T>::v();
+        if (j < P.n && P.order[p * P.n + j] == r) x = v[j++];
+        const int64_t si = mb * P.m + r;
+        if (si < P.view.S) base[si * P.view.stride_s] = x;
+    }
+}
+
+template <typename T> __global__ void gather_kernel(ScatterParams P)
+{
+    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= P.outer * P.cols) return;
+    const int64_t t = gid / P.cols;
+    const int slot = (int)(gid - t * P.cols);
+    const int p = slot / P.g;
+    const int o = P.idx[gid];
+    const int64_t tiles_per_b = P.view.num_chunks * P.view.num_blocks;
+    const int64_t b = t / tiles_per_b;
+    const int64_t rem = t - b * tiles_per_b;
+    const int64_t kc = rem / P.view.num_blocks, mb = rem - kc * P.view.num_blocks;
+    const int64_t gi = kc * P.cols + o;
+    T *v = (T *)P.val + gid * P.n;  // here val is the output
+    const T *base = (const T *)P.dense + b * P.view.stride_b + gi * P.view.stride_g;
+    for (int j = 0; j < P.n; j++) {
+        const int64_t si = mb * P.m + P.order[p * P.n + j];
+        T x = Zero<T>::v();
+        if (o >= 0 && gi < P.view.G && si < P.view.S) x = base[si * P.view.stride_s];
+        v[j] = x;
+    }
+}
+
+struct RowpackParams {
+    const void *val;
+    const int16_t *idx;
+    void *pk_val;
+    void *pk_pat;
+    int64_t G, nb, num_chunks, outer;
+    int n, g, c, cols, pat_bytes;
+};
+
+template <typename T> __global__ void rowpack_kernel(RowpackParams P)
+{
+    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= P.outer * P.cols) return;
+    const int64_t t = gid / P.cols;
+    const int slot = (int)(gid - t * P.cols);
+    const int p = slot / P.g;
+    const int o = P.idx[gid];
+    const int64_t kc = t / P.nb, mb = t - kc * P.nb;
+    const int64_t q = kc * P.cols + o;
+    if (o < 0 || q >= P.G) return;
+    const T *v = (const T *)P.val + gid * P.n;
+    T *dst = (T *)P.pk_val + (q * P.nb + mb) * P.n;
+    for (int j = 0; j < P.n; j++) dst[j] = v[j];
+    if (P.pat_bytes == 1)
+        ((uint8_t *)P.pk_pat)[q * P.nb + mb] = (uint8_t)p;
+    else
+        ((uint16_t *)P.pk_pat)[q * P.nb + mb] = (uint16_t)p;
+}
+
+}  // namespace nmg
+
+using namespace nmg;
+
+extern "C" int nmg_sparsify(const void *d_dense, const nmg_view *view, void *d_val, int16_t *d_idx,
+                            int n, int m, int g, int dtype, void *stream)
+{
+    TileGeom tg;
+    if (int rc = check_common(view, n, m, g, dtype, &tg)) return rc;
+    if (tg.outer == 0) return NMG_OK;
+    NMG_REQUIRE(d_dense && d_val && d_idx, NMG_ERR_ARG, "null device pointer");
+    SparsifyParams P{};
+    P.dense = d_dense;
+    P.val = d_val;
+    P.idx = d_idx;
+    if (int rc = device_order(n, m, &P.order)) return rc;
+    P.view = view_dev(*view, tg);
+    P.outer = tg.outer;
+    P.n = n;
+    P.m = m;
+    P.g = g;
+    P.c = tg.c;
+    P.cols = tg.cols;
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+    case NMG_F32: return dispatch_sparsify<float>(P, s);
+    case NMG_F16: return dispatch_sparsify<__half>(P, s);
+    case NMG_BF16: return dispatch_sparsify<__hip_bfloat16>(P, s);
+    case NMG_F64: return dispatch_sparsify<double>(P, s);
+    }
+    return NMG_ERR_ARG;
+}
+
+template <template <typename> class K> struct Launch;
+
+static int launch_scatter(bool gather, const void *dense, const nmg_view *view, const void *val,
+                          const int16_t *idx, int n, int m, int g, int dtype, void *stream)
+{
+    TileGeom tg;
+    if (int rc = check_common(view, n, m, g, dtype, &tg)) return rc;
+    if (tg.outer == 0) return NMG_OK;
+    NMG_REQUIRE(dense && val && idx, NMG_ERR_ARG, "null device pointer");
+    ScatterParams P{};
+    P.val = val;
+    P.idx = idx;
+    P.dense = (void *)dense;
+    if (int rc = device_order(n, m, &P.order)) return rc;
+    P.view = view_dev(*view, tg);
+    P.outer = tg.outer;
+    P.n = n;
+    P.m = m;
+    P.g = g;
+    P.c = tg.c;
+    P.cols = tg.cols;
+    const int64_t total = tg.outer * tg.cols;
+    const int bs = 256;
+    const int64_t grid = (total + bs - 1) / bs;
+    NMG_REQUIRE(grid <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "too many slots");
+    hipStream_t s = (hipStream_t)stream;
+#define NMG_LAUNCH(T)                                                                         \
+    do {                                                                                      \
+        if (gather)                                                                           \
+            hipLaunchKernelGGL(gather_kernel<T>, dim3((unsigned)grid), dim3(bs), 0, s, P);    \
+        else                                                                                  \
+            hipLaunchKernelGGL(to_dense_kernel<T>, dim3((unsigned)grid), dim3(bs), 0, s, P);  \
+    } while (0)
+    switch (dtype) {
+    case NMG_F32: NMG_LAUNCH(float); break;
+    case NMG_F16: NMG_LAUNCH(__half); break;
+    case NMG_BF16: NMG_LAUNCH(__hip_bfloat16); break;
+    case NMG_F64: NMG_LAUNCH(double); break;
+    }
+#undef NMG_LAUNCH
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
+extern "C" int nmg_to_dense(const void *d_val, const int16_t *d_idx, void *d_dense,
+                            const nmg_view *view, int n, int m, int g, int dtype, void *stream)
+{
+    return launch_scatter(false, d_dense, view, d_val, d_idx, n, m, g, dtype, stream);
+}
+
+extern "C" int nmg_gather(const void *d_dense, const nmg_view *view, const int16_t *d_idx,
+                          void *d_val, int n, int m, int g, int dtype, void *stream)
+{
+    return launch_scatter(true, d_dense, view, d_val, d_idx, n, m, g, dtype, stream);
+}
+
+extern "C" int64_t nmg_rowpack_pat_bytes(int n, int m) { return binom(m, n) <= 256 ? 1 : 2; }
+
+extern "C" int nmg_rowpack(const void *d_val, const int16_t *d_idx, int64_t G, int64_t S,
+                           void *d_pk_val, void *d_pk_pat, int n, int m, int g, int dtype,
+                           void *stream)
+{
+    nmg_view v{1, G, S, 0, S, 1};
+    TileGeom tg;
+    if (int rc = check_common(&v, n, m, g, dtype, &tg)) return rc;
+    NMG_REQUIRE(dtype != NMG_F64, NMG_ERR_UNSUPPORTED, "rowpack supports f32/f16/bf16");
+    if (tg.outer == 0) return NMG_OK;
+    NMG_REQUIRE(d_val && d_idx && d_pk_val && d_pk_pat, NMG_ERR_ARG, "null device pointer");
+    RowpackParams P{};
+    P.val = d_val;
+    P.idx = d_idx;
+    P.pk_val = d_pk_val;
+    P.pk_pat = d_pk_pat;
+    P.G = G;
+    P.nb = tg.num_blocks;
+    P.num_chunks = tg.num_chunks;
+    P.outer = tg.outer;
+    P.n = n;
+    P.g = g;
+    P.c = tg.c;
+    P.cols = tg.cols;
+    P.pat_bytes = (int)nmg_rowpack_pat_bytes(n, m);
+    const int64_t total = tg.outer * tg.cols;
+    const int bs = 256;
+    const int64_t grid = (total + bs - 1) / bs;
+    NMG_REQUIRE(grid <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "too many slots");
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+    case NMG_F32: hipLaunchKernelGGL(rowpack_kernel<float>, dim3((unsigned)grid), dim3(bs), 0, s, P); break;
+    case NMG_F16: hipLaunchKernelGGL(rowpack_kernel<__half>, dim3((unsigned)grid), dim3(bs), 0, s, P); break;
+    case NMG_BF16: hipLaunchKernelGGL(rowpack_kernel<__hip_bfloat16>, dim3((unsigned)grid), dim3(bs), 0, s, P); break;
+    }
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}

@@ -1,0 +1,131 @@
+"""Sparsifier and operator implementations of the grouped n:m format, registered through the
+STen dispatch API (the reference registers its own in src/sten/grouped_nm/sten_impls.py:13-37
+and :143-174; it has no ``torch.mm``, no backward and no ``SameFormatSparsifier`` entry -- those
+are defined here by dense autograd of the same operators).
+
+``install(api)`` registers everything into any module that exposes the STen registration
+functions: this package's own ``dispatch`` module, or a real ``sten``.
+"""
+import torch
+
+from .tensor import GroupedNMTensor, spmm
+
+
+class GroupedNMSparsifier:
+    """n:m:g magnitude sparsifier.  Reference signature ``(n, m, g)`` (sten_impls.py:13-17); the
+    default orientation is the reference's (n:m blocks along dim -2, grouping along dim -1).
+    ``sparse_dim`` / ``group_dim`` select another one, e.g. ``sparse_dim=-1, group_dim=-2`` puts
+    the n:m blocks along the reduction dim of ``F.linear``."""
+
+    def __init__(self, n, m, g, sparse_dim=-2, group_dim=-1):
+        self.n, self.m, self.g = n, m, g
+        self.sparse_dim, self.group_dim = sparse_dim, group_dim
+
+
+def _masked_weight_grad(weight, lhs_t, rhs):
+    """val-layout gradient: (lhs_t^T @ rhs) gathered at the kept positions of ``weight``."""
+    return weight.clone_layout(torch.mm(lhs_t.t(), rhs))
+
+
+def install(api):
+    KeepAll, SameFormat = api.KeepAll, api.SameFormatSparsifier
+    wrap = api.SparseTensorWrapper.wrapped_from_dense
+    dense_fmt = (KeepAll, torch.Tensor)
+    nmg_fmt = (KeepAll, GroupedNMTensor)
+
+    # ---- sparsifiers -----------------------------------------------------------------------
+    @api.register_sparsifier_implementation(
+        sparsifier=GroupedNMSparsifier, inp=torch.Tensor, out=GroupedNMTensor)
+    def dense_to_grouped_nm(sparsifier, tensor, grad_fmt=None):
+        gnm = GroupedNMTensor.from_dense(
+            tensor, sparsifier.n, sparsifier.m,
+            sparse_dim=getattr(sparsifier, "sparse_dim", -2) % tensor.dim(),
+            group_size=sparsifier.g,
+            group_dim=getattr(sparsifier, "group_dim", -1) % tensor.dim())
+        return wrap(gnm, tensor, grad_fmt)
+
+    @api.register_sparsifier_implementation(
+        sparsifier=SameFormat, inp=torch.Tensor, out=GroupedNMTensor)
+    def dense_to_same_grouped_nm(sparsifier, tensor, grad_fmt=None):
+        ref = sparsifier.ref_sp_ten
+        ref_fmt = ref.wrapped_tensor if hasattr(ref, "wrapped_tensor") else ref
+        return wrap(ref_fmt.clone_layout(tensor), tensor,
+                    grad_fmt if grad_fmt is not None else getattr(ref, "grad_fmt", None))
+
+    @api.register_sparsifier_implementation(
+        sparsifier=KeepAll, inp=GroupedNMTensor, out=api.DenseTensor)
+    def grouped_nm_to_dense_tensor(sparsifier, tensor, grad_fmt=None):
+        dense = tensor.wrapped_tensor.to_dense()
+        return wrap(api.DenseTensor(dense), dense, grad_fmt)
+
+    # ---- F.linear(x, W_nmg[, b]) -----------------------------------------------------------
+    def linear_fwd(ctx, inputs, output_sparsifiers):
+        x, weight = inputs[0], inputs[1]
+        bias = inputs[2] if len(inputs) > 2 else None
+        ctx.save_for_backward(*inputs)
+        w = weight.wrapped_tensor
+        x2 = x.reshape(-1, x.shape[-1])
+        y = spmm(w, x2, bias, reduce_dim=1)
+        return y.reshape(*x.shape[:-1], y.shape[-1])
+
+    def linear_bwd_common(ctx, grad_outputs, compressed):
+        saved = ctx.saved_tensors
+        x, weight = saved[0], saved[1]
+        [gy] = grad_outputs
+        w = weight.wrapped_tensor
+        gy2 = gy.reshape(-1, gy.shape[-1])
+        x2 = x.reshape(-1, x.shape[-1])
+        if gy2.dtype != w.dtype:
+            gy2 = gy2.to(w.dtype)
+        gx = spmm(w, gy2.contiguous(), reduce_dim=0).reshape(x.shape)
+        if compressed:
+            gw = wrap(_masked_weight_grad(w, gy2, x2), x2)
+        else:
+            gw = torch.mm(gy2.t(), x2)
+        grads = [gx, gw]
+        if len(saved) > 2:
+            grads.append(gy2.sum(dim=0))
+        return tuple(grads)
+
+    for arity in (2, 3):
+        fmts = (torch.Tensor, GroupedNMTensor) + (torch.Tensor,) * (arity - 2)
+        api.register_fwd_op_impl(operator=torch.nn.functional.linear, inp=fmts, out=[dense_fmt])(linear_fwd)
+        api.register_bwd_op_impl(
+            operator=torch.nn.functional.linear, grad_out=(torch.Tensor,),
+            grad_inp=(dense_fmt,) * arity, inp=fmts,
+        )(lambda ctx, g, s: linear_bwd_common(ctx, g, compressed=False))
+        api.register_bwd_op_impl(
+            operator=torch.nn.functional.linear, grad_out=(torch.Tensor,),
+            grad_inp=(dense_fmt, nmg_fmt) + (dense_fmt,) * (arity - 2), inp=fmts,
+        )(lambda ctx, g, s: linear_bwd_common(ctx, g, compressed=True))
+
+    # ---- torch.mm(W_nmg, B) -----------------------------------------------------------------
+    @api.register_fwd_op_impl(operator=torch.mm, inp=(GroupedNMTensor, torch.Tensor), out=[dense_fmt])
+    def mm_fwd(ctx, inputs, output_sparsifiers):
+        weight, b = inputs
+        ctx.save_for_backward(weight, b)
+        return spmm(weight.wrapped_tensor, b.t().contiguous(), reduce_dim=1).t()
+
+    def mm_bwd_common(ctx, grad_outputs, compressed):
+        weight, b = ctx.saved_tensors
+        [gc] = grad_outputs
+        w = weight.wrapped_tensor
+        gc = gc.to(w.dtype)
+        gb = spmm(w, gc.t().contiguous(), reduce_dim=0).t()
+        if compressed:
+            gw = wrap(_masked_weight_grad(w, gc.t(), b.t()), gc)
+        else:
+            gw = torch.mm(gc, b.t())
+        return gw, gb
+
+    api.register_bwd_op_impl(
+        operator=torch.mm, grad_out=(torch.Tensor,), grad_inp=(dense_fmt, dense_fmt),
+        inp=(GroupedNMTensor, torch.Tensor),
+    )(lambda ctx, g, s: mm_bwd_common(ctx, g, compressed=False))
+    api.register_bwd_op_impl(
+        operator=torch.mm, grad_out=(torch.Tensor,), grad_inp=(nmg_fmt, dense_fmt),
+        inp=(GroupedNMTensor, torch.Tensor),
+    )(lambda ctx, g, s: mm_bwd_common(ctx, g, compressed=True))
+
+    return {"dense_to_grouped_nm": dense_to_grouped_nm,
+            "dense_to_same_grouped_nm": dense_to_same_grouped_nm}

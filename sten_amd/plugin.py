@@ -1,0 +1,32 @@
+"""Install the MI355X grouped n:m implementations into a real STen installation.
+
+    import sten, sten_amd.plugin
+    sten_amd.plugin.register(sten)
+
+replaces STen's CPU/CUDA ``GroupedNMTensor`` sparsifier and ``F.linear`` implementation
+(src/sten/grouped_nm/sten_impls.py:20-37, :143-174) with the HIP ones and adds ``torch.mm``, the
+backward implementations and the ``SameFormatSparsifier`` entry.  STen refuses a second
+registration of a sparsifier key (sten.py:1096-1100), so existing keys are removed first.
+"""
+import torch
+
+from . import impls
+from .tensor import GroupedNMTensor
+
+
+def register(sten_module):
+    reg = getattr(sten_module, "SPARSIFIER_IMPLEMENTATIONS", None)
+    if reg is None and hasattr(sten_module, "sten"):
+        reg = sten_module.sten.SPARSIFIER_IMPLEMENTATIONS
+    keys = [
+        (impls.GroupedNMSparsifier, torch.Tensor, GroupedNMTensor),
+        (sten_module.SameFormatSparsifier, torch.Tensor, GroupedNMTensor),
+        (sten_module.KeepAll, GroupedNMTensor, sten_module.DenseTensor),
+    ]
+    for key in keys:
+        if reg is not None and key in reg:
+            sten_module.unregister_sparsifier_implementation(*key)
+    # expose the GPU classes under the names user code already uses
+    sten_module.GroupedNMTensor = GroupedNMTensor
+    sten_module.GroupedNMSparsifier = impls.GroupedNMSparsifier
+    return impls.install(sten_module)

@@ -1,0 +1,229 @@
+"""``GroupedNMTensor`` -- the grouped n:m container, API-compatible with the reference class
+(src/sten/grouped_nm/grouped_nm_tensor.py:877-958: ``val``, ``idx``, ``nm_strides``,
+``from_dense``, ``to_dense``, ``set_spmm_opt``) and extended with what a wrapped format needs on
+a GPU: ``dtype`` / ``device`` / ``shape`` / ``to``, same-pattern re-compression
+(the disabled ``clone_layout``, :904-951) and in-place ``add_`` / ``mul_`` for optimizers.
+
+All compute goes through libnmg_hip.so; tensors must live on the GPU.
+"""
+import ctypes
+
+import torch
+
+from . import native
+from .layout import NMGLayout, bgs_view
+
+
+class GroupedNMTensor:
+    def __init__(self, val, idx, layout):
+        if isinstance(layout, dict):  # accept the reference's nm_strides dict
+            layout = NMGLayout(tuple(layout["dense_shape"]), layout["n"], layout["m"],
+                               layout["group_size"], layout["sparse_dim"], layout["group_dim"])
+        self.val = val
+        self.idx = idx
+        self.layout = layout
+        self.spmm_opt = {"kernel": "auto"}
+        self._rowpack = None
+
+    # ---- construction ----------------------------------------------------------------------
+    @staticmethod
+    def from_dense(tensor, n, m, sparse_dim, group_size, group_dim):
+        """Per-tile magnitude selection, bit-exact with the reference CPU sparsifier
+        (grouped_nm_tensor.py:883-890 -> :701-710 -> :255-297)."""
+        native.require_gpu(tensor)
+        sparse_dim %= tensor.dim()
+        group_dim %= tensor.dim()
+        lay = NMGLayout(tuple(tensor.shape), n, m, group_size, sparse_dim, group_dim)
+        t = tensor.detach()
+        q, view = bgs_view(t, lay)
+        val = torch.empty(lay.val_shape, dtype=t.dtype, device=t.device)
+        idx = torch.empty(lay.idx_shape, dtype=torch.int16, device=t.device)
+        with torch.cuda.device(t.device):
+            native.check(native.load().nmg_sparsify(
+                native.ptr(q), ctypes.byref(view), native.ptr(val), native.ptr(idx),
+                n, m, group_size, native.dtype_code(t.dtype), native.stream_ptr(t.device)))
+        return GroupedNMTensor(val, idx, lay)
+
+    def clone_layout(self, dense_tensor):
+        """New tensor with this tensor's pattern and the values of ``dense_tensor`` at the kept
+        positions (what grouped_nm_tensor.py:908-951 describes)."""
+        if tuple(dense_tensor.shape) != tuple(self.layout.dense_shape):
+            raise ValueError(
+                f"Shape mismatch: expected {self.layout.dense_shape}, received {tuple(dense_tensor.shape)}")
+        native.require_gpu(dense_tensor, self.val)
+        lay = self.layout
+        t = dense_tensor.detach().to(dtype=self.val.dtype)
+        q, view = bgs_view(t, lay)
+        val = torch.empty_like(self.val)
+        with torch.cuda.device(t.device):
+            native.check(native.load().nmg_gather(
+                native.ptr(q), ctypes.byref(view), native.ptr(self.idx), native.ptr(val),
+                lay.n, lay.m, lay.group_size, native.dtype_code(val.dtype),
+                native.stream_ptr(t.device)))
+        out = GroupedNMTensor(val, self.idx, lay)
+        out.spmm_opt = dict(self.spmm_opt)
+        return out
+
+    # ---- reference-compatible surface ------------------------------------------------------------
+    @property
+    def nm_strides(self):
+        d = self.layout.as_nm_strides()
+        d.update(self.spmm_opt)
+        return d
+
+    def set_spmm_opt(self, tile_a=None, acc_width=None, tile_b=None, kernel=None):
+        """Reference signature (grouped_nm_tensor.py:892-902).  The CPU tile parameters have no
+        meaning here; ``kernel`` selects the GPU matmul kernel: auto | mfma | smfmac | skinny."""
+        if kernel is not None:
+            if kernel not in native.KERNELS:
+                raise ValueError(f"kernel must be one of {sorted(native.KERNELS)}")
+            self.spmm_opt["kernel"] = kernel
+        for k, v in (("tile_a", tile_a), ("acc_width", acc_width), ("tile_b", tile_b)):
+            if v is not None:
+                self.spmm_opt[k] = v
+
+    def to_dense(self):
+        lay = self.layout
+        native.require_gpu(self.val)
+        out = torch.empty(lay.dense_shape, dtype=self.val.dtype, device=self.val.device)
+        q, view = bgs_view(out, lay)
+        aliased = q.untyped_storage().data_ptr() == out.untyped_storage().data_ptr()
+        with torch.cuda.device(out.device):
+            native.check(native.load().nmg_to_dense(
+                native.ptr(self.val), native.ptr(self.idx), native.ptr(q), ctypes.byref(view),
+                lay.n, lay.m, lay.group_size, native.dtype_code(out.dtype),
+                native.stream_ptr(out.device)))
+        if not aliased:
+            sizes = [lay.dense_shape[d] for d in lay.other_dims] + [lay.G, lay.S]
+            perm = lay.other_dims + [lay.group_dim, lay.sparse_dim]
+            inv = sorted(range(len(perm)), key=lambda i: perm[i])
+            out = q.view(sizes).permute(inv).contiguous()
+        return out
+
+    # ---- tensor-like attributes the wrapper machinery looks for -------------------------------
+    @property
+    def dtype(self):
+        return self.val.dtype
+
+    @property
+    def device(self):
+        return self.val.device
+
+    @property
+    def shape(self):
+        return torch.Size(self.layout.dense_shape)
+
+    def size(self, dim=None):
+        return self.shape if dim is None else self.shape[dim]
+
+    def dim(self):
+        return len(self.layout.dense_shape)
+
+    def numel(self):
+        return self.shape.numel()
+
+    def to(self, device=None, dtype=None, non_blocking=False, copy=False, **_):
+        val = self.val.to(device=device, dtype=dtype, non_blocking=non_blocking, copy=copy)
+        idx = self.idx.to(device=device, non_blocking=non_blocking, copy=copy)
+        out = GroupedNMTensor(val, idx, self.layout)
+        out.spmm_opt = dict(self.spmm_opt)
+        return out
+
+    def clone(self):
+        return self.to(copy=True)
+
+    # ---- in-place updates that keep the pattern (used by optimizers) ------------------------
+    def _other_val(self, other):
+        if isinstance(other, GroupedNMTensor):
+            if other.layout != self.layout:
+                raise ValueError("layout mismatch")
+            return other.val
+        if hasattr(other, "wrapped_tensor"):
+            return self._other_val(other.wrapped_tensor)
+        if hasattr(other, "to_dense") and not isinstance(other, torch.Tensor):
+            other = other.to_dense()
+        if isinstance(other, torch.Tensor) and other.dim() > 0:
+            return self.clone_layout(other).val
+        return other
+
+    def add_(self, other, *, alpha=1):
+        self.val.add_(self._other_val(other), alpha=alpha)
+        self._rowpack = None
+        return self
+
+    def mul_(self, other):
+        self.val.mul_(self._other_val(other))
+        self._rowpack = None
+        return self
+
+    def zero_(self):
+        self.val.zero_()
+        self._rowpack = None
+        return self
+
+    def copy_(self, other):
+        self.val.copy_(self._other_val(other))
+        self._rowpack = None
+        return self
+
+    # ---- matmul operand ---------------------------------------------------------------------------
+    def rowpack(self):
+        """(pk_val [G, nb, n], pk_pat [G, nb]) -- per line of the group dim and block of the
+        sparse dim, the kept values and the pattern number; cached until ``val`` changes."""
+        lay = self.layout
+        if len(lay.dense_shape) != 2:
+            raise native.NmgError("matmul needs a 2-D grouped n:m tensor")
+        key = (self.val.data_ptr(), self.val._version, self.idx.data_ptr())
+        if self._rowpack is None or self._rowpack[0] != key:
+            native.require_gpu(self.val)
+            lib = native.load()
+            pat_bytes = lib.nmg_rowpack_pat_bytes(lay.n, lay.m)
+            pk_val = torch.empty((lay.G, lay.num_blocks, lay.n), dtype=self.val.dtype, device=self.val.device)
+            pk_pat = torch.empty((lay.G, lay.num_blocks),
+                                 dtype=torch.uint8 if pat_bytes == 1 else torch.int16,
+                                 device=self.val.device)
+            with torch.cuda.device(self.val.device):
+                native.check(lib.nmg_rowpack(
+                    native.ptr(self.val), native.ptr(self.idx), lay.G, lay.S, native.ptr(pk_val),
+                    native.ptr(pk_pat), lay.n, lay.m, lay.group_size,
+                    native.dtype_code(self.val.dtype), native.stream_ptr(self.val.device)))
+            self._rowpack = (key, pk_val, pk_pat)
+        return self._rowpack[1], self._rowpack[2]
+
+    def __repr__(self):
+        lay = self.layout
+        return (f"GroupedNMTensor(shape={tuple(lay.dense_shape)}, n:m:g={lay.n}:{lay.m}:{lay.group_size}, "
+                f"sparse_dim={lay.sparse_dim}, group_dim={lay.group_dim}, dtype={self.val.dtype}, "
+                f"device={self.val.device})")
+
+
+def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
+    """Y = X @ op(W) for a 2-D ``GroupedNMTensor`` W of shape [R, C].
+
+    ``reduce_dim=1``: X is [T, C], Y = X @ W^T is [T, R]  (F.linear forward).
+    ``reduce_dim=0``: X is [T, R], Y = X @ W   is [T, C]  (gradient w.r.t. the input).
+    """
+    lay = weight.layout
+    native.require_gpu(x, weight.val, bias)
+    if x.dtype != weight.val.dtype:
+        raise native.NmgError(f"dtype mismatch: activations {x.dtype}, weight {weight.val.dtype}")
+    pk_val, pk_pat = weight.rowpack()
+    reduce_sparse = 1 if reduce_dim == lay.sparse_dim else 0
+    K = lay.dense_shape[reduce_dim]
+    O = lay.dense_shape[1 - reduce_dim]
+    if x.dim() != 2 or x.shape[1] != K:
+        raise native.NmgError(f"activations must be [tokens, {K}], got {tuple(x.shape)}")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    T = x.shape[0]
+    y = torch.empty((T, O), dtype=x.dtype, device=x.device)
+    if bias is not None:
+        bias = bias.to(dtype=x.dtype).contiguous()
+    kname = kernel or weight.spmm_opt.get("kernel", "auto")
+    with torch.cuda.device(x.device):
+        native.check(native.load().nmg_spmm(
+            native.ptr(pk_val), native.ptr(pk_pat), lay.G, lay.S, native.ptr(x),
+            x.stride(0) if T > 1 else K, native.ptr(y), O, native.ptr(bias), T, reduce_sparse,
+            lay.n, lay.m, native.dtype_code(x.dtype), native.KERNELS[kname],
+            native.stream_ptr(x.device)))
+    return y
