@@ -1,0 +1,121 @@
+"""Benchmark of the nmg sparse x dense matmul on one MI355X.
+
+Workload (BASELINE config 2): fp16 weight 4096x4096 ~ N(0, 0.02), grouped 2:4 (group 16) along
+the reduction dim; fp16 activations 2048 tokens x 4096 ~ N(0,1); forward only, fp32 accumulate.
+A "step" is one nmg x dense matmul over that batch with every operand resident in HBM.
+
+Prints one JSON line: value = dense-equivalent TFLOP/s (2*M*K*N / time); roofline.achieved uses
+the effective (non-zero) flops 2*M*K*N*n/m against the dense fp16 MFMA peak, i.e. the fraction
+of the density-scaled roofline.  cpu_baseline = the CPU restatement of the reference's
+AVX/OpenMP kernel (oracle/nmg_cpu_simd.cpp) on the host cores, same shape, fp32.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+
+def cpu_baseline(M, K, N, n, m, g, seconds=15.0):
+    import numpy as np
+    from oracle import nmg_oracle as O
+    rng = np.random.default_rng(0)
+    # bounded sample: the reference kernel works on fp32 with the n:m blocks along M; a slab of
+    # M_s rows of the same weight shape keeps the per-row work identical
+    M_s = min(M, 1024)
+    W = (rng.standard_normal((M_s, K)) * 0.02).astype(np.float32)
+    X = rng.standard_normal((K, N)).astype(np.float32)
+    val, idx, lay = O.sparsify(W, n, m, 0, g, 1)
+    O.simd_spmm(val, idx, lay, X)
+    t0 = time.perf_counter()
+    it = 0
+    while True:
+        O.simd_spmm(val, idx, lay, X)
+        it += 1
+        if time.perf_counter() - t0 > seconds or it >= 50:
+            break
+    dt = (time.perf_counter() - t0) / it
+    info = O.simd_info()
+    return {
+        "value": 2.0 * M_s * K * N / dt / 1e12,
+        "unit": "TFLOP/s dense-equiv",
+        "cores": info["threads"],
+        "kind": "port",
+        "sample": f"{M_s}x{K} fp32 slab of the weight x {N} tokens, {it} passes, kernel {info['kernel']}",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--kernel", default="auto")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU; multi-GPU runs are not part of this build", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import sten_amd as sten
+
+    dev = "cuda:0"
+    M, K, N, n, m, g = 4096, 4096, 2048, 2, 4, 16
+    torch.manual_seed(0)
+    W = (torch.randn(M, K) * 0.02).half().to(dev)
+    X = torch.randn(N, K).half().to(dev)
+    w = sten.GroupedNMTensor.from_dense(W, n, m, sparse_dim=1, group_size=g, group_dim=0)
+    w.rowpack()
+    for _ in range(args.warmup):
+        y = sten.spmm(w, X, reduce_dim=1, kernel=args.kernel)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        y = sten.spmm(w, X, reduce_dim=1, kernel=args.kernel)
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / args.steps
+
+    # per-launch kernel time with events on the stream the kernel is launched on
+    stream = torch.cuda.current_stream()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+           for _ in range(args.steps)]
+    for a, b in evs:
+        a.record(stream)
+        sten.spmm(w, X, reduce_dim=1, kernel=args.kernel)
+        b.record(stream)
+    torch.cuda.synchronize()
+    kern_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+
+    dense_flops = 2.0 * M * K * N
+    eff_flops = dense_flops * n / m
+    achieved = eff_flops / (kern_ms * 1e-3) / 1e12
+    out = {
+        "metric": "nmg sparse x dense GEMM TFLOP/s (dense-equiv)",
+        "value": dense_flops / wall / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "configs[1]: W 4096x4096 fp16 2:4:16 along K x 2048 tokens, forward",
+                   "kernel": args.kernel, "effective_tflops": eff_flops / wall / 1e12,
+                   "kernel_ms": kern_ms},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS, "traffic": None,
+                     "flops": "effective non-zero (2*M*K*N*n/m)"},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(M, K, N, n, m, g)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

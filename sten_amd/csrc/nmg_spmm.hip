@@ -272,6 +272,13 @@ extern "C" int nmg_spmm(const void *d_pk_val, const void *d_pk_pat, int64_t G, i
                 "unknown kernel selector %d", kernel);
     if (G == 0 || S == 0 || T == 0) return NMG_OK;
     NMG_REQUIRE(d_pk_val && d_pk_pat && d_x && d_y, NMG_ERR_ARG, "null device pointer");
+    NMG_REQUIRE(ldx >= (reduce_sparse ? S : G) && ldy >= (reduce_sparse ? G : S), NMG_ERR_ARG,
+                "leading dimension smaller than row length");
+    if (kernel == NMG_KERNEL_AUTO) kernel = (reduce_sparse && T <= 16) ? NMG_KERNEL_SKINNY : NMG_KERNEL_MFMA;
+    if (kernel == NMG_KERNEL_SKINNY)
+        NMG_REQUIRE(reduce_sparse && T <= 16, NMG_ERR_UNSUPPORTED,
+                    "skinny kernel needs reduce_sparse=1 and T <= 16");
+    NMG_REQUIRE(kernel != NMG_KERNEL_SMFMAC, NMG_ERR_UNSUPPORTED, "SMFMAC kernel not available");
     SpmmParams P{};
     P.pk_val = d_pk_val;
     P.pk_pat = d_pk_pat;
@@ -291,12 +298,6 @@ extern "C" int nmg_spmm(const void *d_pk_val, const void *d_pk_pat, int64_t G, i
     P.m = m;
     P.c = (int)binom(m, n);
     P.pat_bytes = (int)nmg_rowpack_pat_bytes(n, m);
-    NMG_REQUIRE(ldx >= P.K && ldy >= P.O, NMG_ERR_ARG, "leading dimension smaller than row length");
-    if (kernel == NMG_KERNEL_AUTO) kernel = (reduce_sparse && T <= 16) ? NMG_KERNEL_SKINNY : NMG_KERNEL_MFMA;
-    if (kernel == NMG_KERNEL_SKINNY)
-        NMG_REQUIRE(reduce_sparse && T <= 16, NMG_ERR_UNSUPPORTED,
-                    "skinny kernel needs reduce_sparse=1 and T <= 16");
-    NMG_REQUIRE(kernel != NMG_KERNEL_SMFMAC, NMG_ERR_UNSUPPORTED, "SMFMAC kernel not available");
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
     case NMG_F32: return launch_spmm<float>(P, reduce_sparse, kernel, s);

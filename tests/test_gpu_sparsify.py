@@ -1,0 +1,114 @@
+"""GPU parity of the compressor and its element-wise companions against the CPU oracle.
+Integer / byte results must be identical; kept values are copies and must match bit for bit."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import sten_amd as sten
+from oracle import nmg_oracle as O
+from helpers import oracle_sparsify, same_bits, seeded, to_np
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def check_parity(x_cpu, n, m, sd, g, gd):
+    print(f"case shape={tuple(x_cpu.shape)} dtype={x_cpu.dtype} n:m:g={n}:{m}:{g} sd={sd} gd={gd}", flush=True)
+    val, idx, lay = oracle_sparsify(x_cpu, n, m, sd, g, gd)
+    t = sten.GroupedNMTensor.from_dense(x_cpu.to(DEV), n, m, sparse_dim=sd, group_size=g, group_dim=gd)
+    assert tuple(t.val.shape) == val.shape and tuple(t.idx.shape) == idx.shape
+    assert np.array_equal(to_np(t.idx), idx), "idx differs from the oracle"
+    assert same_bits(t.val, val), "val differs from the oracle"
+    dense = t.to_dense()
+    assert same_bits(dense, O.to_dense(val, idx, lay)), "to_dense differs from the oracle"
+    return t, val, idx, lay
+
+
+def test_config1_fp32_768_bit_exact():
+    # BASELINE config 1: fp32 768x768 N(0,1) seed 0, 2:4, group 16, n:m along the reduction dim
+    torch.manual_seed(0)
+    w = torch.randn(768, 768)
+    check_parity(w, 2, 4, 1, 16, 0)
+    check_parity(w, 2, 4, 0, 16, 1)  # the reference's default orientation
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32, torch.float64])
+@pytest.mark.parametrize("n,m,g", [(2, 4, 16), (1, 8, 32), (2, 8, 32), (3, 6, 4)])
+def test_dtypes_and_ratios(dtype, n, m, g):
+    w = seeded((300, 520), dtype, seed=n * 100 + m, std=0.02)
+    check_parity(w, n, m, 1, g, 0)
+
+
+def test_4_8_32_large_tile():
+    w = seeded((2240 + 100, 72), torch.float16, seed=48, std=0.02)
+    check_parity(w, 4, 8, 1, 32, 0)
+
+
+def test_ties_and_zeros():
+    g = torch.Generator().manual_seed(7)
+    w = torch.randint(-2, 3, (200, 96), generator=g).float()
+    check_parity(w, 2, 4, 1, 16, 0)
+    check_parity(torch.zeros(100, 40), 2, 4, 0, 4, 1)
+    check_parity(w.half(), 1, 4, 0, 8, 1)
+
+
+def test_reference_test_shapes_5_12_2():
+    # tests/test_nmg.py:33-86: shapes (3,a,b), a,b in {17,5,1}, all axis orders, 5:12:2
+    torch.manual_seed(123)
+    dims = [17, 5, 1]
+    for a, b in itertools.product(dims, dims):
+        base = torch.rand(3, a, b)
+        for perm in itertools.permutations(range(3)):
+            x = base.permute(perm).contiguous()
+            layout = "".join("abc"[i] for i in perm)
+            t, val, idx, lay = check_parity(x, 5, 12, layout.index("c"), 2, layout.index("b"))
+            sp = to_np(t.to_dense())
+            xn = x.numpy()
+            assert ((sp == xn) | (sp == 0)).all()
+            assert np.abs(sp).sum() / np.abs(xn).sum() > 5 / 12
+
+
+def test_non_contiguous_input_and_empty():
+    w = seeded((64, 200), torch.float32, seed=3)
+    check_parity(w.t(), 2, 4, 0, 4, 1)           # transposed view, read through strides
+    t = sten.GroupedNMTensor.from_dense(torch.zeros(0, 8, device=DEV), 2, 4, 1, 4, 0)
+    assert t.val.numel() == 0 and tuple(t.to_dense().shape) == (0, 8)
+
+
+def test_clone_layout_matches_oracle_gather():
+    w = seeded((100, 72), torch.float32, seed=11)
+    t, val, idx, lay = check_parity(w, 2, 4, 1, 4, 0)
+    other = seeded((100, 72), torch.float32, seed=12)
+    got = t.clone_layout(other.to(DEV))
+    want = O.gather_merged(O.merge(other.numpy(), lay), idx, 2)
+    assert same_bits(got.val, want)
+    assert got.idx.data_ptr() == t.idx.data_ptr()
+
+
+def test_rejects_cpu_tensor_and_wide_tile():
+    with pytest.raises(sten.NmgError):
+        sten.GroupedNMTensor.from_dense(torch.zeros(8, 8), 2, 4, 1, 1, 0)
+    with pytest.raises(ValueError):
+        sten.GroupedNMTensor.from_dense(torch.zeros(8, 8, device=DEV), 5, 12, 1, 42, 0)
+
+
+def test_full_size_properties_config2():
+    # 4096x4096 fp16 N(0,0.02), 2:4:16 along K: size-independent properties + oracle on a slab
+    torch.manual_seed(0)
+    w = (torch.randn(4096, 4096) * 0.02).half()
+    t = sten.GroupedNMTensor.from_dense(w.to(DEV), 2, 4, 1, 16, 0)
+    lay = t.layout
+    idx = t.idx.view(lay.outer, lay.cols).int()
+    assert bool((idx.sort(dim=1).values == torch.arange(lay.cols, device=DEV, dtype=torch.int32)).all())
+    dense = t.to_dense()
+    wg = w.to(DEV)
+    assert bool(((dense == wg) | (dense == 0)).all())
+    blocks = (dense.view(4096, 1024, 4) != 0).sum(-1)
+    assert int(blocks.max()) <= 2
+    again = sten.GroupedNMTensor.from_dense(dense, 2, 4, 1, 16, 0)      # idempotence of the kept mass
+    assert float(again.to_dense().abs().sum()) == pytest.approx(float(dense.abs().sum()), rel=1e-6)
+    val, idx_o, _ = oracle_sparsify(w[:192], 2, 4, 1, 16, 0)            # first two 96-row chunks
+    k = val.shape[0]
+    assert np.array_equal(to_np(t.idx[:k]), idx_o) and same_bits(t.val[:k], val)

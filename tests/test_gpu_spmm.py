@@ -1,0 +1,190 @@
+"""GPU parity of the nmg x dense matmul, its transposed form and the registered operators.
+Oracle: the equation the reference asserts, C == to_dense(A) @ B (dace_gnm_mult.py:1123,1189-1199),
+evaluated in fp64 from the oracle's own val/idx, plus the CPU restatement of the reference kernel.
+Tolerances: rel-L2 <= 1e-3 for 16-bit inputs with fp32 accumulation, <= 1e-5 for fp32."""
+import copy
+import warnings
+
+import numpy as np
+import pytest
+import torch
+
+import sten_amd as sten
+from oracle import nmg_oracle as O
+from helpers import oracle_sparsify, rel_l2, seeded, to_np
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = {torch.float32: 1e-5, torch.float16: 1e-3, torch.bfloat16: 8e-3}
+
+
+def make(W, n, m, g, sd):
+    return sten.GroupedNMTensor.from_dense(W.to(DEV), n, m, sparse_dim=sd, group_size=g, group_dim=1 - sd)
+
+
+def dense_ref(W, n, m, g, sd):
+    val, idx, lay = oracle_sparsify(W, n, m, sd, g, 1 - sd)
+    return O.to_dense(val, idx, lay).astype(np.float64), (val, idx, lay)
+
+
+@pytest.mark.parametrize("kernel", ["mfma"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,K,T,n,m,g", [
+    (768, 768, 256, 2, 4, 16),
+    (200, 330, 77, 2, 4, 4),
+    (130, 96, 5, 3, 6, 2),
+    (64, 520, 129, 2, 8, 4),
+    (40, 72, 300, 1, 8, 2),
+])
+@pytest.mark.parametrize("sd", [1, 0])
+def test_spmm_both_directions(kernel, dtype, M, K, T, n, m, g, sd):
+    print(f"case {kernel} {dtype} M={M} K={K} T={T} {n}:{m}:{g} sd={sd}", flush=True)
+    W = seeded((M, K), dtype, seed=M + K, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, sd)
+    w = make(W, n, m, g, sd)
+    x = seeded((T, K), dtype, seed=1)
+    y = sten.spmm(w, x.to(DEV), reduce_dim=1, kernel=kernel)            # X @ W^T
+    assert rel_l2(to_np(y), to_np(x).astype(np.float64) @ Wd.T) <= TOL[dtype]
+    gy = seeded((T, M), dtype, seed=2)
+    gx = sten.spmm(w, gy.to(DEV), reduce_dim=0, kernel=kernel)          # G @ W
+    assert rel_l2(to_np(gx), to_np(gy).astype(np.float64) @ Wd) <= TOL[dtype]
+
+
+def test_config1_against_reference_cpu_kernel():
+    # BASELINE config 1 through the reference orientation and the CPU restatement of its kernel
+    torch.manual_seed(0)
+    W = torch.randn(768, 768)
+    X = torch.randn(768, 256)          # B [K, N]
+    val, idx, lay = oracle_sparsify(W, 2, 4, 0, 16, 1)
+    C_cpu = O.simd_spmm(val, idx, lay, X.numpy())
+    w = make(W, 2, 4, 16, 0)
+    C = sten.spmm(w, X.t().contiguous().to(DEV), reduce_dim=1).t()
+    assert rel_l2(to_np(C), C_cpu) <= 1e-5
+    w2 = make(W, 2, 4, 16, 1)          # n:m along the reduction dim (BASELINE wording)
+    Wd, _ = dense_ref(W, 2, 4, 16, 1)
+    C2 = sten.spmm(w2, X.t().contiguous().to(DEV), reduce_dim=1).t()
+    assert rel_l2(to_np(C2), Wd @ X.numpy().astype(np.float64)) <= 1e-5
+
+
+@pytest.mark.parametrize("T", [1, 3, 4, 16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_skinny_kernel(T, dtype):
+    W = seeded((515, 1024), dtype, seed=5, std=0.05)
+    Wd, _ = dense_ref(W, 2, 4, 16, 1)
+    w = make(W, 2, 4, 16, 1)
+    x = seeded((T, 1024), dtype, seed=6)
+    b = seeded((515,), dtype, seed=7)
+    ref = to_np(x).astype(np.float64) @ Wd.T + to_np(b).astype(np.float64)
+    for kernel in ("skinny", "mfma", "auto"):
+        y = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1, kernel=kernel)
+        assert rel_l2(to_np(y), ref) <= TOL[dtype], kernel
+
+
+def test_spmm_argument_errors():
+    w = make(seeded((64, 64), torch.float16, 1), 2, 4, 4, 1)
+    with pytest.raises(sten.NmgError):
+        sten.spmm(w, torch.zeros(4, 64, device=DEV), reduce_dim=1)           # dtype mismatch
+    with pytest.raises(sten.NmgError):
+        sten.spmm(w, torch.zeros(4, 60, device=DEV).half(), reduce_dim=1)    # wrong K
+    with pytest.raises(sten.NmgError):
+        sten.spmm(w, torch.zeros(64, 64, device=DEV).half(), reduce_dim=1, kernel="skinny")
+
+
+def build_sparse_linear(lin, n, m, g, sd, compressed_grad=False):
+    sb = sten.SparsityBuilder()
+    sb.set_weight("weight", initial_sparsifier=sten.GroupedNMSparsifier(n, m, g, sparse_dim=sd, group_dim=1 - sd),
+                  out_format=sten.GroupedNMTensor)
+    if compressed_grad:
+        sb.set_weight_grad("weight", tmp_format=sten.GroupedNMTensor, out_format=sten.GroupedNMTensor)
+    return sb.get_sparse_model(lin)
+
+
+@pytest.mark.parametrize("bias", [True, False])
+@pytest.mark.parametrize("sd", [1, 0])
+@pytest.mark.parametrize("compressed_grad", [False, True])
+def test_linear_module_forward_backward(bias, sd, compressed_grad):
+    # builder flow of tests/test_nmg.py:12-30 on a local nn.Linear; values checked against dense autograd
+    sten.set_dispatch_failure("raise")
+    torch.manual_seed(0)
+    lin = torch.nn.Linear(96, 200, bias=bias).to(DEV)
+    sp = build_sparse_linear(lin, 2, 4, 4, sd, compressed_grad)
+    assert isinstance(sp.weight, sten.SparseParameterWrapper)
+    Wd = sp.weight.wrapped_tensor.to_dense().detach().clone().requires_grad_(True)
+    bd = lin.bias.detach().clone().requires_grad_(True) if bias else None
+    x = torch.randn(3, 7, 96, device=DEV, requires_grad=True)
+    xr = x.detach().clone().requires_grad_(True)
+    y = sp(x)
+    yr = torch.nn.functional.linear(xr, Wd, bd)
+    assert y.shape == yr.shape
+    assert rel_l2(to_np(y), to_np(yr)) <= 1e-5
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    yr.backward(gy)
+    assert rel_l2(to_np(x.grad), to_np(xr.grad)) <= 1e-5
+    mask = (Wd != 0).to(Wd.dtype)
+    gw = sp.weight.grad
+    assert isinstance(gw, sten.SparseTensorWrapper)
+    if compressed_grad:
+        assert isinstance(gw.wrapped_tensor, sten.GroupedNMTensor)
+        # padded / zero-valued kept slots aside, the compressed gradient is the dense one at kept positions
+        got = to_np(gw.wrapped_tensor.to_dense())
+        keep = to_np(sp.weight.wrapped_tensor.clone_layout(torch.ones_like(Wd)).to_dense())
+        assert rel_l2(got, to_np(Wd.grad) * keep) <= 1e-5
+    else:
+        assert isinstance(gw.wrapped_tensor, sten.DenseTensor)
+        assert rel_l2(to_np(gw.wrapped_tensor.to_dense()), to_np(Wd.grad)) <= 1e-5
+    if bias:
+        assert rel_l2(to_np(sp.bias.grad), to_np(bd.grad)) <= 1e-5
+
+
+def test_torch_mm_forward_backward():
+    # registration pattern of tests/test_api.py:272-298 for torch.mm(sparse, dense)
+    sten.set_dispatch_failure("raise")
+    W = seeded((80, 48), torch.float32, 3)
+    B = seeded((48, 33), torch.float32, 4).to(DEV).requires_grad_(True)
+    sp = sten.get_sparsifier_implementation(sten.GroupedNMSparsifier, torch.Tensor, sten.GroupedNMTensor)(
+        sten.GroupedNMSparsifier(2, 4, 4, sparse_dim=1, group_dim=0), W.to(DEV).requires_grad_(True))
+    Wd = sp.wrapped_tensor.to_dense().detach().clone().requires_grad_(True)
+    Br = B.detach().clone().requires_grad_(True)
+    C = torch.mm(sp, B)
+    Cr = torch.mm(Wd, Br)
+    assert rel_l2(to_np(C), to_np(Cr)) <= 1e-5
+    g = torch.randn_like(C)
+    C.backward(g)
+    Cr.backward(g)
+    assert rel_l2(to_np(B.grad), to_np(Br.grad)) <= 1e-5
+    assert rel_l2(to_np(sp.grad.wrapped_tensor.to_dense()), to_np(Wd.grad)) <= 1e-5
+
+
+def test_optimizer_steps_keep_pattern():
+    # optimizer flow of tests/test_api.py:421-450, :512-551 with the nmg format
+    torch.manual_seed(1)
+    lin = torch.nn.Linear(64, 48).to(DEV)
+    sb = sten.SparsityBuilder()
+    sb.set_weight("weight", initial_sparsifier=sten.GroupedNMSparsifier(2, 4, 4, sparse_dim=1, group_dim=0),
+                  out_format=sten.GroupedNMTensor)
+    opt = torch.optim.SGD(lin.parameters(), lr=0.1, momentum=0.9)
+    lin, opt = sb.sparsify_model_and_optimizer_inplace(lin, opt)
+    idx0 = lin.weight.wrapped_tensor.idx.clone()
+    w0 = lin.weight.wrapped_tensor.to_dense().clone()
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        for _ in range(3):
+            loss = lin(torch.randn(5, 64, device=DEV)).abs().sum()
+            loss.backward()
+            opt.step()
+            opt.zero_grad()
+    w1 = lin.weight.wrapped_tensor.to_dense()
+    assert isinstance(lin.weight.wrapped_tensor, sten.GroupedNMTensor)
+    assert torch.equal(lin.weight.wrapped_tensor.idx, idx0)
+    assert not torch.allclose(w0, w1)
+    assert bool(((w1 != 0) <= (w0 != 0)).all())        # nothing outside the pattern became non-zero
+    assert lin.weight.requires_grad
+
+
+def test_unregistered_op_raises_in_raise_mode():
+    sten.set_dispatch_failure("raise")
+    w = sten.SparseTensorWrapper.wrapped_from_dense(
+        make(seeded((16, 16), torch.float32, 1), 2, 4, 1, 1), torch.zeros(1))
+    with pytest.raises(sten.DispatchError):
+        torch.relu(w)
