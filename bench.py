@@ -58,6 +58,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--kernel", default="auto")
+    ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -73,6 +74,7 @@ def main():
     W = (torch.randn(M, K) * 0.02).half().to(dev)
     X = torch.randn(N, K).half().to(dev)
     w = sten.GroupedNMTensor.from_dense(W, n, m, sparse_dim=1, group_size=g, group_dim=0)
+    w.spmm_opt["variant"] = args.variant
     w.rowpack()
     for _ in range(args.warmup):
         y = sten.spmm(w, X, reduce_dim=1, kernel=args.kernel)

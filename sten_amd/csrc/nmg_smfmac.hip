@@ -1,0 +1,721 @@
+// nmg x dense matmul on the sparse matrix cores (V_SMFMAC_F32_32X32X32_{F16,BF16}).
+//
+// Applies when the reduction runs along the sparse dim and every aligned group of 4 positions
+// keeps at most 2 values (2:4, 1:4, 1:8, 2:8, 1:2, ...): the weight is the sparse A operand of
+// the instruction, the activations the dense B operand.
+//
+//   Y[tok, f] = sum_k X[tok, k] * W[f, k] (+ bias[f])
+//
+// Operand ("fragpack", built once per weight by nmg_fragpack):
+//   fp_val [MB][KS][64 lanes][8]  -- for feature block mb (32 rows) and k-step ks (32 dense k),
+//                                    lane l holds the 4 pairs of kept values of row mb*32 + l%32
+//   fp_idx [MB][KP][64 lanes] u32 -- 2-bit positions of those 8 values; low half-word = even
+//                                    k-step of the pair, high half-word = odd k-step (ABID 0/1)
+// Instruction layout (measured on gfx950): with B lane (col = l%32, h = l/32) holding dense
+// k = 16h + e (e = 0..15), A lane (row = l%32, ga = l/32) pair q = 0..3 covers the 4-wide
+// k-group kg = 4*(q/2) + 2*ga + (q%2); element 2q+i is selected by idx bits [4q+2i+1 : 4q+2i].
+//
+// Workgroup: WM x WN wavefronts, each 128 features x 64 tokens (4 x 2 accumulator blocks).
+// A fragments go global -> registers (already in lane order, fully coalesced); the activation
+// tile goes global -> registers -> LDS (double buffered), one barrier per 64-wide K step.
+#include "nmg_common.h"
+
+#include <type_traits>
+
+namespace nmg {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Smf;
+template <> struct Smf<__half> {
+    using A = f16x8;
+    using B = f16x16;
+    template <int ABID> __device__ static f32x16 run(A a, B b, f32x16 c, int idx)
+    {
+        return __builtin_amdgcn_smfmac_f32_32x32x32_f16(a, b, c, idx, 0, ABID);
+    }
+};
+template <> struct Smf<__hip_bfloat16> {
+    using A = bf16x8;
+    using B = bf16x16;
+    template <int ABID> __device__ static f32x16 run(A a, B b, f32x16 c, int idx)
+    {
+        return __builtin_amdgcn_smfmac_f32_32x32x32_bf16(a, b, c, idx, 0, ABID);
+    }
+};
+
+struct SmfParams {
+    const void *fp_val;
+    const uint32_t *fp_idx;
+    const void *x;
+    void *y;
+    const void *bias;
+    int64_t M, K, T, ldx, ldy;
+    int MB, KP;          // feature blocks of 32, k pairs of 64
+    int tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ uint16_t f32_to_bits16(float x, __half *) { return __half_as_ushort(__float2half(x)); }
+__device__ __forceinline__ uint16_t f32_to_bits16(float x, __hip_bfloat16 *)
+{
+    __hip_bfloat16 b = __float2bfloat16(x);
+    return *reinterpret_cast<uint16_t *>(&b);
+}
+
+constexpr int SMF_ROW = 144;  // bytes per token row in LDS: 64 k * 2 B + 16 B pad (conflict-free b128 reads)
+
+// WM x WN wavefronts per workgroup, FB x TB accumulator blocks (32 features x 32 tokens) per
+// wavefront, MINW = wavefronts per SIMD the register budget is sized for.  GUARD = false assumes
+// K % 64 == 0 (no bounds checks in the K loop; token rows are clamped, feature blocks are padded
+// in the operand).
+template <typename T, int WM, int WN, int FB, int TB, int MINW, bool GUARD>
+__global__ __launch_bounds__(64 * WM * WN, MINW) void spmm_smfmac_kernel(SmfParams P)
+{
+    using S = Smf<T>;
+    constexpr int BMf = WM * FB * 32, BNt = WN * TB * 32;   // workgroup tile
+    constexpr int NTHR = 64 * WM * WN;
+    constexpr int NLOAD = BNt * 8 / NTHR;          // 16-byte chunks of the X tile per thread
+    static_assert(NLOAD * NTHR == BNt * 8, "X tile must split evenly over the threads");
+    extern __shared__ __align__(16) unsigned char smf_lds[];
+    unsigned char (*Xs)[BNt * SMF_ROW] = (unsigned char (*)[BNt * SMF_ROW])smf_lds;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+
+    // Workgroup -> tile: consecutive ids are dealt round-robin to the 8 XCDs, so give each XCD a
+    // contiguous run of tiles (token tile fastest) and let it reuse its weight rows from its L2.
+    int id = blockIdx.x;
+    const int ntiles = P.tiles_m * P.tiles_n;
+    if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
+    const int tile_m = id / P.tiles_n, tile_n = id - tile_m * P.tiles_n;
+    const int64_t f0 = (int64_t)tile_m * BMf, t0 = (int64_t)tile_n * BNt;
+
+    const int KS = P.KP * 2;
+    const int mb0 = (int)(f0 / 32) + wm * FB;
+    const u32x4 zero4 = {0, 0, 0, 0};
+
+    f32x16 acc[FB][TB];
+#pragma unroll
+    for (int i = 0; i < FB; i++)
+#pragma unroll
+        for (int j = 0; j < TB; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    // ---- per-thread source pointers (advanced by one K step per iteration) ----
+    const u32x4 *a_ptr[FB];
+    const uint32_t *i_ptr[FB];
+#pragma unroll
+    for (int fb = 0; fb < FB; fb++) {
+        // the operand is padded to whole workgroup tiles of feature blocks, so mb is always valid
+        const int mb = mb0 + fb;
+        a_ptr[fb] = (const u32x4 *)P.fp_val + (int64_t)mb * KS * 64 + lane;
+        i_ptr[fb] = P.fp_idx + (int64_t)mb * P.KP * 64 + lane;
+    }
+    const unsigned char *x_ptr[NLOAD];
+    bool x_ok[NLOAD];
+    int x_lds[NLOAD];
+#pragma unroll
+    for (int i = 0; i < NLOAD; i++) {
+        const int c = tid + i * NTHR;
+        const int row = c >> 3, kc = c & 7;
+        int64_t tok = t0 + row;
+        x_ok[i] = tok < P.T;
+        if (tok >= P.T) tok = P.T - 1;  // clamped rows are computed and never stored
+        x_ptr[i] = (const unsigned char *)P.x + (tok * P.ldx + kc * 8) * 2;
+        x_lds[i] = row * SMF_ROW + kc * 16;
+    }
+
+    u32x4 a_cur[FB][2], a_nxt[FB][2];
+    uint32_t i_cur[FB], i_nxt[FB];
+    u32x4 x_reg[NLOAD];
+
+    auto load_a = [&](u32x4 (&a)[FB][2], uint32_t (&ix)[FB]) {
+#pragma unroll
+        for (int fb = 0; fb < FB; fb++) {
+            a[fb][0] = a_ptr[fb][0];
+            a[fb][1] = a_ptr[fb][64];
+            ix[fb] = *i_ptr[fb];
+            a_ptr[fb] += 128;
+            i_ptr[fb] += 64;
+        }
+    };
+    auto load_x = [&](int kp) {
+#pragma unroll
+        for (int i = 0; i < NLOAD; i++) {
+            if (GUARD) {
+                const int kc = (tid + i * NTHR) & 7;
+                u32x4 v = zero4;
+                if (x_ok[i] && (int64_t)kp * 64 + kc * 8 < P.K) v = *(const u32x4 *)x_ptr[i];
+                x_reg[i] = v;
+            } else {
+                x_reg[i] = *(const u32x4 *)x_ptr[i];
+            }
+            x_ptr[i] += 128;
+        }
+    };
+    auto store_x = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < NLOAD; i++) *(u32x4 *)(&Xs[buf][x_lds[i]]) = x_reg[i];
+    };
+
+    load_a(a_cur, i_cur);
+    load_x(0);
+    store_x(0);
+    __syncthreads();
+
+    const int b_off = (lane & 31) * SMF_ROW + (lane >> 5) * 32 + wn * (TB * 32) * SMF_ROW;
+    for (int kp = 0; kp < P.KP; kp++) {
+        const int cur = kp & 1;
+        const bool more = kp + 1 < P.KP;
+        if (more) {
+            load_a(a_nxt, i_nxt);
+            load_x(kp + 1);
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            typename S::B b[TB];
+#pragma unroll
+            for (int tb = 0; tb < TB; tb++) {
+                const unsigned char *p = &Xs[cur][b_off + tb * 32 * SMF_ROW + ks * 64];
+                union {
+                    u32x4 u[2];
+                    typename S::B v;
+                } cv;
+                cv.u[0] = *(const u32x4 *)p;
+                cv.u[1] = *(const u32x4 *)(p + 16);
+                b[tb] = cv.v;
+            }
+#pragma unroll
+            for (int fb = 0; fb < FB; fb++) {
+                union {
+                    u32x4 u;
+                    typename S::A v;
+                } ca;
+                ca.u = a_cur[fb][ks];
+#pragma unroll
+                for (int tb = 0; tb < TB; tb++) {
+                    if (ks == 0)
+                        acc[fb][tb] = S::template run<0>(ca.v, b[tb], acc[fb][tb], (int)i_cur[fb]);
+                    else
+                        acc[fb][tb] = S::template run<1>(ca.v, b[tb], acc[fb][tb], (int)i_cur[fb]);
+                }
+            }
+        }
+        if (more) {
+            store_x(cur ^ 1);
+#pragma unroll
+            for (int fb = 0; fb < FB; fb++) {
+                a_cur[fb][0] = a_nxt[fb][0];
+                a_cur[fb][1] = a_nxt[fb][1];
+                i_cur[fb] = i_nxt[fb];
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: D[row = feature][col = token]; lane holds token l%32, features
+    //      8*(r/4) + 4*(l/32) + r%4 -> four consecutive features per register quad ----
+    uint16_t *Y = (uint16_t *)P.y;
+    const T *bias = (const T *)P.bias;
+    const bool vec_ok = (P.ldy & 3) == 0 && ((uintptr_t)P.y & 7) == 0;
+#pragma unroll
+    for (int tb = 0; tb < TB; tb++) {
+        const int64_t tok = t0 + (wn * TB + tb) * 32 + (lane & 31);
+        if (tok >= P.T) continue;
+#pragma unroll
+        for (int fb = 0; fb < FB; fb++) {
+#pragma unroll
+            for (int rq = 0; rq < 4; rq++) {
+                const int64_t f = f0 + (wm * FB + fb) * 32 + rq * 8 + (lane >> 5) * 4;
+                if (f >= P.M) continue;
+                uint16_t h[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    float v = acc[fb][tb][rq * 4 + i];
+                    if (bias && f + i < P.M) v += to_f32(bias[f + i]);
+                    h[i] = f32_to_bits16(v, (T *)nullptr);
+                }
+                uint16_t *dst = Y + tok * P.ldy + f;
+                if (vec_ok && f + 3 < P.M) {
+                    uint2 pk;
+                    pk.x = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
+                    pk.y = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
+                    *(uint2 *)dst = pk;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        if (f + i < P.M) dst[i] = h[i];
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------ pipelined kernel
+// Same math, deeper memory pipeline: weight fragments, index words and the activation tile all
+// travel global -> LDS with the LDS-DMA form of global_load (no registers involved), into a ring
+// of PIPE_NS stages, so PIPE_NS-1 K steps of loads are in flight while one is being multiplied.
+// HBM / fabric latency on this part is several K steps long, which a one-step register prefetch
+// cannot cover.  Completion is tracked by hand with s_waitcnt vmcnt; one barrier per K step.
+//
+// Stage layout (bytes): [8 feature blocks x 2 k-steps x 1024] weight values in lane order,
+// [8 x 256] index words, [128 token rows x 128] activations.  A DMA load writes 64 lanes x 16 B
+// contiguously, so the activation rows cannot be padded; instead the 16-byte chunks of a row
+// are XOR-swizzled with (row/2)%8, chosen on the global side, which makes the fragment reads
+// (32 rows x 16 B at one logical chunk) conflict-free.
+// Requires K % 64 == 0.  Workgroup 256 features x 128 tokens, 2x2 wavefronts of 128 x 64.
+constexpr int PIPE_NS = 4;
+constexpr int PIPE_AVAL = 8 * 2 * 1024;
+constexpr int PIPE_AIDX = 8 * 256;
+constexpr int PIPE_X = 128 * 128;
+constexpr int PIPE_STAGE = PIPE_AVAL + PIPE_AIDX + PIPE_X;
+constexpr int PIPE_LPT = 10;  // DMA loads issued per thread per stage: 4 weight + 2 index + 4 activation
+
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+typedef const __attribute__((address_space(1))) void *glb_ptr_t;
+
+template <typename T>
+__global__ __launch_bounds__(256, 1) void spmm_smfmac_pipe_kernel(SmfParams P)
+{
+    using S = Smf<T>;
+    constexpr int FB = 4, TB = 2;
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+
+    int id = blockIdx.x;
+    const int ntiles = P.tiles_m * P.tiles_n;
+    if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
+    const int tile_m = id / P.tiles_n, tile_n = id - tile_m * P.tiles_n;
+    const int64_t f0 = (int64_t)tile_m * 256, t0 = (int64_t)tile_n * 128;
+    const int KP = P.KP, KS = KP * 2;
+    const int mbT = (int)(f0 / 32);
+
+    f32x16 acc[FB][TB];
+#pragma unroll
+    for (int i = 0; i < FB; i++)
+#pragma unroll
+        for (int j = 0; j < TB; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    // ---- DMA sources: wave-uniform base (advanced per K step on the scalar unit) plus a
+    //      32-bit per-lane byte offset ----
+    const unsigned char *av_base = (const unsigned char *)P.fp_val + (int64_t)mbT * KS * 1024;
+    const unsigned char *ai_base = (const unsigned char *)P.fp_idx + (int64_t)mbT * KP * 256;
+    const unsigned char *x_base = (const unsigned char *)P.x;
+    // weight values: wavefront w moves fragments fi = 4w..4w+3 (fi = fb*2 + ks) of every stage
+    uint32_t av_off[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int fi = wave * 4 + i, fb = fi >> 1, ks = fi & 1;
+        av_off[i] = (uint32_t)(((fb * KS + ks) * 64 + lane) * 16);
+    }
+    // index words: wavefront w moves feature blocks 2w, 2w+1
+    uint32_t ai_off[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) ai_off[i] = (uint32_t)((((wave * 2 + i) * KP) * 64 + lane) * 4);
+    // activations: wavefront w moves row groups 4w..4w+3 (8 rows each); lane -> (row, piece)
+    uint32_t x_off[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int row = (wave * 4 + i) * 8 + (lane >> 3);
+        const int piece = lane & 7;
+        const int q = piece ^ ((row >> 1) & 7);       // logical chunk stored at this piece
+        int64_t tok = t0 + row;
+        if (tok >= P.T) tok = P.T - 1;                // clamped rows are computed, never stored
+        x_off[i] = (uint32_t)((tok * P.ldx + q * 8) * 2);
+    }
+
+    auto issue = [&](int kp, int stage) {
+        unsigned char *base = smem + stage * PIPE_STAGE;
+        const unsigned char *avb = av_base + (int64_t)kp * 2048;   // two k-steps of one feature block
+        const unsigned char *aib = ai_base + (int64_t)kp * 256;
+        const unsigned char *xb = x_base + (int64_t)kp * 128;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(avb + av_off[i]),
+                                             (lds_ptr_t)(base + (wave * 4 + i) * 1024), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(aib + ai_off[i]),
+                                             (lds_ptr_t)(base + PIPE_AVAL + (wave * 2 + i) * 256), 4, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[i]),
+                                             (lds_ptr_t)(base + PIPE_AVAL + PIPE_AIDX + (wave * 4 + i) * 1024), 16, 0, 0);
+    };
+
+    // ---- fragment read offsets inside a stage ----
+    const int a_off = (wm * FB) * 2 * 1024 + lane * 16;
+    const int i_off = PIPE_AVAL + (wm * FB) * 256 + lane * 4;
+    const int j = lane & 31, h = lane >> 5, sw = (j >> 1) & 7;
+    int b_off[2][2];  // [ks][c]
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+            b_off[ks][c] = PIPE_AVAL + PIPE_AIDX + (wn * 64 + j) * 128 + (((ks * 4 + h * 2 + c) ^ sw) << 4);
+
+    // Fragment registers of one k-step: 4 weight fragments, their index words, 2 activation
+    // fragments.  Set 0 serves the even k-step of a stage, set 1 the odd one.
+    struct Frags {
+        u32x4 a[FB];
+        uint32_t ix[FB];
+        u32x4 b[TB][2];
+    };
+    Frags fr0, fr1;
+    auto read_frags = [&](Frags &f, const unsigned char *base, int ks) {
+#pragma unroll
+        for (int fb = 0; fb < FB; fb++) {
+            f.a[fb] = *(const u32x4 *)(base + a_off + (fb * 2 + ks) * 1024);
+            f.ix[fb] = *(const uint32_t *)(base + i_off + fb * 256);
+        }
+#pragma unroll
+        for (int tb = 0; tb < TB; tb++) {
+            f.b[tb][0] = *(const u32x4 *)(base + b_off[ks][0] + tb * 32 * 128);
+            f.b[tb][1] = *(const u32x4 *)(base + b_off[ks][1] + tb * 32 * 128);
+        }
+    };
+    auto mma = [&](const Frags &f, auto abid_tag, auto lo_tag, auto hi_tag) {
+        constexpr int ABID = decltype(abid_tag)::value;
+#pragma unroll
+        for (int fb = decltype(lo_tag)::value; fb < decltype(hi_tag)::value; fb++) {
+            union {
+                u32x4 u;
+                typename S::A v;
+            } ca;
+            ca.u = f.a[fb];
+#pragma unroll
+            for (int tb = 0; tb < TB; tb++) {
+                union {
+                    u32x4 u[2];
+                    typename S::B v;
+                } cb;
+                cb.u[0] = f.b[tb][0];
+                cb.u[1] = f.b[tb][1];
+                acc[fb][tb] = S::template run<ABID>(ca.v, cb.v, acc[fb][tb], (int)f.ix[fb]);
+            }
+        }
+    };
+
+    // Fill the ring: K steps 0..PIPE_NS-1 in flight, then wait for step 0.
+#pragma unroll
+    for (int st = 0; st < PIPE_NS; st++) issue(st < KP ? st : KP - 1, st);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((PIPE_NS - 1) * PIPE_LPT) : "memory");
+    asm volatile("s_barrier" ::: "memory");
+    read_frags(fr0, smem, 0);
+
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using IFB = std::integral_constant<int, FB>;
+    // Instruction-group masks of the scheduler: 0x008 MFMA, 0x020 VMEM read, 0x100 LDS read.
+    // One MFMA occupies the matrix pipe for ~32 cycles during which the wavefront can issue a
+    // handful of other instructions for free, so the LDS reads and DMA loads are dealt out a
+    // few per MFMA instead of in bursts between them.
+    for (int kp = 0; kp < KP; kp++) {
+        const int slot = kp & (PIPE_NS - 1);
+        const unsigned char *base = smem + slot * PIPE_STAGE;
+        // ---- even k-step: MFMAs on set 0, fetch set 1 of the same stage ----
+        read_frags(fr1, base, 1);
+        mma(fr0, I0{}, I0{}, IFB{});
+#pragma unroll
+        for (int i = 0; i < FB * TB; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i < 5) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- odd k-step, first MFMA, then hand the stage back ----
+        mma(fr1, I1{}, I0{}, I1{});
+        __builtin_amdgcn_sched_barrier(0);
+        // This wavefront holds all of stage kp in registers; once every wavefront does, the slot
+        // can be refilled with K step kp + PIPE_NS.  Step kp+1 must have landed to fetch its
+        // even-step fragments, which then load under the odd k-step's MFMAs.
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((PIPE_NS - 2) * PIPE_LPT) : "memory");
+        asm volatile("s_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        {
+            const int nk = kp + PIPE_NS;
+            issue(nk < KP ? nk : KP - 1, slot);
+        }
+        read_frags(fr0, smem + ((kp + 1) & (PIPE_NS - 1)) * PIPE_STAGE, 0);
+        mma(fr1, I1{}, I1{}, IFB{});
+#pragma unroll
+        for (int i = 0; i < (FB - 1) * TB; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i < 5) {
+                __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // drain the redundant tail loads before the LDS is released
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    uint16_t *Y = (uint16_t *)P.y;
+    const T *bias = (const T *)P.bias;
+    const bool vec_ok = (P.ldy & 3) == 0 && ((uintptr_t)P.y & 7) == 0;
+#pragma unroll
+    for (int tb = 0; tb < TB; tb++) {
+        const int64_t tok = t0 + (wn * TB + tb) * 32 + (lane & 31);
+        if (tok >= P.T) continue;
+#pragma unroll
+        for (int fb = 0; fb < FB; fb++) {
+#pragma unroll
+            for (int rq = 0; rq < 4; rq++) {
+                const int64_t f = f0 + (wm * FB + fb) * 32 + rq * 8 + (lane >> 5) * 4;
+                if (f >= P.M) continue;
+                uint16_t hh[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    float v = acc[fb][tb][rq * 4 + i];
+                    if (bias && f + i < P.M) v += to_f32(bias[f + i]);
+                    hh[i] = f32_to_bits16(v, (T *)nullptr);
+                }
+                uint16_t *dst = Y + tok * P.ldy + f;
+                if (vec_ok && f + 3 < P.M) {
+                    uint2 pk;
+                    pk.x = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
+                    pk.y = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
+                    *(uint2 *)dst = pk;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        if (f + i < P.M) dst[i] = hh[i];
+                }
+            }
+        }
+    }
+}
+
+template <typename T> static int launch_smfmac_pipe(SmfParams &P, hipStream_t s)
+{
+    P.tiles_m = (int)((P.M + 255) / 256);
+    P.tiles_n = (int)((P.T + 127) / 128);
+    dim3 grid((unsigned)(P.tiles_m * P.tiles_n));
+    const size_t lds = (size_t)PIPE_NS * PIPE_STAGE;
+    auto k = spmm_smfmac_pipe_kernel<T>;
+    NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(k, grid, dim3(256), lds, s, P);
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
+// ------------------------------------------------------------------------------ fragpack
+struct FragpackParams {
+    const void *pk_val;   // rowpack values [G, nb, n]
+    const void *pk_pat;   // rowpack patterns [G, nb]
+    const int8_t *order;
+    void *fp_val;
+    uint32_t *fp_idx;
+    int64_t G, S, nb;
+    int n, m, pat_bytes, MB, KP;
+};
+
+// One thread per (feature block, k pair, lane): emits its 2 x 8 values and one index word.
+template <typename T> __global__ void fragpack_kernel(FragpackParams P)
+{
+    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t total = (int64_t)P.MB * P.KP * 64;
+    if (gid >= total) return;
+    const int lane = (int)(gid & 63);
+    const int64_t rest = gid >> 6;
+    const int kp = (int)(rest % P.KP);
+    const int mb = (int)(rest / P.KP);
+    const int64_t row = (int64_t)mb * 32 + (lane & 31);
+    const int ga = lane >> 5;
+    const T *pkv = (const T *)P.pk_val;
+    uint32_t idxword = 0;
+    for (int ks = 0; ks < 2; ks++) {
+        uint16_t vals[8];
+        uint32_t half = 0;
+        for (int q = 0; q < 4; q++) {
+            const int kg = 4 * (q >> 1) + 2 * ga + (q & 1);
+            const int64_t k4 = ((int64_t)kp * 2 + ks) * 32 + kg * 4;
+            int pos[2] = {0, 1};
+            uint16_t v[2] = {0, 0};
+            int cnt = 0;
+            if (row < P.G) {
+                for (int i = 0; i < 4 && cnt < 2; i++) {
+                    const int64_t k = k4 + i;
+                    if (k >= P.S) break;
+                    const int64_t b = k / P.m;
+                    const int r = (int)(k - b * P.m);
+                    const int p = (P.pat_bytes == 1) ? (int)((const uint8_t *)P.pk_pat)[row * P.nb + b]
+                                                     : (int)((const uint16_t *)P.pk_pat)[row * P.nb + b];
+                    for (int j = 0; j < P.n; j++)
+                        if (P.order[p * P.n + j] == r) {
+                            T x = pkv[(row * P.nb + b) * P.n + j];
+                            pos[cnt] = i;
+                            v[cnt] = *reinterpret_cast<uint16_t *>(&x);
+                            cnt++;
+                            break;
+                        }
+                }
+            }
+            if (cnt == 0) {
+                pos[0] = 0;
+                pos[1] = 1;
+            } else if (cnt == 1) {
+                // add a zero at an unused position, keeping positions increasing
+                if (pos[0] == 3) {
+                    pos[1] = 3;
+                    v[1] = v[0];
+                    pos[0] = 0;
+                    v[0] = 0;
+                } else {
+                    pos[1] = 3;
+                    v[1] = 0;
+                }
+            }
+            vals[2 * q] = v[0];
+            vals[2 * q + 1] = v[1];
+            half |= (uint32_t)(pos[0] | (pos[1] << 2)) << (4 * q);
+        }
+        idxword |= half << (16 * ks);
+        uint16_t *dst = (uint16_t *)P.fp_val + (((int64_t)mb * (P.KP * 2) + kp * 2 + ks) * 64 + lane) * 8;
+        for (int e = 0; e < 8; e++) dst[e] = vals[e];
+    }
+    P.fp_idx[((int64_t)mb * P.KP + kp) * 64 + lane] = idxword;
+}
+
+// Every aligned group of 4 positions inside an m-block must keep <= 2 values.
+static bool pattern_fits_2of4(int n, int m)
+{
+    if (!(m % 4 == 0 || 4 % m == 0)) return false;
+    const int8_t *ord = host_order(n, m);
+    if (!ord) return false;
+    const int64_t c = binom(m, n);
+    if (m < 4) return n * (4 / m) <= 2;
+    for (int64_t p = 0; p < c; p++) {
+        int cnt[16] = {0};
+        for (int j = 0; j < n; j++) {
+            int grp = ord[p * n + j] / 4;
+            if (++cnt[grp] > 2) return false;
+        }
+    }
+    return true;
+}
+
+}  // namespace nmg
+
+using namespace nmg;
+
+extern "C" int nmg_fragpack_supported(int n, int m) { return pattern_fits_2of4(n, m) ? 1 : 0; }
+
+extern "C" int nmg_fragpack_sizes(int64_t G, int64_t S, int64_t *val_elems, int64_t *idx_words)
+{
+    NMG_REQUIRE(G >= 0 && S >= 0 && val_elems && idx_words, NMG_ERR_ARG, "bad fragpack size query");
+    const int64_t MB = (G + 255) / 256 * 8, KP = (S + 63) / 64;  // whole 256-line workgroup tiles
+    *val_elems = MB * KP * 2 * 64 * 8;
+    *idx_words = MB * KP * 64;
+    return NMG_OK;
+}
+
+extern "C" int nmg_fragpack(const void *d_pk_val, const void *d_pk_pat, int64_t G, int64_t S,
+                            void *d_fp_val, void *d_fp_idx, int n, int m, int dtype, void *stream)
+{
+    NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED,
+                "the sparse matrix cores take f16/bf16 only");
+    NMG_REQUIRE(m >= 1 && m <= 64 && n >= 0 && n <= m, NMG_ERR_ARG, "invalid n:m = %d:%d", n, m);
+    NMG_REQUIRE(pattern_fits_2of4(n, m), NMG_ERR_UNSUPPORTED,
+                "%d:%d patterns do not fit 2-of-4 groups", n, m);
+    if (G == 0 || S == 0) return NMG_OK;
+    NMG_REQUIRE(d_pk_val && d_pk_pat && d_fp_val && d_fp_idx, NMG_ERR_ARG, "null device pointer");
+    FragpackParams P{};
+    P.pk_val = d_pk_val;
+    P.pk_pat = d_pk_pat;
+    if (int rc = device_order(n, m, &P.order)) return rc;
+    P.fp_val = d_fp_val;
+    P.fp_idx = (uint32_t *)d_fp_idx;
+    P.G = G;
+    P.S = S;
+    P.nb = (S + m - 1) / m;
+    P.n = n;
+    P.m = m;
+    P.pat_bytes = (int)nmg_rowpack_pat_bytes(n, m);
+    P.MB = (int)((G + 255) / 256 * 8);
+    P.KP = (int)((S + 63) / 64);
+    const int64_t total = (int64_t)P.MB * P.KP * 64;
+    const int bs = 256;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == NMG_F16)
+        hipLaunchKernelGGL(fragpack_kernel<__half>, dim3((unsigned)((total + bs - 1) / bs)), dim3(bs), 0, s, P);
+    else
+        hipLaunchKernelGGL(fragpack_kernel<__hip_bfloat16>, dim3((unsigned)((total + bs - 1) / bs)), dim3(bs), 0, s, P);
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
+template <typename T, int WM, int WN, int FB, int TB, int MINW>
+static int launch_smfmac_cfg(SmfParams &P, hipStream_t s)
+{
+    constexpr int BMf = WM * FB * 32, BNt = WN * TB * 32;
+    P.tiles_m = (int)((P.M + BMf - 1) / BMf);
+    P.tiles_n = (int)((P.T + BNt - 1) / BNt);
+    dim3 grid((unsigned)(P.tiles_m * P.tiles_n));
+    const size_t lds = (size_t)2 * BNt * SMF_ROW;
+    const bool guard = (P.K % 64) != 0;
+    auto k = guard ? spmm_smfmac_kernel<T, WM, WN, FB, TB, MINW, true>
+                   : spmm_smfmac_kernel<T, WM, WN, FB, TB, MINW, false>;
+    if (lds > 64 * 1024)
+        NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(k, grid, dim3(64 * WM * WN), lds, s, P);
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
+template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStream_t s)
+{
+    switch (variant) {
+    case 0: return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);  // 256 lines x 128 tokens, 1 wave/SIMD
+    case 1: return launch_smfmac_cfg<T, 2, 2, 2, 2, 2>(P, s);  // 128 x 128, 2 waves/SIMD
+    case 2: return launch_smfmac_cfg<T, 2, 2, 2, 4, 2>(P, s);  // 128 x 256
+    case 3: return launch_smfmac_cfg<T, 4, 1, 2, 4, 2>(P, s);  // 256 x 128, waves stacked on lines
+    case 4:                                                     // 256 x 128, LDS-DMA ring
+        if (P.K % 64 != 0) return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
+        return launch_smfmac_pipe<T>(P, s);
+    }
+    return NMG_ERR_ARG;
+}
+
+extern "C" int nmg_spmm_smfmac(const void *d_fp_val, const void *d_fp_idx, int64_t M, int64_t K,
+                               const void *d_x, int64_t ldx, void *d_y, int64_t ldy,
+                               const void *d_bias, int64_t T, int dtype, int variant, void *stream)
+{
+    NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED,
+                "the sparse matrix cores take f16/bf16 only");
+    NMG_REQUIRE(M >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
+    NMG_REQUIRE(variant >= 0 && variant <= 4, NMG_ERR_ARG, "unknown tile variant %d", variant);
+    NMG_REQUIRE(ldx >= K && ldy >= M, NMG_ERR_ARG, "leading dimension smaller than row length");
+    NMG_REQUIRE((K % 8) == 0 && (ldx % 8) == 0 && ((uintptr_t)d_x % 16) == 0, NMG_ERR_UNSUPPORTED,
+                "activations must be 16-byte aligned with K and ldx multiples of 8");
+    if (M == 0 || K == 0 || T == 0) return NMG_OK;
+    NMG_REQUIRE(d_fp_val && d_fp_idx && d_x && d_y, NMG_ERR_ARG, "null device pointer");
+    SmfParams P{};
+    P.fp_val = d_fp_val;
+    P.fp_idx = (const uint32_t *)d_fp_idx;
+    P.x = d_x;
+    P.y = d_y;
+    P.bias = d_bias;
+    P.M = M;
+    P.K = K;
+    P.T = T;
+    P.ldx = ldx;
+    P.ldy = ldy;
+    P.MB = (int)((M + 255) / 256 * 8);
+    P.KP = (int)((K + 63) / 64);
+    hipStream_t s = (hipStream_t)stream;
+    return dtype == NMG_F16 ? launch_smfmac<__half>(P, variant, s)
+                            : launch_smfmac<__hip_bfloat16>(P, variant, s);
+}

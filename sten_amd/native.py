@@ -48,6 +48,10 @@ SIGNATURES = {
     "nmg_rowpack_pat_bytes": (_I64, [_I, _I]),
     "nmg_rowpack": (_I, [_P, _P, _I64, _I64, _P, _P, _I, _I, _I, _I, _P]),
     "nmg_spmm": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _I, _I, _I, _P]),
+    "nmg_fragpack_supported": (_I, [_I, _I]),
+    "nmg_fragpack_sizes": (_I, [_I64, _I64, ctypes.POINTER(_I64), ctypes.POINTER(_I64)]),
+    "nmg_fragpack": (_I, [_P, _P, _I64, _I64, _P, _P, _I, _I, _I, _P]),
+    "nmg_spmm_smfmac": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _P]),
 }
 
 _lib = None

@@ -190,6 +190,32 @@ class GroupedNMTensor:
             self._rowpack = (key, pk_val, pk_pat)
         return self._rowpack[1], self._rowpack[2]
 
+    def fragpack(self):
+        """Operand of the sparse-matrix-core kernel (values + 2-bit positions in instruction
+        register order); ``None`` when the n:m pattern does not fit 2-of-4 groups or the dtype is
+        not 16-bit.  Cached until ``val`` changes."""
+        lay = self.layout
+        lib = native.load()
+        if self.val.dtype not in (torch.float16, torch.bfloat16):
+            return None
+        if not lib.nmg_fragpack_supported(lay.n, lay.m):
+            return None
+        pk_val, pk_pat = self.rowpack()
+        key = self._rowpack[0]
+        cached = getattr(self, "_fragpack", None)
+        if cached is None or cached[0] != key:
+            ve, iw = ctypes.c_int64(), ctypes.c_int64()
+            native.check(lib.nmg_fragpack_sizes(lay.G, lay.S, ctypes.byref(ve), ctypes.byref(iw)))
+            fp_val = torch.empty(ve.value, dtype=self.val.dtype, device=self.val.device)
+            fp_idx = torch.empty(iw.value, dtype=torch.int32, device=self.val.device)
+            with torch.cuda.device(self.val.device):
+                native.check(lib.nmg_fragpack(
+                    native.ptr(pk_val), native.ptr(pk_pat), lay.G, lay.S, native.ptr(fp_val),
+                    native.ptr(fp_idx), lay.n, lay.m, native.dtype_code(self.val.dtype),
+                    native.stream_ptr(self.val.device)))
+            self._fragpack = (key, fp_val, fp_idx)
+        return self._fragpack[1], self._fragpack[2]
+
     def __repr__(self):
         lay = self.layout
         return (f"GroupedNMTensor(shape={tuple(lay.dense_shape)}, n:m:g={lay.n}:{lay.m}:{lay.group_size}, "
@@ -207,7 +233,6 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
     native.require_gpu(x, weight.val, bias)
     if x.dtype != weight.val.dtype:
         raise native.NmgError(f"dtype mismatch: activations {x.dtype}, weight {weight.val.dtype}")
-    pk_val, pk_pat = weight.rowpack()
     reduce_sparse = 1 if reduce_dim == lay.sparse_dim else 0
     K = lay.dense_shape[reduce_dim]
     O = lay.dense_shape[1 - reduce_dim]
@@ -220,6 +245,27 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
     if bias is not None:
         bias = bias.to(dtype=x.dtype).contiguous()
     kname = kernel or weight.spmm_opt.get("kernel", "auto")
+    variant = int(weight.spmm_opt.get("variant", 0))
+    smf_ok = (reduce_sparse == 1 and K % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+              and x.dtype in (torch.float16, torch.bfloat16))
+    if kname == "smfmac" or (kname == "auto" and smf_ok and T > 16):
+        packed = weight.fragpack() if smf_ok else None
+        if packed is None:
+            if kname == "smfmac":
+                raise native.NmgError(
+                    "the sparse-matrix-core kernel needs 16-bit data, a 2-of-4 compatible n:m "
+                    "pattern along the reduction dim and 16-byte aligned activations")
+        else:
+            with torch.cuda.device(x.device):
+                native.check(native.load().nmg_spmm_smfmac(
+                    native.ptr(packed[0]), native.ptr(packed[1]), O, K, native.ptr(x),
+                    x.stride(0) if T > 1 else K, native.ptr(y), O, native.ptr(bias), T,
+                    native.dtype_code(x.dtype), variant, native.stream_ptr(x.device)))
+            return y
+        kname = "auto"
+    if kname == "smfmac":
+        kname = "auto"
+    pk_val, pk_pat = weight.rowpack()
     with torch.cuda.device(x.device):
         native.check(native.load().nmg_spmm(
             native.ptr(pk_val), native.ptr(pk_pat), lay.G, lay.S, native.ptr(x),

@@ -188,3 +188,53 @@ def test_unregistered_op_raises_in_raise_mode():
         make(seeded((16, 16), torch.float32, 1), 2, 4, 1, 1), torch.zeros(1))
     with pytest.raises(sten.DispatchError):
         torch.relu(w)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,K,T,n,m,g", [
+    (768, 768, 256, 2, 4, 16),
+    (520, 1024, 300, 2, 4, 16),  # several workgroup tiles, ragged lines / tokens, K % 64 == 0
+    (200, 328, 77, 2, 4, 4),     # ragged lines / tokens, K not a multiple of 64
+    (96, 64, 33, 1, 4, 8),
+    (130, 520, 300, 2, 8, 4),
+    (64, 128, 40, 1, 8, 2),
+    (40, 16, 17, 1, 2, 3),
+])
+def test_spmm_sparse_matrix_cores(variant, dtype, M, K, T, n, m, g):
+    print(f"case smfmac v{variant} {dtype} M={M} K={K} T={T} {n}:{m}:{g}", flush=True)
+    W = seeded((M, K), dtype, seed=M + K + n, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, 1)
+    w = make(W, n, m, g, 1)
+    w.spmm_opt["variant"] = variant
+    x = seeded((T, K), dtype, seed=1)
+    b = seeded((M,), dtype, seed=2)
+    y = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1, kernel="smfmac")
+    ref = to_np(x).astype(np.float64) @ Wd.T + to_np(b).astype(np.float64)
+    assert rel_l2(to_np(y), ref) <= TOL[dtype]
+    y2 = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1, kernel="mfma")
+    assert rel_l2(to_np(y), to_np(y2)) <= 2 * TOL[dtype]
+
+
+def test_sparse_matrix_cores_refuse_incompatible_patterns():
+    w = make(seeded((64, 64), torch.float16, 1), 4, 8, 1, 1)     # 4:8 can keep 3 of an aligned 4
+    with pytest.raises(sten.NmgError):
+        sten.spmm(w, torch.zeros(32, 64, device=DEV).half(), reduce_dim=1, kernel="smfmac")
+    w32 = make(seeded((64, 64), torch.float32, 1), 2, 4, 4, 1)
+    with pytest.raises(sten.NmgError):
+        sten.spmm(w32, torch.zeros(32, 64, device=DEV), reduce_dim=1, kernel="smfmac")
+
+
+def test_full_size_config2_smfmac_vs_mfma_and_linearity():
+    # BASELINE config 2 at full size: the two independent kernels agree, and the op is linear in X
+    torch.manual_seed(0)
+    W = (torch.randn(4096, 4096) * 0.02).half()
+    X = torch.randn(2048, 4096).half().to(DEV)
+    w = make(W, 2, 4, 16, 1)
+    y_s = sten.spmm(w, X, reduce_dim=1, kernel="smfmac").float()
+    y_m = sten.spmm(w, X, reduce_dim=1, kernel="mfma").float()
+    assert float((y_s - y_m).norm() / y_m.norm()) <= 1e-3
+    ref = (X.float() @ w.to_dense().float().t())
+    assert float((y_s - ref).norm() / ref.norm()) <= 1e-3
+    y2 = sten.spmm(w, (2 * X), reduce_dim=1, kernel="smfmac").float()
+    assert float((y2 - 2 * y_s).norm() / y2.norm()) <= 1e-3
