@@ -258,30 +258,42 @@ __global__ __launch_bounds__(64 * WM * WN, MINW) void spmm_smfmac_kernel(SmfPara
 }
 
 // ------------------------------------------------------------------------ pipelined kernel
-// Same math, deeper memory pipeline: weight fragments, index words and the activation tile all
-// travel global -> LDS with the LDS-DMA form of global_load (no registers involved), into a ring
-// of PIPE_NS stages, so PIPE_NS-1 K steps of loads are in flight while one is being multiplied.
-// HBM / fabric latency on this part is several K steps long, which a one-step register prefetch
-// cannot cover.  Completion is tracked by hand with s_waitcnt vmcnt; one barrier per K step.
+// Same math, deeper memory pipeline and specialised wavefronts.
+//
+// Weight fragments, index words and the activation tile all travel global -> LDS with the
+// LDS-DMA form of global_load (no registers involved) into a ring of PIPE_NS stages, so
+// PIPE_NS-1 K steps of loads are in flight while one is being multiplied: HBM / fabric latency
+// is several K steps long, which a one-step register prefetch cannot cover.
+//
+// A workgroup has 8 wavefronts: 4 "matrix" wavefronts (one per SIMD, 128 features x 64 tokens
+// each) that only read fragments from LDS and issue MFMAs, and 4 "loader" wavefronts that only
+// issue the DMA loads and track their completion (s_waitcnt vmcnt is per wavefront).  A single
+// wavefront per SIMD is issue-bound: the DMA instructions, their address arithmetic and M0
+// updates do not fit in the shadow of its own MFMAs; a second wavefront on the SIMD issues them
+// in parallel.  One s_barrier per K step: loaders arrive when step kp+1 has landed, matrix
+// wavefronts when they hold all of step kp in registers; after it the loaders refill slot kp
+// and the matrix wavefronts start on step kp+1.
 //
 // Stage layout (bytes): [8 feature blocks x 2 k-steps x 1024] weight values in lane order,
 // [8 x 256] index words, [128 token rows x 128] activations.  A DMA load writes 64 lanes x 16 B
 // contiguously, so the activation rows cannot be padded; instead the 16-byte chunks of a row
 // are XOR-swizzled with (row/2)%8, chosen on the global side, which makes the fragment reads
 // (32 rows x 16 B at one logical chunk) conflict-free.
-// Requires K % 64 == 0.  Workgroup 256 features x 128 tokens, 2x2 wavefronts of 128 x 64.
+// Requires K % 64 == 0 and activations smaller than 2 GiB (32-bit lane offsets).
+// Workgroup tile 256 features x 128 tokens.
 constexpr int PIPE_NS = 4;
 constexpr int PIPE_AVAL = 8 * 2 * 1024;
 constexpr int PIPE_AIDX = 8 * 256;
 constexpr int PIPE_X = 128 * 128;
 constexpr int PIPE_STAGE = PIPE_AVAL + PIPE_AIDX + PIPE_X;
-constexpr int PIPE_LPT = 10;  // DMA loads issued per thread per stage: 4 weight + 2 index + 4 activation
+constexpr int PIPE_LPT = 10;  // DMA loads per loader thread per stage: 4 weight + 2 index + 4 activation
+constexpr int PIPE_OUT_ROW = 128 * 2 + 16;  // epilogue staging: one token row of a matrix wavefront
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
 typedef const __attribute__((address_space(1))) void *glb_ptr_t;
 
 template <typename T>
-__global__ __launch_bounds__(256, 1) void spmm_smfmac_pipe_kernel(SmfParams P)
+__global__ __launch_bounds__(512, 2) void spmm_smfmac_pipe_kernel(SmfParams P)
 {
     using S = Smf<T>;
     constexpr int FB = 4, TB = 2;
@@ -289,16 +301,91 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_pipe_kernel(SmfParams P)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
 
+    // Workgroup -> tile.  Consecutive ids are dealt round-robin to the 8 XCDs; give each XCD a
+    // contiguous run of ids, and walk the tile grid in bands of 4 feature tiles so that a run
+    // covers a compact block of tiles (weight rows and activation rows both reused from that
+    // XCD's L2).
     int id = blockIdx.x;
     const int ntiles = P.tiles_m * P.tiles_n;
     if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
-    const int tile_m = id / P.tiles_n, tile_n = id - tile_m * P.tiles_n;
+    constexpr int GH = 4;
+    const int band = id / (GH * P.tiles_n);
+    const int band_h = min(P.tiles_m - band * GH, GH);
+    const int in_band = id - band * GH * P.tiles_n;
+    const int tile_m = band * GH + in_band % band_h, tile_n = in_band / band_h;
     const int64_t f0 = (int64_t)tile_m * 256, t0 = (int64_t)tile_n * 128;
     const int KP = P.KP, KS = KP * 2;
     const int mbT = (int)(f0 / 32);
 
+    if (wave >= 4) {
+        // ============================== loader wavefronts ==============================
+        const int lw = wave - 4;
+        const unsigned char *av_base = (const unsigned char *)P.fp_val + (int64_t)mbT * KS * 1024;
+        const unsigned char *ai_base = (const unsigned char *)P.fp_idx + (int64_t)mbT * KP * 256;
+        const unsigned char *x_base = (const unsigned char *)P.x;
+        // weight values: loader lw moves fragments fi = 4lw..4lw+3 (fi = fb*2 + ks) of every stage
+        uint32_t av_off[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int fi = lw * 4 + i, fb = fi >> 1, ks = fi & 1;
+            av_off[i] = (uint32_t)(((fb * KS + ks) * 64 + lane) * 16);
+        }
+        // index words: loader lw moves feature blocks 2lw, 2lw+1
+        uint32_t ai_off[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) ai_off[i] = (uint32_t)((((lw * 2 + i) * KP) * 64 + lane) * 4);
+        // activations: loader lw moves row groups 4lw..4lw+3 (8 rows each); lane -> (row, piece)
+        uint32_t x_off[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int row = (lw * 4 + i) * 8 + (lane >> 3);
+            const int piece = lane & 7;
+            const int q = piece ^ ((row >> 1) & 7);   // logical chunk stored at this piece
+            int64_t tok = t0 + row;
+            if (tok >= P.T) tok = P.T - 1;            // clamped rows are computed, never stored
+            x_off[i] = (uint32_t)((tok * P.ldx + q * 8) * 2);
+        }
+        auto issue = [&](int kp, int stage) {
+            unsigned char *base = smem + stage * PIPE_STAGE;
+            const unsigned char *avb = av_base + (int64_t)kp * 2048;  // two k-steps of a feature block
+            const unsigned char *aib = ai_base + (int64_t)kp * 256;
+            const unsigned char *xb = x_base + (int64_t)kp * 128;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                __builtin_amdgcn_global_load_lds((glb_ptr_t)(avb + av_off[i]),
+                                                 (lds_ptr_t)(base + (lw * 4 + i) * 1024), 16, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                __builtin_amdgcn_global_load_lds((glb_ptr_t)(aib + ai_off[i]),
+                                                 (lds_ptr_t)(base + PIPE_AVAL + (lw * 2 + i) * 256), 4, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                __builtin_amdgcn_global_load_lds(
+                    (glb_ptr_t)(xb + x_off[i]),
+                    (lds_ptr_t)(base + PIPE_AVAL + PIPE_AIDX + (lw * 4 + i) * 1024), 16, 0, 0);
+        };
+        // Fill the ring (steps beyond KP-1 repeat the last one so the load count stays uniform).
+#pragma unroll
+        for (int st = 0; st < PIPE_NS; st++) issue(st < KP ? st : KP - 1, st);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((PIPE_NS - 1) * PIPE_LPT) : "memory");
+        asm volatile("s_barrier" ::: "memory");
+        for (int kp = 0; kp < KP; kp++) {
+            if (kp + PIPE_NS <= KP) {
+                // steps kp+1 .. kp+NS-1 are in flight; kp+1 has landed once NS-2 remain
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"((PIPE_NS - 2) * PIPE_LPT) : "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
+            asm volatile("s_barrier" ::: "memory");
+            if (kp + PIPE_NS < KP) issue(kp + PIPE_NS, kp & (PIPE_NS - 1));
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        return;
+    }
+
+    // ================================ matrix wavefronts ================================
+    const int wm = wave >> 1, wn = wave & 1;
     f32x16 acc[FB][TB];
 #pragma unroll
     for (int i = 0; i < FB; i++)
@@ -306,53 +393,6 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_pipe_kernel(SmfParams P)
         for (int j = 0; j < TB; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
-
-    // ---- DMA sources: wave-uniform base (advanced per K step on the scalar unit) plus a
-    //      32-bit per-lane byte offset ----
-    const unsigned char *av_base = (const unsigned char *)P.fp_val + (int64_t)mbT * KS * 1024;
-    const unsigned char *ai_base = (const unsigned char *)P.fp_idx + (int64_t)mbT * KP * 256;
-    const unsigned char *x_base = (const unsigned char *)P.x;
-    // weight values: wavefront w moves fragments fi = 4w..4w+3 (fi = fb*2 + ks) of every stage
-    uint32_t av_off[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int fi = wave * 4 + i, fb = fi >> 1, ks = fi & 1;
-        av_off[i] = (uint32_t)(((fb * KS + ks) * 64 + lane) * 16);
-    }
-    // index words: wavefront w moves feature blocks 2w, 2w+1
-    uint32_t ai_off[2];
-#pragma unroll
-    for (int i = 0; i < 2; i++) ai_off[i] = (uint32_t)((((wave * 2 + i) * KP) * 64 + lane) * 4);
-    // activations: wavefront w moves row groups 4w..4w+3 (8 rows each); lane -> (row, piece)
-    uint32_t x_off[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int row = (wave * 4 + i) * 8 + (lane >> 3);
-        const int piece = lane & 7;
-        const int q = piece ^ ((row >> 1) & 7);       // logical chunk stored at this piece
-        int64_t tok = t0 + row;
-        if (tok >= P.T) tok = P.T - 1;                // clamped rows are computed, never stored
-        x_off[i] = (uint32_t)((tok * P.ldx + q * 8) * 2);
-    }
-
-    auto issue = [&](int kp, int stage) {
-        unsigned char *base = smem + stage * PIPE_STAGE;
-        const unsigned char *avb = av_base + (int64_t)kp * 2048;   // two k-steps of one feature block
-        const unsigned char *aib = ai_base + (int64_t)kp * 256;
-        const unsigned char *xb = x_base + (int64_t)kp * 128;
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            __builtin_amdgcn_global_load_lds((glb_ptr_t)(avb + av_off[i]),
-                                             (lds_ptr_t)(base + (wave * 4 + i) * 1024), 16, 0, 0);
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-            __builtin_amdgcn_global_load_lds((glb_ptr_t)(aib + ai_off[i]),
-                                             (lds_ptr_t)(base + PIPE_AVAL + (wave * 2 + i) * 256), 4, 0, 0);
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[i]),
-                                             (lds_ptr_t)(base + PIPE_AVAL + PIPE_AIDX + (wave * 4 + i) * 1024), 16, 0, 0);
-    };
 
     // ---- fragment read offsets inside a stage ----
     const int a_off = (wm * FB) * 2 * 1024 + lane * 16;
@@ -407,23 +447,17 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_pipe_kernel(SmfParams P)
         }
     };
 
-    // Fill the ring: K steps 0..PIPE_NS-1 in flight, then wait for step 0.
-#pragma unroll
-    for (int st = 0; st < PIPE_NS; st++) issue(st < KP ? st : KP - 1, st);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((PIPE_NS - 1) * PIPE_LPT) : "memory");
-    asm volatile("s_barrier" ::: "memory");
+    asm volatile("s_barrier" ::: "memory");  // step 0 has landed
     read_frags(fr0, smem, 0);
 
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
     using IFB = std::integral_constant<int, FB>;
-    // Instruction-group masks of the scheduler: 0x008 MFMA, 0x020 VMEM read, 0x100 LDS read.
-    // One MFMA occupies the matrix pipe for ~32 cycles during which the wavefront can issue a
-    // handful of other instructions for free, so the LDS reads and DMA loads are dealt out a
-    // few per MFMA instead of in bursts between them.
+    // Instruction-group masks of the scheduler: 0x008 MFMA, 0x100 LDS read.  One MFMA occupies
+    // the matrix pipe for ~32 cycles during which the wavefront can issue a few other
+    // instructions for free, so the LDS reads are dealt out two per MFMA instead of in bursts.
     for (int kp = 0; kp < KP; kp++) {
-        const int slot = kp & (PIPE_NS - 1);
-        const unsigned char *base = smem + slot * PIPE_STAGE;
+        const unsigned char *base = smem + (kp & (PIPE_NS - 1)) * PIPE_STAGE;
         // ---- even k-step: MFMAs on set 0, fetch set 1 of the same stage ----
         read_frags(fr1, base, 1);
         mma(fr0, I0{}, I0{}, IFB{});
@@ -433,67 +467,78 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_pipe_kernel(SmfParams P)
             if (i < 5) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        // ---- odd k-step, first MFMA, then hand the stage back ----
+        // ---- odd k-step: two MFMAs, then hand the stage back ----
         mma(fr1, I1{}, I0{}, I1{});
         __builtin_amdgcn_sched_barrier(0);
-        // This wavefront holds all of stage kp in registers; once every wavefront does, the slot
-        // can be refilled with K step kp + PIPE_NS.  Step kp+1 must have landed to fetch its
-        // even-step fragments, which then load under the odd k-step's MFMAs.
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((PIPE_NS - 2) * PIPE_LPT) : "memory");
-        asm volatile("s_barrier" ::: "memory");
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // all of stage kp is in registers
+        asm volatile("s_barrier" ::: "memory");             // ... and step kp+1 has landed
         __builtin_amdgcn_sched_barrier(0);
-        {
-            const int nk = kp + PIPE_NS;
-            issue(nk < KP ? nk : KP - 1, slot);
-        }
         read_frags(fr0, smem + ((kp + 1) & (PIPE_NS - 1)) * PIPE_STAGE, 0);
         mma(fr1, I1{}, I1{}, IFB{});
 #pragma unroll
         for (int i = 0; i < (FB - 1) * TB; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i < 5) {
-                __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-            }
+            if (i < 5) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
     }
-    // drain the redundant tail loads before the LDS is released
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    uint16_t *Y = (uint16_t *)P.y;
-    const T *bias = (const T *)P.bias;
-    const bool vec_ok = (P.ldy & 3) == 0 && ((uintptr_t)P.y & 7) == 0;
+    // ---- epilogue: D[row = feature][col = token]; lane holds token l%32 and features
+    //      8*(r/4) + 4*(l/32) + r%4.  Stage the wavefront's 64 tokens x 128 features through
+    //      its own LDS region as [token][feature] so the global stores are 16 B per lane and
+    //      256 B contiguous per token row.  (All DMA traffic has drained: the loaders waited for
+    //      vmcnt(0) before the last barrier.) ----
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    unsigned char *stg = smem + wave * (64 * PIPE_OUT_ROW);
 #pragma unroll
-    for (int tb = 0; tb < TB; tb++) {
-        const int64_t tok = t0 + (wn * TB + tb) * 32 + (lane & 31);
-        if (tok >= P.T) continue;
+    for (int tb = 0; tb < TB; tb++)
 #pragma unroll
-        for (int fb = 0; fb < FB; fb++) {
+        for (int fb = 0; fb < FB; fb++)
 #pragma unroll
             for (int rq = 0; rq < 4; rq++) {
-                const int64_t f = f0 + (wm * FB + fb) * 32 + rq * 8 + (lane >> 5) * 4;
-                if (f >= P.M) continue;
                 uint16_t hh[4];
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    float v = acc[fb][tb][rq * 4 + i];
-                    if (bias && f + i < P.M) v += to_f32(bias[f + i]);
-                    hh[i] = f32_to_bits16(v, (T *)nullptr);
-                }
-                uint16_t *dst = Y + tok * P.ldy + f;
-                if (vec_ok && f + 3 < P.M) {
-                    uint2 pk;
-                    pk.x = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
-                    pk.y = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
-                    *(uint2 *)dst = pk;
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        if (f + i < P.M) dst[i] = hh[i];
-                }
+                for (int i = 0; i < 4; i++) hh[i] = f32_to_bits16(acc[fb][tb][rq * 4 + i], (T *)nullptr);
+                uint2 pk;
+                pk.x = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
+                pk.y = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
+                *(uint2 *)(stg + (tb * 32 + j) * PIPE_OUT_ROW + (fb * 32 + rq * 8 + h * 4) * 2) = pk;
             }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    uint16_t *Y = (uint16_t *)P.y;
+    const T *bias = (const T *)P.bias;
+    const bool vec_ok = (P.ldy & 7) == 0 && ((uintptr_t)P.y & 15) == 0;
+    const int fc = lane & 15;                       // 8-feature chunk of the row
+    const int64_t f = f0 + wm * 128 + fc * 8;
+    float bv[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) bv[i] = (bias && f + i < P.M) ? to_f32(bias[f + i]) : 0.f;
+#pragma unroll 4
+    for (int it = 0; it < 16; it++) {
+        const int tl = it * 4 + (lane >> 4);
+        const int64_t tok = t0 + wn * 64 + tl;
+        u32x4 v = *(const u32x4 *)(stg + tl * PIPE_OUT_ROW + fc * 16);
+        if (tok >= P.T || f >= P.M) continue;
+        if (bias) {
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint16_t lo = (uint16_t)(w[i] & 0xFFFF), hi = (uint16_t)(w[i] >> 16);
+                T tlo = *reinterpret_cast<T *>(&lo), thi = *reinterpret_cast<T *>(&hi);
+                lo = f32_to_bits16(to_f32(tlo) + bv[2 * i], (T *)nullptr);
+                hi = f32_to_bits16(to_f32(thi) + bv[2 * i + 1], (T *)nullptr);
+                w[i] = (uint32_t)lo | ((uint32_t)hi << 16);
+            }
+            v.x = w[0]; v.y = w[1]; v.z = w[2]; v.w = w[3];
+        }
+        uint16_t *dst = Y + tok * P.ldy + f;
+        if (vec_ok && f + 7 < P.M) {
+            *(u32x4 *)dst = v;
+        } else {
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                if (f + i < P.M) dst[i] = (uint16_t)(w[i >> 1] >> ((i & 1) * 16));
         }
     }
 }
@@ -504,9 +549,10 @@ template <typename T> static int launch_smfmac_pipe(SmfParams &P, hipStream_t s)
     P.tiles_n = (int)((P.T + 127) / 128);
     dim3 grid((unsigned)(P.tiles_m * P.tiles_n));
     const size_t lds = (size_t)PIPE_NS * PIPE_STAGE;
+    static_assert(PIPE_NS * PIPE_STAGE >= 4 * 64 * PIPE_OUT_ROW, "epilogue staging must fit in the ring");
     auto k = spmm_smfmac_pipe_kernel<T>;
     NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(k, grid, dim3(256), lds, s, P);
+    hipLaunchKernelGGL(k, grid, dim3(512), lds, s, P);
     NMG_HIP_TRY(hipGetLastError());
     return NMG_OK;
 }
@@ -683,7 +729,8 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
     case 2: return launch_smfmac_cfg<T, 2, 2, 2, 4, 2>(P, s);  // 128 x 256
     case 3: return launch_smfmac_cfg<T, 4, 1, 2, 4, 2>(P, s);  // 256 x 128, waves stacked on lines
     case 4:                                                     // 256 x 128, LDS-DMA ring
-        if (P.K % 64 != 0) return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
+        if (P.K % 64 != 0 || P.T * P.ldx * 2 >= (int64_t)1 << 31)
+            return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
         return launch_smfmac_pipe<T>(P, s);
     }
     return NMG_ERR_ARG;

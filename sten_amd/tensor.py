@@ -245,7 +245,7 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
     if bias is not None:
         bias = bias.to(dtype=x.dtype).contiguous()
     kname = kernel or weight.spmm_opt.get("kernel", "auto")
-    variant = int(weight.spmm_opt.get("variant", 0))
+    variant = int(weight.spmm_opt.get("variant", 4))
     smf_ok = (reduce_sparse == 1 and K % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
               and x.dtype in (torch.float16, torch.bfloat16))
     if kname == "smfmac" or (kname == "auto" and smf_ok and T > 16):
