@@ -557,6 +557,123 @@ template <typename T> static int launch_smfmac_pipe(SmfParams &P, hipStream_t s)
     return NMG_OK;
 }
 
+// --------------------------------------------------------------------------- decode kernel
+// Few tokens (T <= 16): the weight is streamed once from HBM and everything else is noise, so
+// the kernel is built around keeping many coalesced 1 KiB fragment loads in flight.  The sparse
+// matrix core still does the arithmetic -- tokens are padded to the 32 columns of one MFMA,
+// which costs nothing when the kernel is bandwidth-bound and spares any cross-lane reduction.
+// One workgroup owns a block of 32 lines; its SK_NW wavefronts split K, keep two batches of
+// loads in flight (fetch batch i+1, multiply batch i), accumulate in registers, and are summed
+// through LDS at the end.  (Splitting K over several workgroups as well was tried and dropped:
+// the device-scope fences it needs write back and invalidate the XCD's L2 and cost 10x.)
+constexpr int SK_NW = 16;
+constexpr int SK_UNROLL = 2;   // k pairs (64 dense k each) fetched per batch
+
+template <typename T>
+__global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_skinny_kernel(SmfParams P)
+{
+    using S = Smf<T>;
+    __shared__ float red[SK_NW][32][17];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int mb = blockIdx.x;
+    const int KP = P.KP;
+    const int j = lane & 31, h = lane >> 5;
+    const u32x4 zero4 = {0, 0, 0, 0};
+    // this wavefront's k pairs: a contiguous slice
+    const int per = (KP + SK_NW - 1) / SK_NW;
+    const int kp_lo = wave * per, kp_hi = min(KP, kp_lo + per);
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+
+    const u32x4 *aval = (const u32x4 *)P.fp_val + ((int64_t)mb * KP * 2) * 64 + lane;
+    const uint32_t *aidx = P.fp_idx + ((int64_t)mb * KP) * 64 + lane;
+    const bool tok_ok = j < P.T;
+    const unsigned char *xrow = (const unsigned char *)P.x + ((int64_t)(tok_ok ? j : 0) * P.ldx + 16 * h) * 2;
+
+    struct Batch {
+        u32x4 a[SK_UNROLL][2], b[SK_UNROLL][2][2];
+        uint32_t ix[SK_UNROLL];
+    };
+    auto fetch = [&](Batch &B, int kp0) {
+#pragma unroll
+        for (int u = 0; u < SK_UNROLL; u++) {
+            const int kp = kp0 + u;
+            const bool live = kp < kp_hi;
+            B.a[u][0] = live ? aval[(int64_t)kp * 128] : zero4;
+            B.a[u][1] = live ? aval[(int64_t)kp * 128 + 64] : zero4;
+            B.ix[u] = live ? aidx[(int64_t)kp * 64] : 0x44444444u;
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                for (int c = 0; c < 2; c++) {
+                    const int64_t k = (int64_t)kp * 64 + ks * 32 + 16 * h + 8 * c;
+                    B.b[u][ks][c] = (live && tok_ok && k < P.K)
+                                        ? *(const u32x4 *)(xrow + ((int64_t)kp * 64 + ks * 32 + 8 * c) * 2)
+                                        : zero4;
+                }
+        }
+    };
+    auto consume = [&](const Batch &B) {
+#pragma unroll
+        for (int u = 0; u < SK_UNROLL; u++) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                union {
+                    u32x4 u4;
+                    typename S::A v;
+                } ca;
+                ca.u4 = B.a[u][ks];
+                union {
+                    u32x4 u4[2];
+                    typename S::B v;
+                } cb;
+                cb.u4[0] = B.b[u][ks][0];
+                cb.u4[1] = B.b[u][ks][1];
+                if (ks == 0)
+                    acc = S::template run<0>(ca.v, cb.v, acc, (int)B.ix[u]);
+                else
+                    acc = S::template run<1>(ca.v, cb.v, acc, (int)B.ix[u]);
+            }
+        }
+    };
+
+    Batch b0, b1;
+    fetch(b0, kp_lo);
+    for (int kp0 = kp_lo; kp0 < kp_hi; kp0 += 2 * SK_UNROLL) {
+        fetch(b1, kp0 + SK_UNROLL);
+        consume(b0);
+        fetch(b0, kp0 + 2 * SK_UNROLL);
+        consume(b1);
+    }
+    // D[row = line][col = token]: lane holds token j, lines 8*(r/4) + 4*h + r%4
+    if (j < 16) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) red[wave][(r >> 2) * 8 + h * 4 + (r & 3)][j] = acc[r];
+    }
+    __syncthreads();
+    // 32 lines x 16 tokens = 512 sums over SK_NW partials
+    for (int e = tid; e < 32 * 16; e += 64 * SK_NW) {
+        const int line = e & 31, tok = e >> 5;
+        const int64_t f = (int64_t)mb * 32 + line;
+        if (tok >= P.T || f >= P.M) continue;
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < SK_NW; w++) s += red[w][line][tok];
+        if (P.bias) s += to_f32(((const T *)P.bias)[f]);
+        ((uint16_t *)P.y)[tok * P.ldy + f] = f32_to_bits16(s, (T *)nullptr);
+    }
+}
+
+template <typename T> static int launch_smfmac_skinny(SmfParams &P, hipStream_t s)
+{
+    dim3 grid((unsigned)((P.M + 31) / 32));
+    hipLaunchKernelGGL((spmm_smfmac_skinny_kernel<T>), grid, dim3(64 * SK_NW), 0, s, P);
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
 // ------------------------------------------------------------------------------ fragpack
 struct FragpackParams {
     const void *pk_val;   // rowpack values [G, nb, n]
@@ -728,6 +845,9 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
     case 1: return launch_smfmac_cfg<T, 2, 2, 2, 2, 2>(P, s);  // 128 x 128, 2 waves/SIMD
     case 2: return launch_smfmac_cfg<T, 2, 2, 2, 4, 2>(P, s);  // 128 x 256
     case 3: return launch_smfmac_cfg<T, 4, 1, 2, 4, 2>(P, s);  // 256 x 128, waves stacked on lines
+    case 5:                                                     // decode shapes, T <= 16
+        if (P.T > 16) return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
+        return launch_smfmac_skinny<T>(P, s);
     case 4:                                                     // 256 x 128, LDS-DMA ring
         if (P.K % 64 != 0 || P.T * P.ldx * 2 >= (int64_t)1 << 31)
             return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
@@ -743,7 +863,7 @@ extern "C" int nmg_spmm_smfmac(const void *d_fp_val, const void *d_fp_idx, int64
     NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED,
                 "the sparse matrix cores take f16/bf16 only");
     NMG_REQUIRE(M >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
-    NMG_REQUIRE(variant >= 0 && variant <= 4, NMG_ERR_ARG, "unknown tile variant %d", variant);
+    NMG_REQUIRE(variant >= 0 && variant <= 5, NMG_ERR_ARG, "unknown tile variant %d", variant);
     NMG_REQUIRE(ldx >= K && ldy >= M, NMG_ERR_ARG, "leading dimension smaller than row length");
     NMG_REQUIRE((K % 8) == 0 && (ldx % 8) == 0 && ((uintptr_t)d_x % 16) == 0, NMG_ERR_UNSUPPORTED,
                 "activations must be 16-byte aligned with K and ldx multiples of 8");

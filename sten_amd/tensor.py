@@ -248,23 +248,24 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
     variant = int(weight.spmm_opt.get("variant", 4))
     smf_ok = (reduce_sparse == 1 and K % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
               and x.dtype in (torch.float16, torch.bfloat16))
-    if kname == "smfmac" or (kname == "auto" and smf_ok and T > 16):
-        packed = weight.fragpack() if smf_ok else None
-        if packed is None:
-            if kname == "smfmac":
-                raise native.NmgError(
-                    "the sparse-matrix-core kernel needs 16-bit data, a 2-of-4 compatible n:m "
-                    "pattern along the reduction dim and 16-byte aligned activations")
-        else:
-            with torch.cuda.device(x.device):
-                native.check(native.load().nmg_spmm_smfmac(
-                    native.ptr(packed[0]), native.ptr(packed[1]), O, K, native.ptr(x),
-                    x.stride(0) if T > 1 else K, native.ptr(y), O, native.ptr(bias), T,
-                    native.dtype_code(x.dtype), variant, native.stream_ptr(x.device)))
-            return y
-        kname = "auto"
-    if kname == "smfmac":
-        kname = "auto"
+    if kname == "skinny" and T > 16:
+        raise native.NmgError("the skinny kernel serves at most 16 tokens")
+    packed = None
+    if smf_ok and kname in ("auto", "skinny", "smfmac"):
+        packed = weight.fragpack()
+    if kname == "smfmac" and packed is None:
+        raise native.NmgError(
+            "the sparse-matrix-core kernel needs 16-bit data, a 2-of-4 compatible n:m "
+            "pattern along the reduction dim and 16-byte aligned activations")
+    if packed is not None:
+        if T <= 16 and kname in ("auto", "skinny"):
+            variant = 5                 # decode shapes: streaming kernel on the same operand
+        with torch.cuda.device(x.device):
+            native.check(native.load().nmg_spmm_smfmac(
+                native.ptr(packed[0]), native.ptr(packed[1]), O, K, native.ptr(x),
+                x.stride(0) if T > 1 else K, native.ptr(y), O, native.ptr(bias), T,
+                native.dtype_code(x.dtype), variant, native.stream_ptr(x.device)))
+        return y
     pk_val, pk_pat = weight.rowpack()
     with torch.cuda.device(x.device):
         native.check(native.load().nmg_spmm(
