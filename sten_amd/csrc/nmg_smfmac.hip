@@ -566,10 +566,8 @@ template <typename T> static int launch_smfmac_pipe(SmfParams &P, hipStream_t s)
 // loads in flight (fetch batch i+1, multiply batch i), accumulate in registers, and are summed
 // through LDS at the end.  (Splitting K over several workgroups as well was tried and dropped:
 // the device-scope fences it needs write back and invalidate the XCD's L2 and cost 10x.)
-constexpr int SK_NW = 16;
-constexpr int SK_UNROLL = 2;   // k pairs (64 dense k each) fetched per batch
-
-template <typename T>
+// SK_NW wavefronts per workgroup, SK_UNROLL k pairs (64 dense k each) fetched per batch.
+template <typename T, int SK_NW, int SK_UNROLL>
 __global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_skinny_kernel(SmfParams P)
 {
     using S = Smf<T>;
@@ -666,10 +664,10 @@ __global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_skinny_kernel(SmfParam
     }
 }
 
-template <typename T> static int launch_smfmac_skinny(SmfParams &P, hipStream_t s)
+template <typename T, int NW, int UN> static int launch_smfmac_skinny(SmfParams &P, hipStream_t s)
 {
     dim3 grid((unsigned)((P.M + 31) / 32));
-    hipLaunchKernelGGL((spmm_smfmac_skinny_kernel<T>), grid, dim3(64 * SK_NW), 0, s, P);
+    hipLaunchKernelGGL((spmm_smfmac_skinny_kernel<T, NW, UN>), grid, dim3(64 * NW), 0, s, P);
     NMG_HIP_TRY(hipGetLastError());
     return NMG_OK;
 }
@@ -847,7 +845,10 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
     case 3: return launch_smfmac_cfg<T, 4, 1, 2, 4, 2>(P, s);  // 256 x 128, waves stacked on lines
     case 5:                                                     // decode shapes, T <= 16
         if (P.T > 16) return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
-        return launch_smfmac_skinny<T>(P, s);
+        // few line blocks: many wavefronts per workgroup keep enough loads in flight per CU;
+        // many line blocks: small workgroups pack several per CU and balance better
+        if ((P.M + 31) / 32 >= 256) return launch_smfmac_skinny<T, 4, 4>(P, s);
+        return launch_smfmac_skinny<T, 16, 1>(P, s);
     case 4:                                                     // 256 x 128, LDS-DMA ring
         if (P.K % 64 != 0 || P.T * P.ldx * 2 >= (int64_t)1 << 31)
             return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
