@@ -12,6 +12,8 @@
 // outputs of one token row and the stores to row-major Y are contiguous.
 #include "nmg_common.h"
 
+#include <cstdlib>
+
 namespace nmg {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -234,6 +236,11 @@ __global__ __launch_bounds__(256) void spmm_skinny_kernel(SpmmParams P)
     }
 }
 
+bool dense_pipe_supports(int n, int m);
+int spmm_dense_pipe(const void *pk_val, const void *pk_pat, const int8_t *d_order, int64_t G, int64_t S,
+                    const void *x, int64_t ldx, void *y, int64_t ldy, const void *bias, int64_t T,
+                    int reduce_sparse, int n, int m, int dtype, hipStream_t s);
+
 template <typename T> static int launch_spmm(SpmmParams &P, int reduce_sparse, int kernel, hipStream_t s)
 {
     if (kernel == NMG_KERNEL_SKINNY) {
@@ -299,6 +306,13 @@ extern "C" int nmg_spmm(const void *d_pk_val, const void *d_pk_pat, int64_t G, i
     P.c = (int)binom(m, n);
     P.pat_bytes = (int)nmg_rowpack_pat_bytes(n, m);
     hipStream_t s = (hipStream_t)stream;
+    // Large 16-bit problems go to the pipelined dense-MFMA kernel (nmg_dense.hip); the simple
+    // tiled kernel below keeps serving f32, ragged K, unusual n:m and explicit requests.
+    if (kernel == NMG_KERNEL_MFMA && (dtype == NMG_F16 || dtype == NMG_BF16) && T > 16 &&
+        dense_pipe_supports(n, m) && P.K % 64 == 0 && P.K >= 64 && (ldx % 8) == 0 && ((uintptr_t)d_x % 16) == 0 &&
+        T * ldx * 2 < ((int64_t)1 << 31) && binom(m, n) <= 256 && !getenv("NMG_SIMPLE_MFMA"))
+        return spmm_dense_pipe(d_pk_val, d_pk_pat, P.order, G, S, d_x, ldx, d_y, ldy, d_bias, T,
+                               reduce_sparse, n, m, dtype, s);
     switch (dtype) {
     case NMG_F32: return launch_spmm<float>(P, reduce_sparse, kernel, s);
     case NMG_F16: return launch_spmm<__half>(P, reduce_sparse, kernel, s);

@@ -14,7 +14,8 @@ LIB_PATH = os.path.join(_HERE, "libnmg_hip.so")
 
 NMG_F32, NMG_F16, NMG_BF16, NMG_F64 = 0, 1, 2, 3
 KERNEL_AUTO, KERNEL_MFMA, KERNEL_SMFMAC, KERNEL_SKINNY = 0, 1, 2, 3
-KERNELS = {"auto": KERNEL_AUTO, "mfma": KERNEL_MFMA, "smfmac": KERNEL_SMFMAC, "skinny": KERNEL_SKINNY}
+KERNELS = {"auto": KERNEL_AUTO, "mfma": KERNEL_MFMA, "smfmac": KERNEL_SMFMAC, "skinny": KERNEL_SKINNY,
+           "expand": KERNEL_MFMA}
 
 DTYPE_CODE = {
     torch.float32: NMG_F32,
@@ -52,6 +53,7 @@ SIGNATURES = {
     "nmg_fragpack_sizes": (_I, [_I64, _I64, ctypes.POINTER(_I64), ctypes.POINTER(_I64)]),
     "nmg_fragpack": (_I, [_P, _P, _I64, _I64, _P, _P, _I, _I, _I, _P]),
     "nmg_spmm_smfmac": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _P]),
+    "nmg_gemm_nt": (_I, [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I, _P]),
 }
 
 _lib = None

@@ -190,6 +190,24 @@ class GroupedNMTensor:
             self._rowpack = (key, pk_val, pk_pat)
         return self._rowpack[1], self._rowpack[2]
 
+    def dense_operand(self, reduce_dim):
+        """Dense copy [outputs, reduction] of the weight (transposed when the reduction runs along
+        dim 0), written by the to_dense kernel into fresh scratch; not cached."""
+        lay = self.layout
+        native.require_gpu(self.val)
+        O, K = lay.dense_shape[1 - reduce_dim], lay.dense_shape[reduce_dim]
+        out = torch.empty((O, K), dtype=self.val.dtype, device=self.val.device)
+        # element (dim0 = i, dim1 = j) of the weight lives at out[i, j] (reduce_dim == 1) or out[j, i]
+        s0, s1 = (K, 1) if reduce_dim == 1 else (1, K)
+        strides = (s0, s1)
+        view = native.NmgView(1, lay.G, lay.S, 0, strides[lay.group_dim], strides[lay.sparse_dim])
+        with torch.cuda.device(out.device):
+            native.check(native.load().nmg_to_dense(
+                native.ptr(self.val), native.ptr(self.idx), native.ptr(out), ctypes.byref(view),
+                lay.n, lay.m, lay.group_size, native.dtype_code(out.dtype),
+                native.stream_ptr(out.device)))
+        return out
+
     def fragpack(self):
         """Operand of the sparse-matrix-core kernel (values + 2-bit positions in instruction
         register order); ``None`` when the n:m pattern does not fit 2-of-4 groups or the dtype is
@@ -266,6 +284,21 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
                 x.stride(0) if T > 1 else K, native.ptr(y), O, native.ptr(bias), T,
                 native.dtype_code(x.dtype), variant, native.stream_ptr(x.device)))
         return y
+    if (kname in ("auto", "mfma", "expand") and T > 16 and x.dtype in (torch.float16, torch.bfloat16)
+            and K % 64 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+            and T * x.stride(0) * 2 < 2 ** 31 and O * K * 2 < 2 ** 31
+            and (kname == "expand" or weight.spmm_opt.get("expand", True))):
+        # "expand, then multiply": write the dense weight with the reduction contiguous into
+        # scratch (one HBM-bound pass) and run the pipelined dense-MFMA kernel on it
+        a = weight.dense_operand(reduce_dim)
+        with torch.cuda.device(x.device):
+            native.check(native.load().nmg_gemm_nt(
+                native.ptr(a), K, native.ptr(x), x.stride(0), native.ptr(y), O, native.ptr(bias),
+                O, K, T, native.dtype_code(x.dtype), native.stream_ptr(x.device)))
+        return y
+    if kname == "expand":
+        raise native.NmgError("the expand-then-multiply route needs 16-bit data, more than 16 tokens "
+                              "and a reduction extent that is a multiple of 64")
     pk_val, pk_pat = weight.rowpack()
     with torch.cuda.device(x.device):
         native.check(native.load().nmg_spmm(

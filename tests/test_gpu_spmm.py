@@ -238,3 +238,38 @@ def test_full_size_config2_smfmac_vs_mfma_and_linearity():
     assert float((y_s - ref).norm() / ref.norm()) <= 1e-3
     y2 = sten.spmm(w, (2 * X), reduce_dim=1, kernel="smfmac").float()
     assert float((y2 - 2 * y_s).norm() / y2.norm()) <= 1e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,K,T,n,m,g", [
+    (512, 640, 300, 2, 4, 16),     # several workgroup tiles in both directions, ragged tokens
+    (320, 256, 130, 4, 8, 2),      # pattern that does not fit 2-of-4 groups
+    (264, 192, 77, 3, 4, 4),
+    (520, 128, 40, 1, 8, 4),
+    (256, 320, 129, 2, 8, 2),
+    (192, 64, 33, 1, 2, 8),
+])
+def test_dense_pipeline_kernel_both_directions(dtype, M, K, T, n, m, g):
+    # kernel="mfma" with 16-bit data and reduction extents that are multiples of 64 runs the
+    # pipelined dense-MFMA kernel: forward (reduce along the sparse dim) and the transposed product
+    # (reduce along the group dim), the latter being grad_input of F.linear
+    print(f"case dense-pipe {dtype} M={M} K={K} T={T} {n}:{m}:{g}", flush=True)
+    W = seeded((M, K), dtype, seed=M + K + n, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, 1)
+    w = make(W, n, m, g, 1)
+    x = seeded((T, K), dtype, seed=1)
+    b = seeded((M,), dtype, seed=2)
+    ref = to_np(x).astype(np.float64) @ Wd.T + to_np(b).astype(np.float64)
+    gy = seeded((T, M), dtype, seed=3)
+    for expand in (False, True):     # weights expanded inside the kernel / into scratch first
+        w.spmm_opt["expand"] = expand
+        y = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1, kernel="mfma")
+        assert rel_l2(to_np(y), ref) <= TOL[dtype], expand
+        if M % 64 == 0:
+            gx = sten.spmm(w, gy.to(DEV), reduce_dim=0, kernel="mfma")
+            assert rel_l2(to_np(gx), to_np(gy).astype(np.float64) @ Wd) <= TOL[dtype], expand
+    # the reference orientation (n:m along dim 0): forward reduces along the group dim
+    w0 = make(W, n, m, g, 0)
+    Wd0, _ = dense_ref(W, n, m, g, 0)
+    y0 = sten.spmm(w0, x.to(DEV), reduce_dim=1, kernel="expand")
+    assert rel_l2(to_np(y0), to_np(x).astype(np.float64) @ Wd0.T) <= TOL[dtype]
