@@ -257,6 +257,75 @@ __global__ __launch_bounds__(64 * WM * WN, MINW) void spmm_smfmac_kernel(SmfPara
     }
 }
 
+constexpr int PIPE_OUT_ROW = 128 * 2 + 16;  // epilogue staging: one token row of a matrix wavefront
+
+// Epilogue shared by the pipelined kernels.  D[row = feature][col = token]; a lane holds token
+// l%32 and features 8*(r/4) + 4*(l/32) + r%4.  The wavefront's TB*32 tokens x FB*32 features are
+// staged through its own LDS region `stg` as [token][feature] so the global stores are 16 B per
+// lane and FB*64 B contiguous per token row.  fw / tw = first feature / token of the wavefront.
+// The caller guarantees that no load into LDS is pending.
+template <typename T, int FB, int TB>
+__device__ __forceinline__ void smf_store_tile(const f32x16 (&acc)[FB][TB], unsigned char *stg, int lane,
+                                               int64_t fw, int64_t tw, const SmfParams &P)
+{
+    constexpr int ROW = FB * 64 + 16;       // bytes per staged token row (16 B pad: conflict-free)
+    constexpr int CPR = FB * 4;             // 16-byte chunks per row
+    constexpr int RPP = 64 / CPR;           // token rows per pass of the wavefront
+    const int j = lane & 31, h = lane >> 5;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int tb = 0; tb < TB; tb++)
+#pragma unroll
+        for (int fb = 0; fb < FB; fb++)
+#pragma unroll
+            for (int rq = 0; rq < 4; rq++) {
+                uint16_t hh[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) hh[i] = f32_to_bits16(acc[fb][tb][rq * 4 + i], (T *)nullptr);
+                uint2 pk;
+                pk.x = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
+                pk.y = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
+                *(uint2 *)(stg + (tb * 32 + j) * ROW + (fb * 32 + rq * 8 + h * 4) * 2) = pk;
+            }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    uint16_t *Y = (uint16_t *)P.y;
+    const T *bias = (const T *)P.bias;
+    const bool vec_ok = (P.ldy & 7) == 0 && ((uintptr_t)P.y & 15) == 0;
+    const int fc = lane % CPR;                      // 8-feature chunk of the row
+    const int64_t f = fw + fc * 8;
+    float bv[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) bv[i] = (bias && f + i < P.M) ? to_f32(bias[f + i]) : 0.f;
+#pragma unroll 4
+    for (int it = 0; it < TB * 32 / RPP; it++) {
+        const int tl = it * RPP + lane / CPR;
+        const int64_t tok = tw + tl;
+        u32x4 v = *(const u32x4 *)(stg + tl * ROW + fc * 16);
+        if (tok >= P.T || f >= P.M) continue;
+        if (bias) {
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint16_t lo = (uint16_t)(w[i] & 0xFFFF), hi = (uint16_t)(w[i] >> 16);
+                T tlo = *reinterpret_cast<T *>(&lo), thi = *reinterpret_cast<T *>(&hi);
+                lo = f32_to_bits16(to_f32(tlo) + bv[2 * i], (T *)nullptr);
+                hi = f32_to_bits16(to_f32(thi) + bv[2 * i + 1], (T *)nullptr);
+                w[i] = (uint32_t)lo | ((uint32_t)hi << 16);
+            }
+            v.x = w[0]; v.y = w[1]; v.z = w[2]; v.w = w[3];
+        }
+        uint16_t *dst = Y + tok * P.ldy + f;
+        if (vec_ok && f + 7 < P.M) {
+            *(u32x4 *)dst = v;
+        } else {
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                if (f + i < P.M) dst[i] = (uint16_t)(w[i >> 1] >> ((i & 1) * 16));
+        }
+    }
+}
+
 // ------------------------------------------------------------------------ pipelined kernel
 // Same math, deeper memory pipeline and specialised wavefronts.
 //
@@ -287,7 +356,6 @@ constexpr int PIPE_AIDX = 8 * 256;
 constexpr int PIPE_X = 128 * 128;
 constexpr int PIPE_STAGE = PIPE_AVAL + PIPE_AIDX + PIPE_X;
 constexpr int PIPE_LPT = 10;  // DMA loads per loader thread per stage: 4 weight + 2 index + 4 activation
-constexpr int PIPE_OUT_ROW = 128 * 2 + 16;  // epilogue staging: one token row of a matrix wavefront
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
 typedef const __attribute__((address_space(1))) void *glb_ptr_t;
@@ -483,64 +551,7 @@ __global__ __launch_bounds__(512, 2) void spmm_smfmac_pipe_kernel(SmfParams P)
         __builtin_amdgcn_sched_barrier(0);
     }
 
-    // ---- epilogue: D[row = feature][col = token]; lane holds token l%32 and features
-    //      8*(r/4) + 4*(l/32) + r%4.  Stage the wavefront's 64 tokens x 128 features through
-    //      its own LDS region as [token][feature] so the global stores are 16 B per lane and
-    //      256 B contiguous per token row.  (All DMA traffic has drained: the loaders waited for
-    //      vmcnt(0) before the last barrier.) ----
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    unsigned char *stg = smem + wave * (64 * PIPE_OUT_ROW);
-#pragma unroll
-    for (int tb = 0; tb < TB; tb++)
-#pragma unroll
-        for (int fb = 0; fb < FB; fb++)
-#pragma unroll
-            for (int rq = 0; rq < 4; rq++) {
-                uint16_t hh[4];
-#pragma unroll
-                for (int i = 0; i < 4; i++) hh[i] = f32_to_bits16(acc[fb][tb][rq * 4 + i], (T *)nullptr);
-                uint2 pk;
-                pk.x = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
-                pk.y = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
-                *(uint2 *)(stg + (tb * 32 + j) * PIPE_OUT_ROW + (fb * 32 + rq * 8 + h * 4) * 2) = pk;
-            }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    uint16_t *Y = (uint16_t *)P.y;
-    const T *bias = (const T *)P.bias;
-    const bool vec_ok = (P.ldy & 7) == 0 && ((uintptr_t)P.y & 15) == 0;
-    const int fc = lane & 15;                       // 8-feature chunk of the row
-    const int64_t f = f0 + wm * 128 + fc * 8;
-    float bv[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) bv[i] = (bias && f + i < P.M) ? to_f32(bias[f + i]) : 0.f;
-#pragma unroll 4
-    for (int it = 0; it < 16; it++) {
-        const int tl = it * 4 + (lane >> 4);
-        const int64_t tok = t0 + wn * 64 + tl;
-        u32x4 v = *(const u32x4 *)(stg + tl * PIPE_OUT_ROW + fc * 16);
-        if (tok >= P.T || f >= P.M) continue;
-        if (bias) {
-            uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                uint16_t lo = (uint16_t)(w[i] & 0xFFFF), hi = (uint16_t)(w[i] >> 16);
-                T tlo = *reinterpret_cast<T *>(&lo), thi = *reinterpret_cast<T *>(&hi);
-                lo = f32_to_bits16(to_f32(tlo) + bv[2 * i], (T *)nullptr);
-                hi = f32_to_bits16(to_f32(thi) + bv[2 * i + 1], (T *)nullptr);
-                w[i] = (uint32_t)lo | ((uint32_t)hi << 16);
-            }
-            v.x = w[0]; v.y = w[1]; v.z = w[2]; v.w = w[3];
-        }
-        uint16_t *dst = Y + tok * P.ldy + f;
-        if (vec_ok && f + 7 < P.M) {
-            *(u32x4 *)dst = v;
-        } else {
-            uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int i = 0; i < 8; i++)
-                if (f + i < P.M) dst[i] = (uint16_t)(w[i >> 1] >> ((i & 1) * 16));
-        }
-    }
+    smf_store_tile<T, FB, TB>(acc, smem + wave * (64 * PIPE_OUT_ROW), lane, f0 + wm * 128, t0 + wn * 64, P);
 }
 
 template <typename T> static int launch_smfmac_pipe(SmfParams &P, hipStream_t s)
@@ -553,6 +564,229 @@ template <typename T> static int launch_smfmac_pipe(SmfParams &P, hipStream_t s)
     auto k = spmm_smfmac_pipe_kernel<T>;
     NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(k, grid, dim3(512), lds, s, P);
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
+// ------------------------------------------------------------- pipelined kernel, direct weights
+// The fragpack operand is already in the register order of the instruction, so the weight
+// fragments do not have to pass through LDS at all: each wavefront fetches its own fragments and
+// index words from global memory into a ring of DR_D+1 register sets, DR_D K steps ahead of their
+// use, and LDS carries the activation tile only.
+//
+// What bounds these kernels is the path from L2 through the CU's vector cache (64 B per clock):
+// with the MFMAs alone a K step takes 0.29 us, with the LDS reads 0.33 us, and every KiB that a
+// K step pulls through the vector cache adds to that.  So the wavefronts are stacked on the
+// feature dim (WM = 4, each 64 features x all tokens of the tile): no two wavefronts fetch the
+// same weight fragment, and a workgroup moves 18 KiB of weights + 16 KiB of activations per
+// K step, the minimum for its tile.
+//
+// A workgroup is 4 wavefronts, one per SIMD, with the whole register file of the SIMD to
+// itself; each also issues its quarter of the activation tile's DMA loads.  Every K step a
+// wavefront issues XL DMA loads and 3*FB register loads for step kp+DR_D, so "step kp+1 has
+// landed" is vmcnt <= OPS*(DR_D-1); the barrier that follows publishes the activation rows of
+// all four wavefronts.  Tile order, swizzle and preconditions as in the kernel above.
+constexpr int DR_D = 3;                 // K steps in flight
+constexpr int DR_NS = 4;                // activation stages in LDS (>= DR_D + 1)
+
+template <typename T, int FB, int TB, int WM, int WN>
+__global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
+{
+    using S = Smf<T>;
+    static_assert(WM * WN == 4, "four wavefronts");
+    constexpr int TF = WM * FB * 32, TT = WN * TB * 32;   // workgroup tile: features x tokens
+    constexpr int STAGE = TT * 128;                       // activation bytes per K step
+    constexpr int XL = TT / 32;                           // DMA loads per wavefront per K step
+    constexpr int OPS = XL + 3 * FB;                      // memory operations per wavefront per K step
+    static_assert(OPS * DR_D < 64, "vmcnt is a 6-bit counter");
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    int id = blockIdx.x;
+    const int ntiles = P.tiles_m * P.tiles_n;
+    if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
+    constexpr int GH = 4;
+    const int band = id / (GH * P.tiles_n);
+    const int band_h = min(P.tiles_m - band * GH, GH);
+    const int in_band = id - band * GH * P.tiles_n;
+    const int tile_m = band * GH + in_band % band_h, tile_n = in_band / band_h;
+    const int64_t f0 = (int64_t)tile_m * TF, t0 = (int64_t)tile_n * TT;
+    const int KP = P.KP, KS = KP * 2;
+    const int wm = wave / WN, wn = wave % WN;
+    const int mb0 = (int)(f0 / 32) + wm * FB;
+
+    // ---- global sources (wavefront-uniform bases in scalar registers, the lane's share as a
+    //      32-bit offset) ----
+    const unsigned char *av_base[FB];
+    const unsigned char *ai_base[FB];
+#pragma unroll
+    for (int fb = 0; fb < FB; fb++) {
+        av_base[fb] = (const unsigned char *)P.fp_val + ((int64_t)(mb0 + fb) * KS) * 1024;
+        ai_base[fb] = (const unsigned char *)P.fp_idx + ((int64_t)(mb0 + fb) * KP) * 256;
+    }
+    const uint32_t lane16 = lane * 16, lane4 = lane * 4;
+    const unsigned char *x_base = (const unsigned char *)P.x;
+    uint32_t x_off[XL];
+#pragma unroll
+    for (int i = 0; i < XL; i++) {
+        const int row = (wave * XL + i) * 8 + (lane >> 3);
+        const int piece = lane & 7;
+        const int q = piece ^ ((row >> 1) & 7);
+        int64_t tok = t0 + row;
+        if (tok >= P.T) tok = P.T - 1;
+        x_off[i] = (uint32_t)((tok * P.ldx + q * 8) * 2);
+    }
+
+    struct WSet {
+        u32x4 a[FB][2];
+        uint32_t ix[FB];
+    };
+    WSet ws[DR_D + 1];
+    // Steps beyond the last repeat it: the operation count stays uniform, the data is unused.
+    auto issue_x = [&](int kp) {
+        if (kp >= KP) kp = KP - 1;
+        unsigned char *base = smem + (kp & (DR_NS - 1)) * STAGE;
+        const unsigned char *xb = x_base + (int64_t)kp * 128;
+#pragma unroll
+        for (int i = 0; i < XL; i++)
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[i]),
+                                             (lds_ptr_t)(base + (wave * XL + i) * 1024), 16, 0, 0);
+    };
+    auto issue_a = [&](int kp, WSet &w) {
+        if (kp >= KP) kp = KP - 1;
+#pragma unroll
+        for (int fb = 0; fb < FB; fb++) {
+            // Written as instructions so that their completion is tracked by the explicit vmcnt
+            // waits below and by nothing else (left to itself the compiler waits for vmcnt(0) at
+            // the loop head, which empties the pipeline every K step), and with accumulation
+            // registers as targets: the ring does not fit beside the accumulators in the 256
+            // architectural registers, and a compiler-made copy of a register whose load is
+            // still in flight would copy stale data.
+            const unsigned char *av = av_base[fb] + (int64_t)kp * 2048;
+            const unsigned char *ai = ai_base[fb] + (int64_t)kp * 256;
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=a"(w.a[fb][0]) : "v"(lane16), "s"(av) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=a"(w.a[fb][1]) : "v"(lane16), "s"(av) : "memory");
+            asm volatile("global_load_dword %0, %1, %2" : "=v"(w.ix[fb]) : "v"(lane4), "s"(ai) : "memory");
+        }
+    };
+
+    f32x16 acc[FB][TB];
+#pragma unroll
+    for (int i = 0; i < FB; i++)
+#pragma unroll
+        for (int j = 0; j < TB; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    const int j = lane & 31, h = lane >> 5, sw = (j >> 1) & 7;
+    int b_off[2][2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+            b_off[ks][c] = (wn * TB * 32 + j) * 128 + (((ks * 4 + h * 2 + c) ^ sw) << 4);
+
+    struct BFrags {
+        u32x4 b[TB][2];
+    };
+    BFrags fr0, fr1;
+    auto read_b = [&](BFrags &f, const unsigned char *base, int ks) {
+#pragma unroll
+        for (int tb = 0; tb < TB; tb++) {
+            f.b[tb][0] = *(const u32x4 *)(base + b_off[ks][0] + tb * 32 * 128);
+            f.b[tb][1] = *(const u32x4 *)(base + b_off[ks][1] + tb * 32 * 128);
+        }
+    };
+    // MFMAs lo..hi-1 of a k-step, numbered fb * TB + tb
+    auto mma = [&](const WSet &w, const BFrags &f, auto ks_tag, int lo, int hi) {
+        constexpr int KSI = decltype(ks_tag)::value;
+#pragma unroll
+        for (int fb = 0; fb < FB; fb++) {
+            union {
+                u32x4 u;
+                typename S::A v;
+            } ca;
+            ca.u = w.a[fb][KSI];
+#pragma unroll
+            for (int tb = 0; tb < TB; tb++) {
+                if (fb * TB + tb < lo || fb * TB + tb >= hi) continue;
+                union {
+                    u32x4 u[2];
+                    typename S::B v;
+                } cb;
+                cb.u[0] = f.b[tb][0];
+                cb.u[1] = f.b[tb][1];
+                acc[fb][tb] = S::template run<KSI>(ca.v, cb.v, acc[fb][tb], (int)w.ix[fb]);
+            }
+        }
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    constexpr int NM = FB * TB;             // MFMAs per k-step
+
+    // prologue: steps 0 .. DR_D-1 in flight, then wait for step 0
+#pragma unroll
+    for (int st = 0; st < DR_D; st++) {
+        issue_x(st);
+        issue_a(st, ws[st]);
+    }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DR_D - 1) * OPS) : "memory");
+    asm volatile("s_barrier" ::: "memory");
+    read_b(fr0, smem, 0);
+
+    for (int kp0 = 0; kp0 < KP; kp0 += DR_D + 1) {
+#pragma unroll
+        for (int u = 0; u <= DR_D; u++) {
+            const int kp = kp0 + u;
+            if (kp >= KP) break;
+            const unsigned char *base = smem + (kp & (DR_NS - 1)) * STAGE;
+            // The instruction statements fence the scheduler, so the order below is the issue
+            // order: two MFMAs, the LDS reads of the odd k-step, then the loads of step kp+DR_D
+            // dealt out between the remaining MFMAs of the even k-step.
+            mma(ws[u], fr0, I0{}, 0, 2);
+            __builtin_amdgcn_sched_barrier(0);
+            read_b(fr1, base, 1);
+            issue_x(kp + DR_D);
+            mma(ws[u], fr0, I0{}, 2, 4);
+            issue_a(kp + DR_D, ws[(u + DR_D) % (DR_D + 1)]);
+            mma(ws[u], fr0, I0{}, 4, NM);
+            mma(ws[u], fr1, I1{}, 0, 2);
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // activation fragments of step kp are in registers
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DR_D - 1) * OPS) : "memory");  // my share of kp+1 landed
+            asm volatile("s_barrier" ::: "memory");              // ... and everybody else's
+            __builtin_amdgcn_sched_barrier(0);
+            read_b(fr0, smem + ((kp + 1) & (DR_NS - 1)) * STAGE, 0);
+            mma(ws[u], fr1, I1{}, 2, NM);
+#pragma unroll
+            for (int i = 0; i < TB; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_barrier" ::: "memory");
+    smf_store_tile<T, FB, TB>(acc, smem + wave * (TB * 32 * (FB * 64 + 16)), lane, f0 + wm * FB * 32,
+                              t0 + wn * TB * 32, P);
+}
+
+template <typename T, int FB, int TB, int WM, int WN> static int launch_smfmac_direct(SmfParams &P, hipStream_t s)
+{
+    constexpr int TF = WM * FB * 32, TT = WN * TB * 32;
+    static_assert(TF == 256, "the operand is padded to 256 lines");
+    P.tiles_m = (int)((P.M + TF - 1) / TF);
+    P.tiles_n = (int)((P.T + TT - 1) / TT);
+    dim3 grid((unsigned)(P.tiles_m * P.tiles_n));
+    constexpr size_t ring = (size_t)DR_NS * TT * 128, stg = (size_t)4 * TB * 32 * (FB * 64 + 16);
+    constexpr size_t lds = ring > stg ? ring : stg;
+    static_assert(lds <= 160 * 1024, "LDS");
+    auto k = spmm_smfmac_direct_kernel<T, FB, TB, WM, WN>;
+    NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(k, grid, dim3(256), lds, s, P);
     NMG_HIP_TRY(hipGetLastError());
     return NMG_OK;
 }
@@ -853,6 +1087,12 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
         if (P.K % 64 != 0 || P.T * P.ldx * 2 >= (int64_t)1 << 31)
             return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
         return launch_smfmac_pipe<T>(P, s);
+    case 6:                                                     // 256 x 128, weights straight to registers
+    case 7:                                                     // same, wavefronts 2 x 2 (shared weight fetches)
+        if (P.K % 64 != 0 || P.T * P.ldx * 2 >= (int64_t)1 << 31)
+            return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
+        if (variant == 7) return launch_smfmac_direct<T, 4, 2, 2, 2>(P, s);
+        return launch_smfmac_direct<T, 2, 4, 4, 1>(P, s);
     }
     return NMG_ERR_ARG;
 }
@@ -864,7 +1104,7 @@ extern "C" int nmg_spmm_smfmac(const void *d_fp_val, const void *d_fp_idx, int64
     NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED,
                 "the sparse matrix cores take f16/bf16 only");
     NMG_REQUIRE(M >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
-    NMG_REQUIRE(variant >= 0 && variant <= 5, NMG_ERR_ARG, "unknown tile variant %d", variant);
+    NMG_REQUIRE(variant >= 0 && variant <= 7, NMG_ERR_ARG, "unknown tile variant %d", variant);
     NMG_REQUIRE(ldx >= K && ldy >= M, NMG_ERR_ARG, "leading dimension smaller than row length");
     NMG_REQUIRE((K % 8) == 0 && (ldx % 8) == 0 && ((uintptr_t)d_x % 16) == 0, NMG_ERR_UNSUPPORTED,
                 "activations must be 16-byte aligned with K and ldx multiples of 8");

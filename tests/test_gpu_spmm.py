@@ -190,10 +190,12 @@ def test_unregistered_op_raises_in_raise_mode():
         torch.relu(w)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 6, 7])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M,K,T,n,m,g", [
     (768, 768, 256, 2, 4, 16),
+    (512, 64, 128, 2, 4, 16),    # a single K step
+    (256, 320, 100, 2, 4, 16),   # K steps not a multiple of the pipeline depth
     (520, 1024, 300, 2, 4, 16),  # several workgroup tiles, ragged lines / tokens, K % 64 == 0
     (200, 328, 77, 2, 4, 4),     # ragged lines / tokens, K not a multiple of 64
     (96, 64, 33, 1, 4, 8),
