@@ -98,7 +98,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--kernel", default="auto")
-    ap.add_argument("--variant", type=int, default=4)
+    ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true")
     args = ap.parse_args()

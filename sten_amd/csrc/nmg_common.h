@@ -28,8 +28,8 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line);
     } while (0)
 
 // ---- pattern order tables -----------------------------------------------------------------
-constexpr int kOrderSlotBytes = 8192;  // c*n int8 entries of one (n, m) pair
-constexpr int kOrderSlots = 8;
+constexpr int kOrderSlotBytes = 8192;      // largest table: c*n int8 entries of one (n, m) pair
+constexpr int kOrderPoolBytes = 64 * 1024;  // all tables of one device, packed 16-byte aligned
 
 int64_t binom(int m, int n);
 // Host copy of the table (cached per (n, m)); nullptr when (n, m) is invalid.

@@ -544,6 +544,72 @@ int spmm_dense_pipe(const void *pk_val, const void *pk_pat, const int8_t *d_orde
                             : launch_dense<__hip_bfloat16>(P, reduce_sparse, n, m, s);
 }
 
+// ------------------------------------------------------------------ rowpack -> dense weight
+// Expands the rowpack operand into a plain dense matrix, either as [lines, positions] or
+// transposed, through an LDS tile of 64 lines x (up to) 128 positions so that both the reads
+// (values in rowpack order) and the writes (whole rows of the tile) are contiguous.
+constexpr int EX_L = 64, EX_P = 128;
+
+struct ExpandParams {
+    const void *pk_val;
+    const void *pk_pat;
+    void *out;
+    const int8_t *order;
+    int64_t G, S, nb, ld;
+    int n, m, pat_bytes, bpt, transpose;   // bpt = blocks per tile
+};
+
+template <typename T> __global__ __launch_bounds__(256) void expand_kernel(ExpandParams P)
+{
+    // [64][128 + pad] or, transposed, [128][64 + pad]; pad keeps 16-byte rows and spreads banks
+    constexpr int PAD = 16 / sizeof(T);
+    __shared__ __align__(16) T tile[EX_L * (EX_P + PAD) > EX_P * (EX_L + PAD) ? EX_L * (EX_P + PAD)
+                                                                             : EX_P * (EX_L + PAD)];
+    const int tid = threadIdx.x;
+    const int tp = P.bpt * P.m;                              // positions per tile
+    const int64_t q0 = (int64_t)blockIdx.y * EX_L, b0 = (int64_t)blockIdx.x * P.bpt;
+    const int rows = P.transpose ? tp : EX_L, cols = P.transpose ? EX_L : tp;
+    const int pitch = (P.transpose ? EX_L : EX_P) + PAD;
+    for (int i = tid; i < rows * pitch; i += 256) tile[i] = Zero<T>::v();
+    __syncthreads();
+    const T *pv = (const T *)P.pk_val;
+    const int per_line = P.bpt * P.n;
+    for (int i = tid; i < EX_L * per_line; i += 256) {
+        const int ql = i / per_line, r = i - ql * per_line;
+        const int bl = r / P.n, j = r - bl * P.n;
+        const int64_t q = q0 + ql, b = b0 + bl;
+        if (q >= P.G || b >= P.nb) continue;
+        const int64_t blk = q * P.nb + b;
+        const int pat = P.pat_bytes == 1 ? (int)((const uint8_t *)P.pk_pat)[blk]
+                                         : (int)((const uint16_t *)P.pk_pat)[blk];
+        const int pos = bl * P.m + P.order[pat * P.n + j];
+        const T v = pv[blk * P.n + j];
+        if (P.transpose)
+            tile[pos * pitch + ql] = v;
+        else
+            tile[ql * pitch + pos] = v;
+    }
+    __syncthreads();
+    // rows of the tile -> global, 16 bytes per lane where the row is aligned
+    T *out = (T *)P.out;
+    const int64_t r0 = P.transpose ? b0 * P.m : q0, c0 = P.transpose ? q0 : b0 * P.m;
+    const int64_t R = P.transpose ? P.S : P.G, C = P.transpose ? P.G : P.S;
+    constexpr int V = 16 / sizeof(T);
+    const bool vec = (P.ld % V) == 0 && (c0 % V) == 0 && ((uintptr_t)P.out % 16) == 0;
+    const int cv = (cols + V - 1) / V;
+    for (int i = tid; i < rows * cv; i += 256) {
+        const int r = i / cv, cc = (i - r * cv) * V;
+        if (r0 + r >= R || c0 + cc >= C) continue;
+        T *dst = out + (r0 + r) * P.ld + c0 + cc;
+        const T *src = tile + r * pitch + cc;
+        if (vec && cc + V <= cols && c0 + cc + V <= C) {
+            *(uint4 *)dst = *(const uint4 *)src;
+        } else {
+            for (int e = 0; e < V && cc + e < cols && c0 + cc + e < C; e++) dst[e] = src[e];
+        }
+    }
+}
+
 }  // namespace nmg
 
 using namespace nmg;
@@ -579,4 +645,42 @@ extern "C" int nmg_gemm_nt(const void *d_a, int64_t lda, const void *d_x, int64_
     hipStream_t s = (hipStream_t)stream;
     return dtype == NMG_F16 ? launch_dense_nm<__half, 0, 4>(P, 1, s)
                             : launch_dense_nm<__hip_bfloat16, 0, 4>(P, 1, s);
+}
+
+extern "C" int nmg_rowpack_expand(const void *d_pk_val, const void *d_pk_pat, int64_t G, int64_t S,
+                                  void *d_out, int64_t ld_out, int transpose, int n, int m, int dtype,
+                                  void *stream)
+{
+    NMG_REQUIRE(m >= 1 && m <= 64 && n >= 0 && n <= m, NMG_ERR_ARG, "invalid n:m = %d:%d", n, m);
+    NMG_REQUIRE(dtype == NMG_F32 || dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED,
+                "rowpack supports f32/f16/bf16");
+    NMG_REQUIRE(G >= 0 && S >= 0, NMG_ERR_ARG, "negative extent");
+    NMG_REQUIRE(ld_out >= (transpose ? G : S), NMG_ERR_ARG, "leading dimension smaller than row length");
+    if (G == 0 || S == 0) return NMG_OK;
+    NMG_REQUIRE(d_pk_val && d_pk_pat && d_out, NMG_ERR_ARG, "null device pointer");
+    ExpandParams P{};
+    if (int rc = device_order(n, m, &P.order)) return rc;
+    P.pk_val = d_pk_val;
+    P.pk_pat = d_pk_pat;
+    P.out = d_out;
+    P.G = G;
+    P.S = S;
+    P.nb = (S + m - 1) / m;
+    P.ld = ld_out;
+    P.n = n;
+    P.m = m;
+    P.pat_bytes = binom(m, n) <= 256 ? 1 : 2;
+    P.bpt = EX_P / m;
+    P.transpose = transpose ? 1 : 0;
+    const int64_t gx = (P.nb + P.bpt - 1) / P.bpt, gy = (G + EX_L - 1) / EX_L;
+    NMG_REQUIRE(gx <= 0x7fffffffLL && gy <= 65535, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
+    dim3 grid((unsigned)gx, (unsigned)gy);
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+    case NMG_F32: hipLaunchKernelGGL(expand_kernel<float>, grid, dim3(256), 0, s, P); break;
+    case NMG_F16: hipLaunchKernelGGL(expand_kernel<__half>, grid, dim3(256), 0, s, P); break;
+    case NMG_BF16: hipLaunchKernelGGL(expand_kernel<__hip_bfloat16>, grid, dim3(256), 0, s, P); break;
+    }
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
 }

@@ -79,11 +79,12 @@ const int8_t *host_order(int n, int m)
 }
 
 // Device-side table: one file-scope array per GPU, addressed through hipGetSymbolAddress.
-static __device__ __align__(256) int8_t g_order_dev[kOrderSlots * kOrderSlotBytes];
+static __device__ __align__(256) int8_t g_order_dev[kOrderPoolBytes];
 
 struct DevTables {
     int8_t *base = nullptr;
-    std::vector<std::pair<int, int>> slots;
+    size_t used = 0;                                   // bytes of the pool handed out
+    std::map<std::pair<int, int>, size_t> offset;      // (n, m) -> offset of its table
 };
 static std::map<int, DevTables> g_dev_tables;
 
@@ -104,16 +105,19 @@ int device_order(int n, int m, const int8_t **d_order)
         NMG_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(g_order_dev)));
         dt.base = (int8_t *)p;
     }
-    for (size_t i = 0; i < dt.slots.size(); i++)
-        if (dt.slots[i] == std::make_pair(n, m)) {
-            *d_order = dt.base + i * kOrderSlotBytes;
-            return NMG_OK;
-        }
-    NMG_REQUIRE((int)dt.slots.size() < kOrderSlots, NMG_ERR_UNSUPPORTED,
-                "more than %d distinct n:m pairs used on one device", kOrderSlots);
-    int8_t *dst = dt.base + dt.slots.size() * kOrderSlotBytes;
+    auto it = dt.offset.find(std::make_pair(n, m));
+    if (it != dt.offset.end()) {
+        *d_order = dt.base + it->second;
+        return NMG_OK;
+    }
+    const size_t need = ((size_t)bytes + 15) & ~(size_t)15;
+    NMG_REQUIRE(dt.used + need <= (size_t)kOrderPoolBytes, NMG_ERR_UNSUPPORTED,
+                "pattern tables of this device are full (%d bytes): too many distinct n:m pairs",
+                kOrderPoolBytes);
+    int8_t *dst = dt.base + dt.used;
     if (bytes > 0) NMG_HIP_TRY(hipMemcpy(dst, h, (size_t)bytes, hipMemcpyHostToDevice));
-    dt.slots.emplace_back(n, m);
+    dt.offset.emplace(std::make_pair(n, m), dt.used);
+    dt.used += need > 0 ? need : 16;
     *d_order = dst;
     return NMG_OK;
 }

@@ -589,16 +589,21 @@ template <typename T> static int launch_smfmac_pipe(SmfParams &P, hipStream_t s)
 constexpr int DR_D = 3;                 // K steps in flight
 constexpr int DR_NS = 4;                // activation stages in LDS (>= DR_D + 1)
 
-template <typename T, int FB, int TB, int WM, int WN>
+template <typename T, int FB, int TB, int WM, int WN, int NH>
 __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
 {
     using S = Smf<T>;
     static_assert(WM * WN == 4, "four wavefronts");
+    static_assert(TB % NH == 0, "token blocks split evenly into phases");
     constexpr int TF = WM * FB * 32, TT = WN * TB * 32;   // workgroup tile: features x tokens
     constexpr int STAGE = TT * 128;                       // activation bytes per K step
     constexpr int XL = TT / 32;                           // DMA loads per wavefront per K step
     constexpr int OPS = XL + 3 * FB;                      // memory operations per wavefront per K step
+    constexpr int BT = TB / NH;                           // token blocks per phase
+    constexpr int NP = 2 * NH;                            // phases per K step: (k-step, token part)
+    constexpr int NM = FB * BT;                           // MFMAs per phase
     static_assert(OPS * DR_D < 64, "vmcnt is a 6-bit counter");
+    static_assert(NM >= 4, "phase too short to hide the loads behind");
     extern __shared__ __align__(16) unsigned char smem[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -680,6 +685,17 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
+    // 256 accumulators fill the architectural registers exactly; left alone the allocator
+    // puts them all there and spills everything else.  Pin half of them to the accumulation
+    // registers (the MFMA takes its C/D operand from either file).
+    auto pin_acc = [&]() {
+        if constexpr (FB * TB * 16 > 128) {
+#pragma unroll
+            for (int tb = 0; tb < TB; tb++) asm volatile("" : "+a"(acc[FB - 1][tb]));
+        }
+    };
+    pin_acc();
+
     const int j = lane & 31, h = lane >> 5, sw = (j >> 1) & 7;
     int b_off[2][2];
 #pragma unroll
@@ -688,20 +704,22 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
         for (int c = 0; c < 2; c++)
             b_off[ks][c] = (wn * TB * 32 + j) * 128 + (((ks * 4 + h * 2 + c) ^ sw) << 4);
 
+    // Activation fragments of one phase (k-step ks, token part hh); two sets alternate.
     struct BFrags {
-        u32x4 b[TB][2];
+        u32x4 b[BT][2];
     };
-    BFrags fr0, fr1;
-    auto read_b = [&](BFrags &f, const unsigned char *base, int ks) {
+    BFrags fr[2];
+    auto read_b = [&](BFrags &f, const unsigned char *base, int ph) {
+        const int ks = ph / NH, hh = ph % NH;
 #pragma unroll
-        for (int tb = 0; tb < TB; tb++) {
-            f.b[tb][0] = *(const u32x4 *)(base + b_off[ks][0] + tb * 32 * 128);
-            f.b[tb][1] = *(const u32x4 *)(base + b_off[ks][1] + tb * 32 * 128);
+        for (int t = 0; t < BT; t++) {
+            f.b[t][0] = *(const u32x4 *)(base + b_off[ks][0] + (hh * BT + t) * 32 * 128);
+            f.b[t][1] = *(const u32x4 *)(base + b_off[ks][1] + (hh * BT + t) * 32 * 128);
         }
     };
-    // MFMAs lo..hi-1 of a k-step, numbered fb * TB + tb
-    auto mma = [&](const WSet &w, const BFrags &f, auto ks_tag, int lo, int hi) {
-        constexpr int KSI = decltype(ks_tag)::value;
+    // MFMAs lo..hi-1 of phase PH, numbered fb * BT + t
+    auto mma = [&](const WSet &w, const BFrags &f, auto ph_tag, int lo, int hi) {
+        constexpr int PH = decltype(ph_tag)::value, KSI = PH / NH, HH = PH % NH;
 #pragma unroll
         for (int fb = 0; fb < FB; fb++) {
             union {
@@ -710,21 +728,18 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
             } ca;
             ca.u = w.a[fb][KSI];
 #pragma unroll
-            for (int tb = 0; tb < TB; tb++) {
-                if (fb * TB + tb < lo || fb * TB + tb >= hi) continue;
+            for (int t = 0; t < BT; t++) {
+                if (fb * BT + t < lo || fb * BT + t >= hi) continue;
                 union {
                     u32x4 u[2];
                     typename S::B v;
                 } cb;
-                cb.u[0] = f.b[tb][0];
-                cb.u[1] = f.b[tb][1];
-                acc[fb][tb] = S::template run<KSI>(ca.v, cb.v, acc[fb][tb], (int)w.ix[fb]);
+                cb.u[0] = f.b[t][0];
+                cb.u[1] = f.b[t][1];
+                acc[fb][HH * BT + t] = S::template run<KSI>(ca.v, cb.v, acc[fb][HH * BT + t], (int)w.ix[fb]);
             }
         }
     };
-    using I0 = std::integral_constant<int, 0>;
-    using I1 = std::integral_constant<int, 1>;
-    constexpr int NM = FB * TB;             // MFMAs per k-step
 
     // prologue: steps 0 .. DR_D-1 in flight, then wait for step 0
 #pragma unroll
@@ -734,7 +749,7 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
     }
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DR_D - 1) * OPS) : "memory");
     asm volatile("s_barrier" ::: "memory");
-    read_b(fr0, smem, 0);
+    read_b(fr[0], smem, 0);
 
     for (int kp0 = 0; kp0 < KP; kp0 += DR_D + 1) {
 #pragma unroll
@@ -742,39 +757,63 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
             const int kp = kp0 + u;
             if (kp >= KP) break;
             const unsigned char *base = smem + (kp & (DR_NS - 1)) * STAGE;
-            // The instruction statements fence the scheduler, so the order below is the issue
-            // order: two MFMAs, the LDS reads of the odd k-step, then the loads of step kp+DR_D
-            // dealt out between the remaining MFMAs of the even k-step.
-            mma(ws[u], fr0, I0{}, 0, 2);
-            __builtin_amdgcn_sched_barrier(0);
-            read_b(fr1, base, 1);
-            issue_x(kp + DR_D);
-            mma(ws[u], fr0, I0{}, 2, 4);
-            issue_a(kp + DR_D, ws[(u + DR_D) % (DR_D + 1)]);
-            mma(ws[u], fr0, I0{}, 4, NM);
-            mma(ws[u], fr1, I1{}, 0, 2);
-            __builtin_amdgcn_sched_barrier(0);
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // activation fragments of step kp are in registers
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DR_D - 1) * OPS) : "memory");  // my share of kp+1 landed
-            asm volatile("s_barrier" ::: "memory");              // ... and everybody else's
-            __builtin_amdgcn_sched_barrier(0);
-            read_b(fr0, smem + ((kp + 1) & (DR_NS - 1)) * STAGE, 0);
-            mma(ws[u], fr1, I1{}, 2, NM);
+            const unsigned char *next = smem + ((kp + 1) & (DR_NS - 1)) * STAGE;
+            // One phase: two MFMAs; the LDS reads of the next phase into the other fragment set;
+            // in the first phases the loads of step kp+DR_D; the rest of the MFMAs.  Before the
+            // reads of the last phase, which fetch from the next stage, the barrier.  The
+            // instruction statements fence the scheduler, so this is also the issue order.
+            auto phase = [&](auto ph_tag) {
+                constexpr int PH = decltype(ph_tag)::value;
+                mma(ws[u], fr[PH % 2], ph_tag, 0, 2);
+                __builtin_amdgcn_sched_barrier(0);
+                if (PH == NP - 1) {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // fragments of step kp are in registers
+                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DR_D - 1) * OPS) : "memory");  // my share of kp+1 landed
+                    asm volatile("s_barrier" ::: "memory");              // ... and everybody else's
+                    __builtin_amdgcn_sched_barrier(0);
+                    read_b(fr[(PH + 1) % 2], next, 0);
+                } else {
+                    read_b(fr[(PH + 1) % 2], base, PH + 1);
+                }
+                if (PH == 0) {
+                    issue_x(kp + DR_D);
+                    if (NP == 2) {
+                        mma(ws[u], fr[PH % 2], ph_tag, 2, 4);
+                        issue_a(kp + DR_D, ws[(u + DR_D) % (DR_D + 1)]);
+                        mma(ws[u], fr[PH % 2], ph_tag, 4, NM);
+                    } else {
+                        mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
+                    }
+                } else if (PH == 1 && NP > 2) {
+                    issue_a(kp + DR_D, ws[(u + DR_D) % (DR_D + 1)]);
+                    mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
+                } else {
+                    mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
 #pragma unroll
-            for (int i = 0; i < TB; i++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    for (int i = 0; i < BT; i++) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            phase(std::integral_constant<int, 0>{});
+            phase(std::integral_constant<int, 1>{});
+            if constexpr (NP == 4) {
+                phase(std::integral_constant<int, 2>{});
+                phase(std::integral_constant<int, 3>{});
             }
-            __builtin_amdgcn_sched_barrier(0);
+            static_assert(NP == 2 || NP == 4, "one or two token parts");
         }
     }
+    pin_acc();
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     asm volatile("s_barrier" ::: "memory");
     smf_store_tile<T, FB, TB>(acc, smem + wave * (TB * 32 * (FB * 64 + 16)), lane, f0 + wm * FB * 32,
                               t0 + wn * TB * 32, P);
 }
 
-template <typename T, int FB, int TB, int WM, int WN> static int launch_smfmac_direct(SmfParams &P, hipStream_t s)
+template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_smfmac_direct(SmfParams &P, hipStream_t s)
 {
     constexpr int TF = WM * FB * 32, TT = WN * TB * 32;
     static_assert(TF == 256, "the operand is padded to 256 lines");
@@ -784,7 +823,7 @@ template <typename T, int FB, int TB, int WM, int WN> static int launch_smfmac_d
     constexpr size_t ring = (size_t)DR_NS * TT * 128, stg = (size_t)4 * TB * 32 * (FB * 64 + 16);
     constexpr size_t lds = ring > stg ? ring : stg;
     static_assert(lds <= 160 * 1024, "LDS");
-    auto k = spmm_smfmac_direct_kernel<T, FB, TB, WM, WN>;
+    auto k = spmm_smfmac_direct_kernel<T, FB, TB, WM, WN, NH>;
     NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(k, grid, dim3(256), lds, s, P);
     NMG_HIP_TRY(hipGetLastError());
@@ -1072,6 +1111,15 @@ static int launch_smfmac_cfg(SmfParams &P, hipStream_t s)
 
 template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStream_t s)
 {
+    if (variant < 0) {
+        // Large-batch default.  The 256 x 256 tile moves a quarter fewer bytes per flop through
+        // the vector caches and runs a tile pair in ~0.8 of the time of two 256 x 128 tiles, but
+        // there are half as many tiles to spread over the 256 CUs: compare rounds of tiles.
+        const int64_t tm = (P.M + 255) / 256;
+        const int64_t n128 = tm * ((P.T + 127) / 128), n256 = tm * ((P.T + 255) / 256);
+        const double cost128 = (double)((n128 + 255) / 256), cost256 = 1.6 * (double)((n256 + 255) / 256);
+        variant = cost256 < cost128 ? 8 : 6;
+    }
     switch (variant) {
     case 0: return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);  // 256 lines x 128 tokens, 1 wave/SIMD
     case 1: return launch_smfmac_cfg<T, 2, 2, 2, 2, 2>(P, s);  // 128 x 128, 2 waves/SIMD
@@ -1089,10 +1137,12 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
         return launch_smfmac_pipe<T>(P, s);
     case 6:                                                     // 256 x 128, weights straight to registers
     case 7:                                                     // same, wavefronts 2 x 2 (shared weight fetches)
+    case 8:                                                     // 256 x 256
         if (P.K % 64 != 0 || P.T * P.ldx * 2 >= (int64_t)1 << 31)
             return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
-        if (variant == 7) return launch_smfmac_direct<T, 4, 2, 2, 2>(P, s);
-        return launch_smfmac_direct<T, 2, 4, 4, 1>(P, s);
+        if (variant == 7) return launch_smfmac_direct<T, 4, 2, 2, 2, 1>(P, s);
+        if (variant == 8) return launch_smfmac_direct<T, 2, 8, 4, 1, 2>(P, s);
+        return launch_smfmac_direct<T, 2, 4, 4, 1, 1>(P, s);
     }
     return NMG_ERR_ARG;
 }
@@ -1104,7 +1154,7 @@ extern "C" int nmg_spmm_smfmac(const void *d_fp_val, const void *d_fp_idx, int64
     NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED,
                 "the sparse matrix cores take f16/bf16 only");
     NMG_REQUIRE(M >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
-    NMG_REQUIRE(variant >= 0 && variant <= 7, NMG_ERR_ARG, "unknown tile variant %d", variant);
+    NMG_REQUIRE(variant >= -1 && variant <= 8, NMG_ERR_ARG, "unknown tile variant %d", variant);
     NMG_REQUIRE(ldx >= K && ldy >= M, NMG_ERR_ARG, "leading dimension smaller than row length");
     NMG_REQUIRE((K % 8) == 0 && (ldx % 8) == 0 && ((uintptr_t)d_x % 16) == 0, NMG_ERR_UNSUPPORTED,
                 "activations must be 16-byte aligned with K and ldx multiples of 8");

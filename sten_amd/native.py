@@ -48,6 +48,7 @@ SIGNATURES = {
     "nmg_gather": (_I, [_P, _VP, _P, _P, _I, _I, _I, _I, _P]),
     "nmg_rowpack_pat_bytes": (_I64, [_I, _I]),
     "nmg_rowpack": (_I, [_P, _P, _I64, _I64, _P, _P, _I, _I, _I, _I, _P]),
+    "nmg_rowpack_expand": (_I, [_P, _P, _I64, _I64, _P, _I64, _I, _I, _I, _I, _P]),
     "nmg_spmm": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _I, _I, _I, _P]),
     "nmg_fragpack_supported": (_I, [_I, _I]),
     "nmg_fragpack_sizes": (_I, [_I64, _I64, ctypes.POINTER(_I64), ctypes.POINTER(_I64)]),

@@ -192,20 +192,17 @@ class GroupedNMTensor:
 
     def dense_operand(self, reduce_dim):
         """Dense copy [outputs, reduction] of the weight (transposed when the reduction runs along
-        dim 0), written by the to_dense kernel into fresh scratch; not cached."""
+        dim 0), expanded from the rowpack operand into fresh scratch; not cached."""
         lay = self.layout
-        native.require_gpu(self.val)
+        pk_val, pk_pat = self.rowpack()
         O, K = lay.dense_shape[1 - reduce_dim], lay.dense_shape[reduce_dim]
         out = torch.empty((O, K), dtype=self.val.dtype, device=self.val.device)
-        # element (dim0 = i, dim1 = j) of the weight lives at out[i, j] (reduce_dim == 1) or out[j, i]
-        s0, s1 = (K, 1) if reduce_dim == 1 else (1, K)
-        strides = (s0, s1)
-        view = native.NmgView(1, lay.G, lay.S, 0, strides[lay.group_dim], strides[lay.sparse_dim])
+        # rowpack lines run along the group dim; the scratch has the reduction dim contiguous
+        transpose = 1 if lay.group_dim == reduce_dim else 0
         with torch.cuda.device(out.device):
-            native.check(native.load().nmg_to_dense(
-                native.ptr(self.val), native.ptr(self.idx), native.ptr(out), ctypes.byref(view),
-                lay.n, lay.m, lay.group_size, native.dtype_code(out.dtype),
-                native.stream_ptr(out.device)))
+            native.check(native.load().nmg_rowpack_expand(
+                native.ptr(pk_val), native.ptr(pk_pat), lay.G, lay.S, native.ptr(out), K, transpose,
+                lay.n, lay.m, native.dtype_code(out.dtype), native.stream_ptr(out.device)))
         return out
 
     def fragpack(self):
@@ -263,7 +260,7 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
     if bias is not None:
         bias = bias.to(dtype=x.dtype).contiguous()
     kname = kernel or weight.spmm_opt.get("kernel", "auto")
-    variant = int(weight.spmm_opt.get("variant", 4))
+    variant = int(weight.spmm_opt.get("variant", -1))
     smf_ok = (reduce_sparse == 1 and K % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
               and x.dtype in (torch.float16, torch.bfloat16))
     if kname == "skinny" and T > 16:

@@ -190,7 +190,7 @@ def test_unregistered_op_raises_in_raise_mode():
         torch.relu(w)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 6, 7])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 6, 7, 8])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M,K,T,n,m,g", [
     (768, 768, 256, 2, 4, 16),
@@ -275,3 +275,40 @@ def test_dense_pipeline_kernel_both_directions(dtype, M, K, T, n, m, g):
     Wd0, _ = dense_ref(W, n, m, g, 0)
     y0 = sten.spmm(w0, x.to(DEV), reduce_dim=1, kernel="expand")
     assert rel_l2(to_np(y0), to_np(x).astype(np.float64) @ Wd0.T) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("R,C,n,m,g", [
+    (768, 768, 2, 4, 16),
+    (200, 330, 2, 4, 4),     # ragged on both dims
+    (130, 96, 3, 6, 2),      # m does not divide the tile width
+    (64, 520, 2, 8, 4),
+    (70, 130, 5, 12, 1),     # 792 patterns: two-byte pattern numbers
+])
+@pytest.mark.parametrize("sd", [1, 0])
+def test_dense_operand_matches_oracle_bit_exactly(dtype, R, C, n, m, g, sd):
+    print(f"case expand {dtype} {R}x{C} {n}:{m}:{g} sd={sd}", flush=True)
+    W = seeded((R, C), dtype, seed=R + C + m, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, sd)
+    w = make(W, n, m, g, sd)
+    a1 = w.dense_operand(1)          # [dim0, dim1]
+    a0 = w.dense_operand(0)          # transposed
+    assert a1.shape == (R, C) and a0.shape == (C, R)
+    assert np.array_equal(to_np(a1).astype(np.float64), Wd)
+    assert np.array_equal(to_np(a0).astype(np.float64), Wd.T)
+    assert torch.equal(a1, w.to_dense())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("O_,K,T", [(256, 64, 128), (300, 320, 77), (1024, 1024, 512)])
+def test_dense_nt_gemm_entry_point(dtype, O_, K, T):
+    from sten_amd import native
+    print(f"case gemm_nt {dtype} O={O_} K={K} T={T}", flush=True)
+    A = seeded((O_, K), dtype, seed=3, std=0.5).to(DEV)
+    X = seeded((T, K), dtype, seed=4).to(DEV)
+    b = seeded((O_,), dtype, seed=5).to(DEV)
+    Y = torch.empty((T, O_), dtype=dtype, device=DEV)
+    native.check(native.load().nmg_gemm_nt(A.data_ptr(), K, X.data_ptr(), K, Y.data_ptr(), O_, b.data_ptr(),
+                                           O_, K, T, native.dtype_code(dtype), native.stream_ptr(X.device)))
+    ref = to_np(X).astype(np.float64) @ to_np(A).astype(np.float64).T + to_np(b).astype(np.float64)
+    assert rel_l2(to_np(Y), ref) <= TOL[dtype]
