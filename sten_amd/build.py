@@ -6,7 +6,8 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libnmg_hip.so")
-SOURCES = ["nmg_runtime.hip", "nmg_sparsify.hip", "nmg_spmm.hip", "nmg_smfmac.hip", "nmg_dense.hip"]
+SOURCES = ["nmg_runtime.hip", "nmg_sparsify.hip", "nmg_spmm.hip", "nmg_smfmac.hip", "nmg_dense.hip",
+           "nmg_densefrag.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

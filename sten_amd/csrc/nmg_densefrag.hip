@@ -1,0 +1,441 @@
+// nmg x dense matmul on the dense matrix cores (V_MFMA_F32_32X32X16_{F16,BF16}) with the weight
+// expanded beforehand into the register order of the instruction ("densefrag" operand).
+//
+// Serves what the sparse matrix cores cannot: patterns that do not fit 2-of-4 groups (4:8,
+// 3:4, ...) and the reduction along the *group* dim, i.e. the gradient with respect to the
+// activations of a weight that is n:m along its own reduction dim:
+//
+//   transpose = 0:  Y[tok, q] = sum_s X[tok, s] * W2[q, s]      (q = line, s = sparse position)
+//   transpose = 1:  Y[tok, s] = sum_q X[tok, q] * W2[q, s]
+//
+// Two kernels:
+//   densefrag_kernel   rowpack -> densefrag, through an LDS tile (reads and writes contiguous);
+//   dense_direct_kernel  the multiplication, same skeleton as the direct-weights kernel of the
+//                        sparse matrix cores: 4 wavefronts stacked on the output dim, weight
+//                        fragments global -> registers DD_D K steps ahead, activation tile
+//                        global -> LDS by DMA, one barrier per K step of 64.
+//
+// densefrag [OB][K16][64 lanes][8]: for output block ob (32 outputs) and k-step k16 (16 reduction
+// positions), lane l holds the 8 weights of output ob*32 + l%32 at reduction positions
+// k16*16 + 8*(l/32) + 0..7 -- the A operand of the instruction.  OB is padded to a multiple of 8
+// (256 outputs), the reduction extent must be a multiple of 64; padding is zero.
+#include "nmg_common.h"
+#include "nmg_tile.h"
+
+#include <type_traits>
+
+namespace nmg {
+
+typedef _Float16 df_f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 df_bf16x8 __attribute__((ext_vector_type(8)));
+
+template <typename T> struct DfMma;
+template <> struct DfMma<__half> {
+    using F = df_f16x8;
+    __device__ static f32x16 run(F a, F b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
+template <> struct DfMma<__hip_bfloat16> {
+    using F = df_bf16x8;
+    __device__ static f32x16 run(F a, F b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+
+// ------------------------------------------------------------------ rowpack -> densefrag
+constexpr int DFX_L = 64, DFX_P = 128;   // LDS tile: lines x positions
+
+struct DfExpandParams {
+    const void *pk_val;
+    const void *pk_pat;
+    void *df;
+    const int8_t *order;
+    int64_t G, S, nb;
+    int64_t OB, K16;                      // blocks of the operand
+    int n, m, pat_bytes, bpt, transpose;  // bpt = blocks of m positions per tile (bpt * m == 128)
+};
+
+template <typename T> __global__ __launch_bounds__(256) void densefrag_kernel(DfExpandParams P)
+{
+    // transpose = 0: tile[line][position], outputs = lines;  transpose = 1: tile[position][line],
+    // outputs = positions.  Rows are outputs, columns the reduction; +8 elements of padding keep
+    // rows 16-byte aligned and spread the banks.
+    constexpr int PAD = 8;
+    __shared__ __align__(16) uint16_t tile[DFX_L * (DFX_P + PAD) > DFX_P * (DFX_L + PAD) ? DFX_L * (DFX_P + PAD)
+                                                                                        : DFX_P * (DFX_L + PAD)];
+    static_assert(sizeof(T) == 2, "16-bit data");
+    const int tid = threadIdx.x;
+    const int64_t q0 = (int64_t)blockIdx.y * DFX_L, b0 = (int64_t)blockIdx.x * P.bpt;
+    const int rows = P.transpose ? DFX_P : DFX_L, cols = P.transpose ? DFX_L : DFX_P;
+    const int pitch = cols + PAD;
+    {
+        uint4 z = {0, 0, 0, 0};
+        for (int i = tid; i < rows * pitch / 8; i += 256) ((uint4 *)tile)[i] = z;
+    }
+    __syncthreads();
+    const uint16_t *pv = (const uint16_t *)P.pk_val;
+    for (int i = tid; i < DFX_L * P.bpt; i += 256) {
+        const int ql = i / P.bpt, bl = i - ql * P.bpt;
+        const int64_t q = q0 + ql, b = b0 + bl;
+        if (q >= P.G || b >= P.nb) continue;
+        const int64_t blk = q * P.nb + b;
+        const int pat = P.pat_bytes == 1 ? (int)((const uint8_t *)P.pk_pat)[blk]
+                                         : (int)((const uint16_t *)P.pk_pat)[blk];
+        const int8_t *ord = P.order + pat * P.n;
+        for (int j = 0; j < P.n; j++) {
+            const int pos = bl * P.m + ord[j];
+            const uint16_t v = pv[blk * P.n + j];
+            if (P.transpose)
+                tile[pos * pitch + ql] = v;
+            else
+                tile[ql * pitch + pos] = v;
+        }
+    }
+    __syncthreads();
+    // tile -> fragments: (rows/32) x (cols/16) fragments of 64 lanes x 16 B
+    const int64_t ob0 = (P.transpose ? b0 * P.m : q0) / 32, k0 = (P.transpose ? q0 : b0 * P.m) / 16;
+    const int nfk = cols / 16, nfrag = (rows / 32) * nfk;
+    uint4 *df = (uint4 *)P.df;
+    for (int i = tid; i < nfrag * 64; i += 256) {
+        const int f = i >> 6, l = i & 63;
+        const int fo = f / nfk, fk = f - fo * nfk;
+        const int64_t ob = ob0 + fo, k16 = k0 + fk;
+        if (ob >= P.OB || k16 >= P.K16) continue;
+        const uint4 v = *(const uint4 *)(tile + (fo * 32 + (l & 31)) * pitch + fk * 16 + 8 * (l >> 5));
+        df[(ob * P.K16 + k16) * 64 + l] = v;
+    }
+}
+
+// ----------------------------------------------------------------------------- the matmul
+struct DfParams {
+    const void *df;
+    const void *x;
+    void *y;
+    const void *bias;
+    int64_t O, K, T, ldx, ldy;
+    int KP;              // K steps of 64
+    int tiles_m, tiles_n;
+};
+
+constexpr int DD_D = 2;    // K steps in flight (a dense K step takes twice the MFMA time of a sparse one)
+constexpr int DD_NS = 4;   // activation stages in LDS (>= DD_D + 1)
+
+// FB x TB accumulator blocks (32 outputs x 32 tokens) per wavefront, WM x WN wavefronts, NH token
+// parts per k-step.  A K step (64) is 4 k-steps of 16; a phase is one (k-step, token part) pair:
+// its MFMAs run while the activation fragments of the next phase are read from LDS, and the
+// loads of K step kp+DD_D are issued in the first two phases.
+template <typename T, int FB, int TB, int WM, int WN, int NH>
+__global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
+{
+    using Mm = DfMma<T>;
+    static_assert(WM * WN == 4, "four wavefronts");
+    static_assert(TB % NH == 0, "token blocks split evenly into phases");
+    constexpr int TF = WM * FB * 32, TT = WN * TB * 32;   // workgroup tile: outputs x tokens
+    constexpr int STAGE = TT * 128;                       // activation bytes per K step
+    constexpr int XL = TT / 32;                           // DMA loads per wavefront per K step
+    constexpr int OPS = XL + 4 * FB;                      // memory operations per wavefront per K step
+    constexpr int BT = TB / NH;                           // token blocks per phase
+    constexpr int NP = 4 * NH;                            // phases per K step
+    constexpr int NM = FB * BT;                           // MFMAs per phase
+    static_assert(OPS * DD_D < 64, "vmcnt is a 6-bit counter");
+    static_assert(NM >= 4, "phase too short to hide the loads behind");
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    // Workgroup -> tile: consecutive ids are dealt round-robin to the 8 XCDs; give each XCD a
+    // contiguous run of ids and walk the grid in bands of 4 output tiles, so that a run covers
+    // a compact block of tiles whose weights and activations stay in that XCD's L2.
+    int id = blockIdx.x;
+    const int ntiles = P.tiles_m * P.tiles_n;
+    if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
+    constexpr int GH = 4;
+    const int band = id / (GH * P.tiles_n);
+    const int band_h = min(P.tiles_m - band * GH, GH);
+    const int in_band = id - band * GH * P.tiles_n;
+    const int tile_m = band * GH + in_band % band_h, tile_n = in_band / band_h;
+    const int64_t f0 = (int64_t)tile_m * TF, t0 = (int64_t)tile_n * TT;
+    const int KP = P.KP;
+    const int wm = wave / WN, wn = wave % WN;
+    const int ob0 = (int)(f0 / 32) + wm * FB;
+
+    // ---- global sources (wavefront-uniform bases in scalar registers, the lane's share as a
+    //      32-bit offset) ----
+    const unsigned char *av_base[FB];
+#pragma unroll
+    for (int fb = 0; fb < FB; fb++)
+        av_base[fb] = (const unsigned char *)P.df + ((int64_t)(ob0 + fb) * KP * 4) * 1024;
+    const uint32_t lane16 = lane * 16;
+    const unsigned char *x_base = (const unsigned char *)P.x;
+    uint32_t x_off[XL];
+#pragma unroll
+    for (int i = 0; i < XL; i++) {
+        const int row = (wave * XL + i) * 8 + (lane >> 3);
+        const int piece = lane & 7;
+        const int q = piece ^ ((row >> 1) & 7);   // logical 16-byte chunk stored at this piece
+        int64_t tok = t0 + row;
+        if (tok >= P.T) tok = P.T - 1;            // clamped rows are computed, never stored
+        x_off[i] = (uint32_t)((tok * P.ldx + q * 8) * 2);
+    }
+
+    struct WSet {
+        u32x4 a[FB][4];
+    };
+    WSet ws[DD_D + 1];
+    // Steps beyond the last repeat it: the operation count stays uniform, the data is unused.
+    auto issue_x = [&](int kp) {
+        if (kp >= KP) kp = KP - 1;
+        unsigned char *base = smem + (kp & (DD_NS - 1)) * STAGE;
+        const unsigned char *xb = x_base + (int64_t)kp * 128;
+#pragma unroll
+        for (int i = 0; i < XL; i++)
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[i]),
+                                             (lds_ptr_t)(base + (wave * XL + i) * 1024), 16, 0, 0);
+    };
+    auto issue_a = [&](int kp, WSet &w) {
+        if (kp >= KP) kp = KP - 1;
+#pragma unroll
+        for (int fb = 0; fb < FB; fb++) {
+            // Written as instructions so that their completion is tracked by the explicit vmcnt
+            // waits below and by nothing else, and with accumulation registers as targets: a
+            // compiler-made copy of a register whose load is still in flight would copy stale
+            // data, and the ring does not fit in the architectural registers.
+            const unsigned char *av = av_base[fb] + (int64_t)kp * 4096;
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(w.a[fb][0]) : "v"(lane16), "s"(av) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(w.a[fb][1]) : "v"(lane16), "s"(av) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, %2 offset:2048" : "=v"(w.a[fb][2]) : "v"(lane16), "s"(av) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, %2 offset:3072" : "=v"(w.a[fb][3]) : "v"(lane16), "s"(av) : "memory");
+        }
+    };
+
+    f32x16 acc[FB][TB];
+#pragma unroll
+    for (int i = 0; i < FB; i++)
+#pragma unroll
+        for (int j = 0; j < TB; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+    // 256 accumulators would fill the architectural registers exactly; pin half of them to
+    // the accumulation registers (the MFMA takes its C/D operand from either file).
+    auto pin_acc = [&]() {
+        if constexpr (FB * TB * 16 > 128) {
+#pragma unroll
+            for (int tb = 0; tb < TB; tb++) asm volatile("" : "+a"(acc[FB - 1][tb]));
+        }
+    };
+    pin_acc();
+
+    // Activation fragment of k-step k16 (B operand): lane (token j = l%32, h = l/32) holds the 8
+    // reduction positions 16*k16 + 8h + 0..7 = 16-byte chunk 2*k16 + h of its token row; chunks
+    // are stored XOR-swizzled with (row/2)%8, so that 16 consecutive rows hit all banks.
+    const int j = lane & 31, h = lane >> 5, sw = (j >> 1) & 7;
+    int b_off[4];
+#pragma unroll
+    for (int k16 = 0; k16 < 4; k16++) b_off[k16] = (wn * TB * 32 + j) * 128 + (((k16 * 2 + h) ^ sw) << 4);
+
+    struct BFrags {
+        u32x4 b[BT];
+    };
+    BFrags fr[2];
+    auto read_b = [&](BFrags &f, const unsigned char *base, int ph) {
+        const int k16 = ph / NH, hh = ph % NH;
+#pragma unroll
+        for (int t = 0; t < BT; t++) f.b[t] = *(const u32x4 *)(base + b_off[k16] + (hh * BT + t) * 32 * 128);
+    };
+    // MFMAs lo..hi-1 of phase PH, numbered fb * BT + t
+    auto mma = [&](const WSet &w, const BFrags &f, auto ph_tag, int lo, int hi) {
+        constexpr int PH = decltype(ph_tag)::value, K16 = PH / NH, HH = PH % NH;
+#pragma unroll
+        for (int fb = 0; fb < FB; fb++) {
+            union {
+                u32x4 u;
+                typename Mm::F v;
+            } ca;
+            ca.u = w.a[fb][K16];
+#pragma unroll
+            for (int t = 0; t < BT; t++) {
+                if (fb * BT + t < lo || fb * BT + t >= hi) continue;
+                union {
+                    u32x4 u;
+                    typename Mm::F v;
+                } cb;
+                cb.u = f.b[t];
+                acc[fb][HH * BT + t] = Mm::run(ca.v, cb.v, acc[fb][HH * BT + t]);
+            }
+        }
+    };
+
+    // prologue: steps 0 .. DD_D-1 in flight, then wait for step 0
+#pragma unroll
+    for (int st = 0; st < DD_D; st++) {
+        issue_x(st);
+        issue_a(st, ws[st]);
+    }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DD_D - 1) * OPS) : "memory");
+    asm volatile("s_barrier" ::: "memory");
+    read_b(fr[0], smem, 0);
+
+    for (int kp0 = 0; kp0 < KP; kp0 += DD_D + 1) {
+#pragma unroll
+        for (int u = 0; u <= DD_D; u++) {
+            const int kp = kp0 + u;
+            if (kp >= KP) break;
+            const unsigned char *base = smem + (kp & (DD_NS - 1)) * STAGE;
+            const unsigned char *next = smem + ((kp + 1) & (DD_NS - 1)) * STAGE;
+            // One phase: two MFMAs; the LDS reads of the next phase into the other fragment set;
+            // in the first two phases the loads of step kp+DD_D; the rest of the MFMAs.  Before
+            // the reads of the last phase, which fetch from the next stage, the barrier.  The
+            // instruction statements fence the scheduler, so this is also the issue order.
+            auto phase = [&](auto ph_tag) {
+                constexpr int PH = decltype(ph_tag)::value;
+                mma(ws[u], fr[PH % 2], ph_tag, 0, 2);
+                __builtin_amdgcn_sched_barrier(0);
+                if (PH == NP - 1) {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // fragments of step kp are in registers
+                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DD_D - 1) * OPS) : "memory");  // my share of kp+1 landed
+                    asm volatile("s_barrier" ::: "memory");              // ... and everybody else's
+                    __builtin_amdgcn_sched_barrier(0);
+                    read_b(fr[(PH + 1) % 2], next, 0);
+                } else {
+                    read_b(fr[(PH + 1) % 2], base, PH + 1);
+                }
+                if (PH == 0) issue_x(kp + DD_D);
+                if (PH == 1) issue_a(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)]);
+                mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            phase(std::integral_constant<int, 0>{});
+            phase(std::integral_constant<int, 1>{});
+            phase(std::integral_constant<int, 2>{});
+            phase(std::integral_constant<int, 3>{});
+            if constexpr (NP == 8) {
+                phase(std::integral_constant<int, 4>{});
+                phase(std::integral_constant<int, 5>{});
+                phase(std::integral_constant<int, 6>{});
+                phase(std::integral_constant<int, 7>{});
+            }
+            static_assert(NP == 4 || NP == 8, "one or two token parts");
+        }
+    }
+    pin_acc();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_barrier" ::: "memory");
+    const TileOut out{P.y, P.bias, P.O, P.T, P.ldy};
+    smf_store_tile<T, FB, TB>(acc, smem + wave * (TB * 32 * (FB * 64 + 16)), lane, f0 + wm * FB * 32,
+                              t0 + wn * TB * 32, out);
+}
+
+template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_dense_direct(DfParams &P, hipStream_t s)
+{
+    constexpr int TF = WM * FB * 32, TT = WN * TB * 32;
+    static_assert(TF == 256, "the operand is padded to 256 outputs");
+    P.tiles_m = (int)((P.O + TF - 1) / TF);
+    P.tiles_n = (int)((P.T + TT - 1) / TT);
+    dim3 grid((unsigned)(P.tiles_m * P.tiles_n));
+    constexpr size_t ring = (size_t)DD_NS * TT * 128, stg = (size_t)4 * TB * 32 * (FB * 64 + 16);
+    constexpr size_t lds = ring > stg ? ring : stg;
+    static_assert(lds <= 160 * 1024, "LDS");
+    auto k = dense_direct_kernel<T, FB, TB, WM, WN, NH>;
+    NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(k, grid, dim3(256), lds, s, P);
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
+template <typename T> static int launch_dense(DfParams &P, int variant, hipStream_t s)
+{
+    if (variant < 0) {
+        // 256 x 256 tiles move fewer bytes per flop through the vector caches but there are half
+        // as many of them to spread over the 256 CUs: compare rounds of tiles.
+        const int64_t tm = (P.O + 255) / 256;
+        const int64_t n128 = tm * ((P.T + 127) / 128), n256 = tm * ((P.T + 255) / 256);
+        const double cost128 = (double)((n128 + 255) / 256), cost256 = 1.7 * (double)((n256 + 255) / 256);
+        variant = cost256 < cost128 ? 1 : 0;
+    }
+    if (variant == 1) return launch_dense_direct<T, 2, 8, 4, 1, 2>(P, s);
+    return launch_dense_direct<T, 2, 4, 4, 1, 1>(P, s);
+}
+
+}  // namespace nmg
+
+using namespace nmg;
+
+extern "C" int nmg_densefrag_supported(int n, int m)
+{
+    return (m >= 1 && m <= 64 && n >= 0 && n <= m && (m & (m - 1)) == 0) ? 1 : 0;
+}
+
+extern "C" int nmg_densefrag_elems(int64_t O, int64_t K, int64_t *elems)
+{
+    NMG_REQUIRE(O >= 0 && K >= 0 && elems, NMG_ERR_ARG, "invalid extents");
+    NMG_REQUIRE(K % 64 == 0, NMG_ERR_UNSUPPORTED, "the reduction extent must be a multiple of 64");
+    *elems = ((O + 255) / 256) * 256 * K;
+    return NMG_OK;
+}
+
+extern "C" int nmg_densefrag(const void *d_pk_val, const void *d_pk_pat, int64_t G, int64_t S, int transpose,
+                             void *d_df, int n, int m, int dtype, void *stream)
+{
+    NMG_REQUIRE(nmg_densefrag_supported(n, m), NMG_ERR_UNSUPPORTED,
+                "densefrag needs m to be a power of two, got %d:%d", n, m);
+    NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED, "densefrag takes f16/bf16");
+    NMG_REQUIRE(G >= 0 && S >= 0, NMG_ERR_ARG, "negative extent");
+    const int64_t O = transpose ? S : G, K = transpose ? G : S;
+    NMG_REQUIRE(K % 64 == 0, NMG_ERR_UNSUPPORTED, "the reduction extent (%lld) must be a multiple of 64",
+                (long long)K);
+    if (O == 0 || K == 0) return NMG_OK;
+    NMG_REQUIRE(d_pk_val && d_pk_pat && d_df, NMG_ERR_ARG, "null device pointer");
+    DfExpandParams P{};
+    if (int rc = device_order(n, m, &P.order)) return rc;
+    P.pk_val = d_pk_val;
+    P.pk_pat = d_pk_pat;
+    P.df = d_df;
+    P.G = G;
+    P.S = S;
+    P.nb = (S + m - 1) / m;
+    P.OB = (O + 255) / 256 * 8;
+    P.K16 = K / 16;
+    P.n = n;
+    P.m = m;
+    P.pat_bytes = binom(m, n) <= 256 ? 1 : 2;
+    P.bpt = DFX_P / m;
+    P.transpose = transpose ? 1 : 0;
+    // the grid covers the padded operand: outputs up to a multiple of 256
+    const int64_t Gp = transpose ? G : P.OB * 32, Sp = transpose ? P.OB * 32 : S;
+    const int64_t gx = (Sp + DFX_P - 1) / DFX_P, gy = (Gp + DFX_L - 1) / DFX_L;
+    NMG_REQUIRE(gx <= 0x7fffffffLL && gy <= 65535, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
+    dim3 grid((unsigned)gx, (unsigned)gy);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == NMG_F16)
+        hipLaunchKernelGGL(densefrag_kernel<__half>, grid, dim3(256), 0, s, P);
+    else
+        hipLaunchKernelGGL(densefrag_kernel<__hip_bfloat16>, grid, dim3(256), 0, s, P);
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
+extern "C" int nmg_spmm_densefrag(const void *d_df, int64_t O, int64_t K, const void *d_x, int64_t ldx,
+                                  void *d_y, int64_t ldy, const void *d_bias, int64_t T, int dtype,
+                                  int variant, void *stream)
+{
+    NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED, "densefrag takes f16/bf16");
+    NMG_REQUIRE(O >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
+    NMG_REQUIRE(variant >= -1 && variant <= 1, NMG_ERR_ARG, "unknown tile variant %d", variant);
+    NMG_REQUIRE(ldx >= K && ldy >= O, NMG_ERR_ARG, "leading dimension smaller than row length");
+    NMG_REQUIRE(K % 64 == 0 && K > 0 && ldx % 8 == 0 && ((uintptr_t)d_x % 16) == 0, NMG_ERR_UNSUPPORTED,
+                "needs K %% 64 == 0 and 16-byte aligned activation rows");
+    NMG_REQUIRE(T * ldx * 2 < ((int64_t)1 << 31), NMG_ERR_UNSUPPORTED, "activations must be smaller than 2 GiB");
+    if (O == 0 || T == 0) return NMG_OK;
+    NMG_REQUIRE(d_df && d_x && d_y, NMG_ERR_ARG, "null device pointer");
+    DfParams P{};
+    P.df = d_df;
+    P.x = d_x;
+    P.y = d_y;
+    P.bias = d_bias;
+    P.O = O;
+    P.K = K;
+    P.T = T;
+    P.ldx = ldx;
+    P.ldy = ldy;
+    P.KP = (int)(K / 64);
+    hipStream_t s = (hipStream_t)stream;
+    return dtype == NMG_F16 ? launch_dense<__half>(P, variant, s) : launch_dense<__hip_bfloat16>(P, variant, s);
+}

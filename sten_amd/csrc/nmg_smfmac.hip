@@ -19,17 +19,16 @@
 // A fragments go global -> registers (already in lane order, fully coalesced); the activation
 // tile goes global -> registers -> LDS (double buffered), one barrier per 64-wide K step.
 #include "nmg_common.h"
+#include "nmg_tile.h"
 
 #include <type_traits>
 
 namespace nmg {
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x16 __attribute__((ext_vector_type(16)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 template <typename T> struct Smf;
 template <> struct Smf<__half> {
@@ -59,13 +58,6 @@ struct SmfParams {
     int MB, KP;          // feature blocks of 32, k pairs of 64
     int tiles_m, tiles_n;
 };
-
-__device__ __forceinline__ uint16_t f32_to_bits16(float x, __half *) { return __half_as_ushort(__float2half(x)); }
-__device__ __forceinline__ uint16_t f32_to_bits16(float x, __hip_bfloat16 *)
-{
-    __hip_bfloat16 b = __float2bfloat16(x);
-    return *reinterpret_cast<uint16_t *>(&b);
-}
 
 constexpr int SMF_ROW = 144;  // bytes per token row in LDS: 64 k * 2 B + 16 B pad (conflict-free b128 reads)
 
@@ -259,73 +251,6 @@ __global__ __launch_bounds__(64 * WM * WN, MINW) void spmm_smfmac_kernel(SmfPara
 
 constexpr int PIPE_OUT_ROW = 128 * 2 + 16;  // epilogue staging: one token row of a matrix wavefront
 
-// Epilogue shared by the pipelined kernels.  D[row = feature][col = token]; a lane holds token
-// l%32 and features 8*(r/4) + 4*(l/32) + r%4.  The wavefront's TB*32 tokens x FB*32 features are
-// staged through its own LDS region `stg` as [token][feature] so the global stores are 16 B per
-// lane and FB*64 B contiguous per token row.  fw / tw = first feature / token of the wavefront.
-// The caller guarantees that no load into LDS is pending.
-template <typename T, int FB, int TB>
-__device__ __forceinline__ void smf_store_tile(const f32x16 (&acc)[FB][TB], unsigned char *stg, int lane,
-                                               int64_t fw, int64_t tw, const SmfParams &P)
-{
-    constexpr int ROW = FB * 64 + 16;       // bytes per staged token row (16 B pad: conflict-free)
-    constexpr int CPR = FB * 4;             // 16-byte chunks per row
-    constexpr int RPP = 64 / CPR;           // token rows per pass of the wavefront
-    const int j = lane & 31, h = lane >> 5;
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-    for (int tb = 0; tb < TB; tb++)
-#pragma unroll
-        for (int fb = 0; fb < FB; fb++)
-#pragma unroll
-            for (int rq = 0; rq < 4; rq++) {
-                uint16_t hh[4];
-#pragma unroll
-                for (int i = 0; i < 4; i++) hh[i] = f32_to_bits16(acc[fb][tb][rq * 4 + i], (T *)nullptr);
-                uint2 pk;
-                pk.x = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
-                pk.y = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
-                *(uint2 *)(stg + (tb * 32 + j) * ROW + (fb * 32 + rq * 8 + h * 4) * 2) = pk;
-            }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    uint16_t *Y = (uint16_t *)P.y;
-    const T *bias = (const T *)P.bias;
-    const bool vec_ok = (P.ldy & 7) == 0 && ((uintptr_t)P.y & 15) == 0;
-    const int fc = lane % CPR;                      // 8-feature chunk of the row
-    const int64_t f = fw + fc * 8;
-    float bv[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) bv[i] = (bias && f + i < P.M) ? to_f32(bias[f + i]) : 0.f;
-#pragma unroll 4
-    for (int it = 0; it < TB * 32 / RPP; it++) {
-        const int tl = it * RPP + lane / CPR;
-        const int64_t tok = tw + tl;
-        u32x4 v = *(const u32x4 *)(stg + tl * ROW + fc * 16);
-        if (tok >= P.T || f >= P.M) continue;
-        if (bias) {
-            uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                uint16_t lo = (uint16_t)(w[i] & 0xFFFF), hi = (uint16_t)(w[i] >> 16);
-                T tlo = *reinterpret_cast<T *>(&lo), thi = *reinterpret_cast<T *>(&hi);
-                lo = f32_to_bits16(to_f32(tlo) + bv[2 * i], (T *)nullptr);
-                hi = f32_to_bits16(to_f32(thi) + bv[2 * i + 1], (T *)nullptr);
-                w[i] = (uint32_t)lo | ((uint32_t)hi << 16);
-            }
-            v.x = w[0]; v.y = w[1]; v.z = w[2]; v.w = w[3];
-        }
-        uint16_t *dst = Y + tok * P.ldy + f;
-        if (vec_ok && f + 7 < P.M) {
-            *(u32x4 *)dst = v;
-        } else {
-            uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int i = 0; i < 8; i++)
-                if (f + i < P.M) dst[i] = (uint16_t)(w[i >> 1] >> ((i & 1) * 16));
-        }
-    }
-}
-
 // ------------------------------------------------------------------------ pipelined kernel
 // Same math, deeper memory pipeline and specialised wavefronts.
 //
@@ -357,8 +282,6 @@ constexpr int PIPE_X = 128 * 128;
 constexpr int PIPE_STAGE = PIPE_AVAL + PIPE_AIDX + PIPE_X;
 constexpr int PIPE_LPT = 10;  // DMA loads per loader thread per stage: 4 weight + 2 index + 4 activation
 
-typedef __attribute__((address_space(3))) void *lds_ptr_t;
-typedef const __attribute__((address_space(1))) void *glb_ptr_t;
 
 template <typename T>
 __global__ __launch_bounds__(512, 2) void spmm_smfmac_pipe_kernel(SmfParams P)
@@ -551,7 +474,8 @@ __global__ __launch_bounds__(512, 2) void spmm_smfmac_pipe_kernel(SmfParams P)
         __builtin_amdgcn_sched_barrier(0);
     }
 
-    smf_store_tile<T, FB, TB>(acc, smem + wave * (64 * PIPE_OUT_ROW), lane, f0 + wm * 128, t0 + wn * 64, P);
+    const TileOut out{P.y, P.bias, P.M, P.T, P.ldy};
+    smf_store_tile<T, FB, TB>(acc, smem + wave * (64 * PIPE_OUT_ROW), lane, f0 + wm * 128, t0 + wn * 64, out);
 }
 
 template <typename T> static int launch_smfmac_pipe(SmfParams &P, hipStream_t s)
@@ -809,8 +733,9 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
     pin_acc();
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     asm volatile("s_barrier" ::: "memory");
+    const TileOut out{P.y, P.bias, P.M, P.T, P.ldy};
     smf_store_tile<T, FB, TB>(acc, smem + wave * (TB * 32 * (FB * 64 + 16)), lane, f0 + wm * FB * 32,
-                              t0 + wn * TB * 32, P);
+                              t0 + wn * TB * 32, out);
 }
 
 template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_smfmac_direct(SmfParams &P, hipStream_t s)

@@ -1,0 +1,94 @@
+// Pieces shared by the pipelined matrix-core kernels: vector types, LDS-DMA pointer types and the
+// output-tile epilogue.
+#pragma once
+#include "nmg_common.h"
+
+namespace nmg {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+typedef const __attribute__((address_space(1))) void *glb_ptr_t;
+
+__device__ __forceinline__ uint16_t f32_to_bits16(float x, __half *) { return __half_as_ushort(__float2half(x)); }
+__device__ __forceinline__ uint16_t f32_to_bits16(float x, __hip_bfloat16 *)
+{
+    __hip_bfloat16 b = __float2bfloat16(x);
+    return *reinterpret_cast<uint16_t *>(&b);
+}
+
+// Where an output tile goes: Y[T, M] row-major with leading dimension ldy, optional bias[M].
+struct TileOut {
+    void *y;
+    const void *bias;
+    int64_t M, T, ldy;
+};
+
+// Epilogue of the pipelined kernels.  D[row = feature][col = token]; a lane holds token
+// l%32 and features 8*(r/4) + 4*(l/32) + r%4.  The wavefront's TB*32 tokens x FB*32 features are
+// staged through its own LDS region `stg` as [token][feature] so the global stores are 16 B per
+// lane and FB*64 B contiguous per token row.  fw / tw = first feature / token of the wavefront.
+// The caller guarantees that no load into LDS is pending.
+template <typename T, int FB, int TB>
+__device__ __forceinline__ void smf_store_tile(const f32x16 (&acc)[FB][TB], unsigned char *stg, int lane,
+                                               int64_t fw, int64_t tw, const TileOut &P)
+{
+    constexpr int ROW = FB * 64 + 16;       // bytes per staged token row (16 B pad: conflict-free)
+    constexpr int CPR = FB * 4;             // 16-byte chunks per row
+    constexpr int RPP = 64 / CPR;           // token rows per pass of the wavefront
+    const int j = lane & 31, h = lane >> 5;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int tb = 0; tb < TB; tb++)
+#pragma unroll
+        for (int fb = 0; fb < FB; fb++)
+#pragma unroll
+            for (int rq = 0; rq < 4; rq++) {
+                uint16_t hh[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) hh[i] = f32_to_bits16(acc[fb][tb][rq * 4 + i], (T *)nullptr);
+                uint2 pk;
+                pk.x = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
+                pk.y = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
+                *(uint2 *)(stg + (tb * 32 + j) * ROW + (fb * 32 + rq * 8 + h * 4) * 2) = pk;
+            }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    uint16_t *Y = (uint16_t *)P.y;
+    const T *bias = (const T *)P.bias;
+    const bool vec_ok = (P.ldy & 7) == 0 && ((uintptr_t)P.y & 15) == 0;
+    const int fc = lane % CPR;                      // 8-feature chunk of the row
+    const int64_t f = fw + fc * 8;
+    float bv[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) bv[i] = (bias && f + i < P.M) ? to_f32(bias[f + i]) : 0.f;
+#pragma unroll 4
+    for (int it = 0; it < TB * 32 / RPP; it++) {
+        const int tl = it * RPP + lane / CPR;
+        const int64_t tok = tw + tl;
+        u32x4 v = *(const u32x4 *)(stg + tl * ROW + fc * 16);
+        if (tok >= P.T || f >= P.M) continue;
+        if (bias) {
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint16_t lo = (uint16_t)(w[i] & 0xFFFF), hi = (uint16_t)(w[i] >> 16);
+                T tlo = *reinterpret_cast<T *>(&lo), thi = *reinterpret_cast<T *>(&hi);
+                lo = f32_to_bits16(to_f32(tlo) + bv[2 * i], (T *)nullptr);
+                hi = f32_to_bits16(to_f32(thi) + bv[2 * i + 1], (T *)nullptr);
+                w[i] = (uint32_t)lo | ((uint32_t)hi << 16);
+            }
+            v.x = w[0]; v.y = w[1]; v.z = w[2]; v.w = w[3];
+        }
+        uint16_t *dst = Y + tok * P.ldy + f;
+        if (vec_ok && f + 7 < P.M) {
+            *(u32x4 *)dst = v;
+        } else {
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                if (f + i < P.M) dst[i] = (uint16_t)(w[i >> 1] >> ((i & 1) * 16));
+        }
+    }
+}
+
+}  // namespace nmg

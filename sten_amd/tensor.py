@@ -190,6 +190,24 @@ class GroupedNMTensor:
             self._rowpack = (key, pk_val, pk_pat)
         return self._rowpack[1], self._rowpack[2]
 
+    def densefrag(self, reduce_dim):
+        """The weight as the A operand of the dense matrix cores, [outputs, reduction] in
+        fragment order, expanded from the rowpack operand into fresh scratch (not cached: it
+        is as large as the dense weight)."""
+        lay = self.layout
+        lib = native.load()
+        pk_val, pk_pat = self.rowpack()
+        O, K = lay.dense_shape[1 - reduce_dim], lay.dense_shape[reduce_dim]
+        elems = ctypes.c_int64(0)
+        native.check(lib.nmg_densefrag_elems(O, K, ctypes.byref(elems)))
+        df = torch.empty((elems.value,), dtype=self.val.dtype, device=self.val.device)
+        transpose = 1 if lay.group_dim == reduce_dim else 0   # rowpack lines run along the group dim
+        with torch.cuda.device(df.device):
+            native.check(lib.nmg_densefrag(
+                native.ptr(pk_val), native.ptr(pk_pat), lay.G, lay.S, transpose, native.ptr(df),
+                lay.n, lay.m, native.dtype_code(df.dtype), native.stream_ptr(df.device)))
+        return df
+
     def dense_operand(self, reduce_dim):
         """Dense copy [outputs, reduction] of the weight (transposed when the reduction runs along
         dim 0), expanded from the rowpack operand into fresh scratch; not cached."""
@@ -281,21 +299,34 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
                 x.stride(0) if T > 1 else K, native.ptr(y), O, native.ptr(bias), T,
                 native.dtype_code(x.dtype), variant, native.stream_ptr(x.device)))
         return y
-    if (kname in ("auto", "mfma", "expand") and T > 16 and x.dtype in (torch.float16, torch.bfloat16)
-            and K % 64 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
-            and T * x.stride(0) * 2 < 2 ** 31 and O * K * 2 < 2 ** 31
-            and (kname == "expand" or weight.spmm_opt.get("expand", True))):
-        # "expand, then multiply": write the dense weight with the reduction contiguous into
-        # scratch (one HBM-bound pass) and run the pipelined dense-MFMA kernel on it
+    dense16 = (T > 16 and x.dtype in (torch.float16, torch.bfloat16) and K % 64 == 0
+               and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and T * x.stride(0) * 2 < 2 ** 31)
+    if (kname in ("auto", "mfma", "densefrag") and dense16
+            and native.load().nmg_densefrag_supported(lay.n, lay.m)
+            and (kname == "densefrag" or weight.spmm_opt.get("expand", True))):
+        # "expand, then multiply": one HBM-bound pass writes the weight in the register order of
+        # the dense matrix cores into scratch, the pipelined kernel multiplies from there
+        df = weight.densefrag(reduce_dim)
+        with torch.cuda.device(x.device):
+            native.check(native.load().nmg_spmm_densefrag(
+                native.ptr(df), O, K, native.ptr(x), x.stride(0), native.ptr(y), O, native.ptr(bias), T,
+                native.dtype_code(x.dtype), int(weight.spmm_opt.get("dense_variant", -1)),
+                native.stream_ptr(x.device)))
+        return y
+    if kname == "densefrag":
+        raise native.NmgError("the densefrag route needs 16-bit data, more than 16 tokens, a power-of-two m "
+                              "and a reduction extent that is a multiple of 64")
+    if kname == "expand":
+        if not (dense16 and O * K * 2 < 2 ** 31):
+            raise native.NmgError("the expand-then-multiply route needs 16-bit data, more than 16 tokens "
+                                  "and a reduction extent that is a multiple of 64")
+        # the same idea with a plain row-major dense copy of the weight
         a = weight.dense_operand(reduce_dim)
         with torch.cuda.device(x.device):
             native.check(native.load().nmg_gemm_nt(
                 native.ptr(a), K, native.ptr(x), x.stride(0), native.ptr(y), O, native.ptr(bias),
                 O, K, T, native.dtype_code(x.dtype), native.stream_ptr(x.device)))
         return y
-    if kname == "expand":
-        raise native.NmgError("the expand-then-multiply route needs 16-bit data, more than 16 tokens "
-                              "and a reduction extent that is a multiple of 64")
     pk_val, pk_pat = weight.rowpack()
     with torch.cuda.device(x.device):
         native.check(native.load().nmg_spmm(

@@ -312,3 +312,29 @@ def test_dense_nt_gemm_entry_point(dtype, O_, K, T):
                                            O_, K, T, native.dtype_code(dtype), native.stream_ptr(X.device)))
     ref = to_np(X).astype(np.float64) @ to_np(A).astype(np.float64).T + to_np(b).astype(np.float64)
     assert rel_l2(to_np(Y), ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dense_variant", [-1, 0, 1])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,K,T,n,m,g", [
+    (256, 64, 128, 2, 4, 16),     # one tile, one K step
+    (512, 320, 300, 4, 8, 4),     # 4:8 does not fit the sparse matrix cores; ragged tokens
+    (320, 448, 77, 2, 4, 16),     # ragged outputs in both directions
+    (1024, 1024, 512, 1, 2, 8),
+    (192, 128, 40, 3, 16, 1),
+])
+def test_densefrag_route_both_directions(dense_variant, dtype, M, K, T, n, m, g):
+    print(f"case densefrag v{dense_variant} {dtype} M={M} K={K} T={T} {n}:{m}:{g}", flush=True)
+    W = seeded((M, K), dtype, seed=M + K + n, std=0.5)
+    x = seeded((T, K), dtype, seed=1)
+    b = seeded((M,), dtype, seed=2)
+    gy = seeded((T, M), dtype, seed=3)
+    for sd in (1, 0):
+        Wd, _ = dense_ref(W, n, m, g, sd)
+        w = make(W, n, m, g, sd)
+        w.spmm_opt["dense_variant"] = dense_variant
+        y = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1, kernel="densefrag")
+        ref = to_np(x).astype(np.float64) @ Wd.T + to_np(b).astype(np.float64)
+        assert rel_l2(to_np(y), ref) <= TOL[dtype], sd
+        gx = sten.spmm(w, gy.to(DEV), reduce_dim=0, kernel="densefrag")
+        assert rel_l2(to_np(gx), to_np(gy).astype(np.float64) @ Wd) <= TOL[dtype], sd
