@@ -1,19 +1,23 @@
-"""Benchmark of the nmg sparse x dense matmul on one MI355X.
+"""Benchmark of the grouped n:m (nmg) hot path on one MI355X.
 
-Workload (BASELINE config 2): fp16 weight 4096x4096 ~ N(0, 0.02), grouped 2:4 (group 16) along
-the reduction dim; fp16 activations 2048 tokens x 4096 ~ N(0,1); forward only, fp32 accumulate.
-A "step" is one nmg x dense matmul over that batch with every operand resident in HBM.
+Default workload (BASELINE config 2): fp16 weight 4096x4096 ~ N(0, 0.02), grouped 2:4 (group 16)
+along the reduction dim; fp16 activations 2048 tokens x 4096 ~ N(0,1); forward only, fp32
+accumulate.  A "step" is one pass of the measured operation over that batch with every operand
+resident in HBM.
 
-Prints one JSON line.  value = dense-equivalent TFLOP/s (2*M*K*N / step time).
-roofline.achieved counts the effective (non-zero) flops 2*M*K*N*n/m per launch over the kernel's
-average launch duration, measured with HIP events on the stream the kernel is launched on, against
-the dense fp16 MFMA peak -- i.e. the fraction of the density-scaled MFMA roofline.
-roofline.traffic is read from the committed rocprofv3 --pmc summary of this same command.
-cpu_baseline = the CPU restatement of the reference's AVX/OpenMP kernel (oracle/nmg_cpu_simd.cpp)
-on the host cores, same shape, fp32.
+Prints one JSON line.  For the matmul workloads value = dense-equivalent TFLOP/s (2*M*K*N / step
+time) and roofline.achieved counts the effective (non-zero) flops 2*M*K*N*n/m per launch over the
+kernel's average launch duration, measured with HIP events on the stream the kernel is launched
+on, against the dense fp16 MFMA peak -- i.e. the fraction of the density-scaled MFMA roofline.
+For the bandwidth-bound workloads (decode shapes, sparsifier) value = GB/s of algorithmic bytes
+(weight values + int16 indices + activations + output; dense input + val + idx for the
+sparsifier) and the roofline is HBM.  roofline.traffic is read from the committed rocprofv3 --pmc
+summary of the same command, when there is one.
+cpu_baseline (default workload only) = the CPU restatement of the reference's AVX/OpenMP kernel
+(oracle/nmg_cpu_simd.cpp) on the host cores, same shape, fp32.
 
-Other modes: --workload picks another BASELINE shape for ad-hoc measurement; --calibrate-copy
-runs a plain device copy of known size (the counter calibration for FETCH_SIZE / WRITE_SIZE).
+Other modes: --workload picks another BASELINE shape; --calibrate-copy runs a plain device copy
+of known size (the counter calibration for FETCH_SIZE / WRITE_SIZE).
 """
 import argparse
 import json
@@ -30,13 +34,20 @@ PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 
 WORKLOADS = {
-    # name: (M, K, tokens, n, m, g, description)
-    "c2": (4096, 4096, 2048, 2, 4, 16, "configs[1]: W 4096x4096 fp16 2:4:16 along K x 2048 tokens, forward"),
-    "target_2_4": (4096, 11008, 2048, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 2048 tokens, forward"),
-    "c3_1_8": (8192, 8192, 4096, 1, 8, 32, "configs[2]: W 8192x8192 fp16 1:8:32 x 4096 tokens, forward"),
-    "c3_2_8": (8192, 8192, 4096, 2, 8, 32, "configs[2]: W 8192x8192 fp16 2:8:32 x 4096 tokens, forward"),
-    "c3_4_8": (8192, 8192, 4096, 4, 8, 32, "configs[2]: W 8192x8192 fp16 4:8:32 x 4096 tokens, forward"),
-    "c5_fwd": (16384, 4096, 4096, 2, 4, 16, "configs[4]: W 16384x4096 fp16 2:4:16 x 4096 tokens, forward"),
+    # name: (kind, M, K, tokens, n, m, g, description)
+    "c2": ("fwd", 4096, 4096, 2048, 2, 4, 16, "configs[1]: W 4096x4096 fp16 2:4:16 along K x 2048 tokens, forward"),
+    "target_2_4": ("fwd", 4096, 11008, 2048, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 2048 tokens, forward"),
+    "target_2_4_4k": ("fwd", 4096, 11008, 4096, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 4096 tokens, forward"),
+    "c3_1_8": ("fwd", 8192, 8192, 4096, 1, 8, 32, "configs[2]: W 8192x8192 fp16 1:8:32 x 4096 tokens, forward"),
+    "c3_2_8": ("fwd", 8192, 8192, 4096, 2, 8, 32, "configs[2]: W 8192x8192 fp16 2:8:32 x 4096 tokens, forward"),
+    "c3_4_8": ("fwd", 8192, 8192, 4096, 4, 8, 32, "configs[2]: W 8192x8192 fp16 4:8:32 x 4096 tokens, forward"),
+    "c5_fwd": ("fwd", 16384, 4096, 4096, 2, 4, 16, "configs[4]: W 16384x4096 fp16 2:4:16 x 4096 tokens, forward"),
+    "c5_grad_x": ("grad_x", 16384, 4096, 4096, 2, 4, 16, "configs[4]: dY 4096x16384 x W 16384x4096 fp16 2:4:16, grad_input"),
+    "c2_grad_x": ("grad_x", 4096, 4096, 2048, 2, 4, 16, "configs[1] shape: dY 2048x4096 x W 4096x4096 fp16 2:4:16, grad_input"),
+    "decode_1": ("decode", 4096, 11008, 1, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 1 token"),
+    "decode_16": ("decode", 4096, 11008, 16, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 16 tokens"),
+    "sparsify_c2": ("sparsify", 4096, 4096, 0, 2, 4, 16, "configs[1]: sparsify W 4096x4096 fp16 to 2:4:16"),
+    "sparsify_c3_2_8": ("sparsify", 8192, 8192, 0, 2, 8, 32, "configs[2]: sparsify W 8192x8192 fp16 to 2:8:32"),
 }
 
 
@@ -71,13 +82,15 @@ def cpu_baseline(M, K, N, n, m, g, seconds=15.0):
 
 def committed_traffic(workload):
     """HBM bytes per launch from profiles/ (FETCH_SIZE + WRITE_SIZE, calibrated), or None."""
-    path = os.path.join(ROOT, "profiles", f"spmm_{workload}_pmc.txt")
-    try:
-        text = open(path).read()
-    except OSError:
-        return None
-    mt = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", text, re.M)
-    return float(mt.group(1)) if mt else None
+    for name in (f"spmm_{workload}_pmc.txt", f"{workload}_pmc.txt"):
+        try:
+            text = open(os.path.join(ROOT, "profiles", name)).read()
+        except OSError:
+            continue
+        mt = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", text, re.M)
+        if mt:
+            return float(mt.group(1))
+    return None
 
 
 def calibrate_copy():
@@ -113,52 +126,82 @@ def main():
     import sten_amd as sten
 
     dev = "cuda:0"
-    M, K, N, n, m, g, desc = WORKLOADS[args.workload]
+    kind, M, K, N, n, m, g, desc = WORKLOADS[args.workload]
     torch.manual_seed(0)
     W = (torch.randn(M, K) * 0.02).half().to(dev)
-    X = torch.randn(N, K).half().to(dev)
-    w = sten.GroupedNMTensor.from_dense(W, n, m, sparse_dim=1, group_size=g, group_dim=0)
-    w.spmm_opt["variant"] = args.variant
-    del W
+
+    if kind == "sparsify":
+        def step():
+            return sten.GroupedNMTensor.from_dense(W, n, m, sparse_dim=1, group_size=g, group_dim=0)
+        w = step()
+        algo_bytes = M * K * 2 + w.val.numel() * 2 + w.idx.numel() * 2
+    else:
+        w = sten.GroupedNMTensor.from_dense(W, n, m, sparse_dim=1, group_size=g, group_dim=0)
+        w.spmm_opt["variant"] = args.variant
+        del W
+        if kind == "grad_x":
+            X = torch.randn(N, M).half().to(dev)      # upstream gradient dY [tokens, out features]
+            rd = 0
+        else:
+            X = torch.randn(N, K).half().to(dev)
+            rd = 1
+
+        def step():
+            return sten.spmm(w, X, reduce_dim=rd, kernel=args.kernel)
+        # weight values + one int16 index per (line, block) + activations + output
+        algo_bytes = M * K * n // m * 2 + M * K // m * 2 + N * K * 2 + N * M * 2
+
     for _ in range(args.warmup):
-        y = sten.spmm(w, X, reduce_dim=1, kernel=args.kernel)
+        step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        y = sten.spmm(w, X, reduce_dim=1, kernel=args.kernel)
+        step()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / args.steps
 
-    # average launch duration of the kernel: one HIP event pair around K back-to-back launches,
-    # recorded on the stream the kernel is launched on (torch's current stream)
+    # average duration of a step on the device: one HIP event pair around K back-to-back steps,
+    # recorded on the stream the kernels are launched on (torch's current stream)
     stream = torch.cuda.current_stream()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record(stream)
     for _ in range(args.steps):
-        sten.spmm(w, X, reduce_dim=1, kernel=args.kernel)
+        step()
     e1.record(stream)
     torch.cuda.synchronize()
     kern_ms = e0.elapsed_time(e1) / args.steps
 
-    dense_flops = 2.0 * M * K * N
-    eff_flops = dense_flops * n / m
-    achieved = eff_flops / (kern_ms * 1e-3) / 1e12
     out = {
-        "metric": "nmg sparse x dense GEMM TFLOP/s (dense-equiv)",
-        "value": dense_flops / wall / 1e12,
-        "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": wall * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": desc, "kernel": args.kernel, "variant": args.variant,
-                   "effective_tflops": eff_flops / wall / 1e12, "kernel_ms": kern_ms},
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS,
-                     "traffic": committed_traffic(args.workload),
-                     "flops": "effective non-zero (2*M*K*N*n/m); dense-equivalent is m/n times this"},
     }
-    if not args.no_cpu:
+    if kind in ("fwd", "grad_x"):
+        dense_flops = 2.0 * M * K * N
+        eff_flops = dense_flops * n / m
+        achieved = eff_flops / (kern_ms * 1e-3) / 1e12
+        out.update({
+            "metric": "nmg sparse x dense GEMM TFLOP/s (dense-equiv)",
+            "value": dense_flops / wall / 1e12, "unit": "TFLOP/s",
+            "config": {"workload": desc, "kernel": args.kernel, "variant": args.variant,
+                       "effective_tflops": eff_flops / wall / 1e12, "kernel_ms": kern_ms},
+            "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP16_TFLOPS,
+                         "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS,
+                         "traffic": committed_traffic(args.workload),
+                         "flops": "effective non-zero (2*M*K*N*n/m); dense-equivalent is m/n times this"},
+        })
+    else:
+        achieved = algo_bytes / (kern_ms * 1e-3) / 1e9
+        out.update({
+            "metric": "nmg sparsifier GB/s" if kind == "sparsify" else "nmg sparse x dense GEMV-like GB/s",
+            "value": algo_bytes / wall / 1e9, "unit": "GB/s",
+            "config": {"workload": desc, "kernel": args.kernel, "kernel_ms": kern_ms,
+                       "algorithmic_bytes": algo_bytes},
+            "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": achieved / PEAK_HBM_GBS, "traffic": committed_traffic(args.workload)},
+        })
+    if not args.no_cpu and args.workload == "c2":
         out["cpu_baseline"] = cpu_baseline(M, K, N, n, m, g)
     print(json.dumps(out))
 

@@ -268,11 +268,330 @@ static int launch_sparsify(SparsifyParams &P, hipStream_t stream)
     return NMG_OK;
 }
 
+// ------------------------------------------------------------- small tiles: lane teams
+// For tiles of a few hundred columns a wavefront-wide arg-max per step wastes most of the
+// machine on communication.  Here a tile belongs to a *team* of L consecutive lanes (16 tiles
+// per wavefront for L = 4); lane j of the team owns the columns o = j (mod L) and keeps the best
+// of them in registers, so a step is a short scan of the owner's own columns plus log2(L)
+// exchanges inside the team.
+//
+// Heads are maintained lazily: when a pattern fills up, the heads that point to it are left
+// stale.  A stale head is an upper bound of the column's true key (the true head is the best over
+// a subset of the patterns), so the largest head over the free columns is either valid -- then it
+// is the true maximum and is accepted -- or stale, and then only that one column is recomputed
+// over the patterns that still have room and the step is repeated.  Every iteration of a team
+// is therefore one "pop": accept or repair, followed by the owner's rescan.
+//
+// LDS per team: the tile's data, head score (+1, 0 = column taken), head pattern, pattern
+// counters and the idx output; a team region is padded to L (mod 64) words so that the teams of
+// a wavefront, which all touch the same offsets of their regions, hit distinct banks.
+// Exchange inside a team of L consecutive lanes without going through LDS: DPP lane
+// permutations.  After the stages for L the value has been combined over the whole team:
+// quad_perm [1,0,3,2] and [2,3,0,1] reduce a quad, row_half_mirror (i <-> 7-i) joins the two
+// quads of 8 lanes, row_mirror (i <-> 15-i) the two halves of 16.
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_u32(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+template <int CTRL> __device__ __forceinline__ uint64_t dpp_u64(uint64_t v)
+{
+    return ((uint64_t)dpp_u32<CTRL>((uint32_t)(v >> 32)) << 32) | dpp_u32<CTRL>((uint32_t)v);
+}
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_bits(uint32_t v) { return dpp_u32<CTRL>(v); }
+template <int CTRL> __device__ __forceinline__ uint64_t dpp_bits(uint64_t v) { return dpp_u64<CTRL>(v); }
+
+template <int CTRL, typename SB> __device__ __forceinline__ void team_stage(Key<SB> &b)
+{
+    Key<SB> o;
+    o.s = dpp_bits<CTRL>(b.s);
+    o.op = dpp_u32<CTRL>(b.op);
+    if (key_gt(o, b)) b = o;
+}
+template <int L, typename SB> __device__ __forceinline__ Key<SB> team_max(Key<SB> b)
+{
+    if (L >= 2) team_stage<0xB1>(b);    // quad_perm [1,0,3,2]
+    if (L >= 4) team_stage<0x4E>(b);    // quad_perm [2,3,0,1]
+    if (L >= 8) team_stage<0x141>(b);   // row_half_mirror
+    if (L >= 16) team_stage<0x140>(b);  // row_mirror
+    static_assert(L <= 16, "a team lives inside one DPP row of 16 lanes");
+    return b;
+}
+
+struct TeamParams {
+    SparsifyParams sp;
+    int region_bytes;                  // LDS bytes of one team
+    int t_hs, t_hp, t_cnt, t_oidx;     // offsets inside a team region
+    int teams;                         // teams (= tiles) per workgroup
+};
+
+template <typename T, int L>
+__global__ __launch_bounds__(128) void sparsify_teams_kernel(TeamParams Q)
+{
+    using CT = typename ScoreOf<T>::type;
+    using SB = typename ScoreOf<T>::bits;
+    const SparsifyParams &P = Q.sp;
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int n = P.n, m = P.m, g = P.g, c = P.c, cols = P.cols;
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    const int team = tid / L, tl = tid % L;
+    const int teams = Q.teams;
+
+    // LDS: [order table][pattern masks (m <= 8)][team regions]
+    int8_t *s_order = (int8_t *)smem;
+    uint8_t *s_mask = (uint8_t *)(smem + ((c * n + 15) & ~15));
+    const int order_bytes = ((c * n + 15) & ~15) + ((c + 15) & ~15);
+    unsigned char *region = smem + order_bytes + (size_t)team * Q.region_bytes;
+    T *s_d = (T *)region;
+    SB *s_hs = (SB *)(region + Q.t_hs);
+    uint16_t *s_hp = (uint16_t *)(region + Q.t_hp);
+    int16_t *s_cnt = (int16_t *)(region + Q.t_cnt);
+    int16_t *s_oidx = (int16_t *)(region + Q.t_oidx);
+
+    for (int i = tid; i < c * n; i += nthr) s_order[i] = P.order[i];
+    if (m <= 8)
+        for (int p = tid; p < c; p += nthr) {
+            int mk = 0;
+            for (int j = 0; j < n; j++) mk |= 1 << P.order[p * n + j];
+            s_mask[p] = (uint8_t)mk;
+        }
+
+    // ---- cooperative load of the workgroup's tiles (zero beyond G / S); consecutive threads
+    //      take the same column of consecutive tiles, which are adjacent along the sparse dim ----
+    const int64_t tile0 = (int64_t)blockIdx.x * teams;
+    const T *dense = (const T *)P.dense;
+    const int per_tile = cols * m;
+    const int64_t tiles_per_b = P.view.num_chunks * P.view.num_blocks;
+    for (int e = tid; e < teams * per_tile; e += nthr) {
+        const int r = e % m;
+        const int rest = e / m;
+        const int tm = rest % teams;
+        const int o = rest / teams;
+        const int64_t t = tile0 + tm;
+        T v = Zero<T>::v();
+        if (t < P.outer) {
+            const int64_t b = t / tiles_per_b;
+            const int64_t rem = t - b * tiles_per_b;
+            const int64_t kc = rem / P.view.num_blocks;
+            const int64_t mb = rem - kc * P.view.num_blocks;
+            const int64_t gi = kc * cols + o, si = mb * m + r;
+            if (gi < P.view.G && si < P.view.S)
+                v = dense[b * P.view.stride_b + gi * P.view.stride_g + si * P.view.stride_s];
+        }
+        ((T *)(smem + order_bytes + (size_t)tm * Q.region_bytes))[o * m + r] = v;
+    }
+    if (team < teams)
+        for (int p = tl; p < c; p += L) s_cnt[p] = 0;
+    __syncthreads();
+
+    const bool live = team < teams && tile0 + team < P.outer;
+
+    // Best key of column o over the patterns that still have room: score bits + 1 and pattern.
+    // LDS reads are issued in batches of independent loads (the column first, then 8 patterns'
+    // masks and counters at a time): the loop is latency-bound, not throughput-bound.
+    auto head_of = [&](int o, SB &best_s, int &best_p) {
+        best_p = 0;
+        best_s = 0;
+        const T *col = s_d + o * m;
+        if (m <= 8) {
+            CT a[8];
+#pragma unroll
+            for (int r = 0; r < 8; r++) a[r] = score_of(col[r < m ? r : 0]);
+            for (int p0 = 0; p0 < c; p0 += 8) {
+                int mk[8], cn[8];
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const int p = p0 + i < c ? p0 + i : c - 1;
+                    mk[i] = s_mask[p];
+                    cn[i] = s_cnt[p];
+                }
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    if (p0 + i >= c || cn[i] >= g) continue;
+                    // left-to-right sum over the pattern's positions (ascending), as the reference
+                    CT acc = 0;
+#pragma unroll
+                    for (int r = 0; r < 8; r++)
+                        if ((mk[i] >> r) & 1) acc += a[r];
+                    const SB sb = score_bits(acc) + 1;
+                    if (sb >= best_s) {  // ties: larger p wins
+                        best_s = sb;
+                        best_p = p0 + i;
+                    }
+                }
+            }
+            return;
+        }
+        for (int p = 0; p < c; p++) {
+            if (s_cnt[p] >= g) continue;
+            CT acc = 0;
+            for (int j = 0; j < n; j++) acc += score_of(col[s_order[p * n + j]]);
+            const SB sb = score_bits(acc) + 1;
+            if (sb >= best_s) {
+                best_s = sb;
+                best_p = p;
+            }
+        }
+    };
+    // Largest head among this lane's free columns (ties: larger o wins); s == 0 when none is left.
+    // A lane owns at most 32 columns (the launcher picks L accordingly).
+    auto local_best = [&]() {
+        Key<SB> lb;
+        lb.s = 0;
+        lb.op = 0;
+        SB v[32];
+#pragma unroll
+        for (int i = 0; i < 32; i++) {
+            const int o = tl + L * i;
+            v[i] = s_hs[o < cols ? o : tl];
+        }
+        SB best_s = 1;
+        int best_o = -1;
+#pragma unroll
+        for (int i = 0; i < 32; i++) {
+            const int o = tl + L * i;
+            if (o < cols && v[i] >= best_s) {
+                best_s = v[i];
+                best_o = o;
+            }
+        }
+        if (best_o >= 0) {
+            lb.s = best_s;
+            lb.op = ((uint32_t)best_o << 16) | s_hp[best_o];
+        }
+        return lb;
+    };
+
+    Key<SB> lb;
+    lb.s = 0;
+    lb.op = 0;
+    if (live) {
+        for (int o = tl; o < cols; o += L) {
+            SB bs;
+            int bp;
+            head_of(o, bs, bp);
+            s_hs[o] = bs;
+            s_hp[o] = (uint16_t)bp;
+        }
+        lb = local_best();
+    }
+
+    // Every column is accepted once and repaired at most once per pattern that fills up, which
+    // bounds the loop whatever the data.
+    int accepted = live ? 0 : cols;
+    const int max_iter = cols * (c + 1);
+    for (int iter = 0; iter < max_iter && __any(accepted < cols); iter++) {
+        if (accepted < cols) {
+            // ---- team arg-max ----
+            const Key<SB> b = team_max<L>(lb);
+            const int o_star = (int)(b.op >> 16), p_star = (int)(b.op & 0xFFFFu);
+            const int cntp = s_cnt[p_star];
+            const bool stale = cntp >= g;
+            if (o_star % L == tl) {
+                if (stale) {
+                    SB bs;
+                    int bp;
+                    head_of(o_star, bs, bp);
+                    s_hs[o_star] = bs;
+                    s_hp[o_star] = (uint16_t)bp;
+                } else {
+                    s_cnt[p_star] = (int16_t)(cntp + 1);
+                    s_hs[o_star] = 0;
+                    s_oidx[p_star * g + cntp] = (int16_t)o_star;
+                }
+                lb = local_best();
+            }
+            if (!stale) accepted++;
+        }
+        // the team's LDS writes must be visible to its other lanes in the next iteration
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    // ---- coalesced store of the workgroup's tiles: val is gathered from the tile data ----
+    __syncthreads();
+    T *val = (T *)P.val;
+    for (int e = tid; e < teams * cols * n; e += nthr) {
+        const int tm = e / (cols * n), i = e - tm * (cols * n);
+        const int64_t t = tile0 + tm;
+        if (t >= P.outer) break;
+        const unsigned char *reg = smem + order_bytes + (size_t)tm * Q.region_bytes;
+        const int slot = i / n, j = i - slot * n;
+        const int o = ((const int16_t *)(reg + Q.t_oidx))[slot];
+        val[t * (int64_t)(cols * n) + i] = ((const T *)reg)[o * m + s_order[(slot / g) * n + j]];
+    }
+    for (int e = tid; e < teams * cols; e += nthr) {
+        const int tm = e / cols, slot = e - tm * cols;
+        const int64_t t = tile0 + tm;
+        if (t >= P.outer) break;
+        P.idx[t * (int64_t)cols + slot] =
+            ((const int16_t *)(smem + order_bytes + (size_t)tm * Q.region_bytes + Q.t_oidx))[slot];
+    }
+}
+
+template <typename T, int L> static int launch_sparsify_teams(SparsifyParams &P, hipStream_t stream, bool *done)
+{
+    using SB = typename ScoreOf<T>::bits;
+    *done = false;
+    TeamParams Q{};
+    Q.sp = P;
+    const int cols = P.cols, m = P.m, c = P.c, n = P.n;
+    int off = align_up(cols * m * (int)sizeof(T), 8);
+    Q.t_hs = off;
+    off = align_up(off + cols * (int)sizeof(SB), 4);
+    Q.t_hp = off;
+    off = align_up(off + cols * 2, 4);
+    Q.t_cnt = off;
+    off = align_up(off + c * 2, 4);
+    Q.t_oidx = off;
+    off = align_up(off + cols * 2, 4);
+    // region size = L (mod 64) words spreads the teams of a wavefront over the banks; regions of
+    // 8-byte data stay 8-byte aligned (an even number of words)
+    int words = off / 4, target = L % 64;
+    if ((sizeof(T) == 8 || sizeof(SB) == 8) && (target & 1)) target++;
+    while (words % 64 != target) words++;
+    Q.region_bytes = words * 4;
+    const size_t order_bytes = (size_t)align_up(c * n, 16) + (size_t)align_up(c, 16);
+    // workgroups of 128 threads when two of them fit in a CU's LDS, else 64 threads
+    int threads = 128;
+    size_t lds = order_bytes + (size_t)(threads / L) * Q.region_bytes;
+    if (lds > 80 * 1024) {
+        threads = 64;
+        lds = order_bytes + (size_t)(threads / L) * Q.region_bytes;
+    }
+    if (lds > 160 * 1024) return NMG_OK;   // too large for this kernel: the caller falls back
+    Q.teams = threads / L;
+    auto kern = sparsify_teams_kernel<T, L>;
+    if (lds > 64 * 1024)
+        NMG_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)lds));
+    const int64_t grid = (P.outer + Q.teams - 1) / Q.teams;
+    NMG_REQUIRE(grid <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "too many tiles (%lld)", (long long)grid);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(threads), lds, stream, Q);
+    NMG_HIP_TRY(hipGetLastError());
+    *done = true;
+    return NMG_OK;
+}
+
 template <typename T> static int dispatch_sparsify(SparsifyParams &P, hipStream_t stream)
 {
+    // Small tiles: one wavefront per tile, four tiles per workgroup.  Larger tiles: four
+    // wavefronts per tile -- more of them lose to the two workgroup barriers of every step
+    // (measured on 896-column tiles: 1 / 2 / 4 / 8 / 16 wavefronts -> 17.6 / 12.6 / 10.9 / 21.1 / 69 ms
+    // for an 8192 x 8192 weight).
+    if (P.cols <= 512 && P.n > 0) {
+        // lane teams: about 16 to 32 columns per lane
+        bool done = false;
+        int rc;
+        if (P.cols <= 32) rc = launch_sparsify_teams<T, 1>(P, stream, &done);
+        else if (P.cols <= 64) rc = launch_sparsify_teams<T, 2>(P, stream, &done);
+        else if (P.cols <= 128) rc = launch_sparsify_teams<T, 4>(P, stream, &done);
+        else if (P.cols <= 256) rc = launch_sparsify_teams<T, 8>(P, stream, &done);
+        else rc = launch_sparsify_teams<T, 16>(P, stream, &done);
+        if (rc != NMG_OK || done) return rc;
+    }
     if (P.cols <= 128) return launch_sparsify<T, 1, 4>(P, stream);
-    if (P.cols <= 512) return launch_sparsify<T, 4, 1>(P, stream);
-    return launch_sparsify<T, 16, 1>(P, stream);
+    return launch_sparsify<T, 4, 1>(P, stream);
 }
 
 static int check_common(const nmg_view *view, int n, int m, int g, int dtype, TileGeom *tg)

@@ -41,6 +41,25 @@ def test_dtypes_and_ratios(dtype, n, m, g):
     check_parity(w, n, m, 1, g, 0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.float64])
+@pytest.mark.parametrize("n,m,g", [
+    (1, 2, 3),     # 6 columns per tile: one lane per tile
+    (2, 4, 4),     # 24 columns
+    (1, 4, 16),    # 64 columns: two lanes per tile
+    (2, 4, 8),     # 48 columns
+    (2, 8, 4),     # 112 columns, 28 patterns: four lanes per tile
+    (3, 6, 16),    # 320 columns: sixteen lanes per tile
+    (2, 8, 16),    # 448 columns
+    (4, 4, 5),     # n == m: one pattern
+])
+def test_small_tile_team_kernel_sizes(dtype, n, m, g):
+    # many ties (few distinct magnitudes) in one input, continuous values in the other
+    gen = torch.Generator().manual_seed(n * 1000 + m * 10 + g)
+    ties = torch.randint(-3, 4, (150, 200), generator=gen).to(dtype)
+    check_parity(ties, n, m, 1, g, 0)
+    check_parity(seeded((257, 130), dtype, seed=g, std=0.02), n, m, 0, g, 1)
+
+
 def test_4_8_32_large_tile():
     w = seeded((2240 + 100, 72), torch.float16, seed=48, std=0.02)
     check_parity(w, 4, 8, 1, 32, 0)
