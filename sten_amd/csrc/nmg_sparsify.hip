@@ -360,25 +360,30 @@ __global__ __launch_bounds__(128) void sparsify_teams_kernel(TeamParams Q)
     //      take the same column of consecutive tiles, which are adjacent along the sparse dim ----
     const int64_t tile0 = (int64_t)blockIdx.x * teams;
     const T *dense = (const T *)P.dense;
-    const int per_tile = cols * m;
     const int64_t tiles_per_b = P.view.num_chunks * P.view.num_blocks;
-    for (int e = tid; e < teams * per_tile; e += nthr) {
-        const int r = e % m;
-        const int rest = e / m;
-        const int tm = rest % teams;
-        const int o = rest / teams;
+    // A thread keeps one (tile, position r) pair and walks the tile's columns, so the 64-bit
+    // index arithmetic is done once per pair and the loads of the walk are independent.
+    for (int pair = tid; pair < teams * m; pair += nthr) {
+        const int tm = pair / m, r = pair - tm * m;
         const int64_t t = tile0 + tm;
-        T v = Zero<T>::v();
+        T *dst = (T *)(smem + order_bytes + (size_t)tm * Q.region_bytes) + r;
+        const T *src = nullptr;
+        int valid_cols = 0;
         if (t < P.outer) {
             const int64_t b = t / tiles_per_b;
             const int64_t rem = t - b * tiles_per_b;
             const int64_t kc = rem / P.view.num_blocks;
             const int64_t mb = rem - kc * P.view.num_blocks;
-            const int64_t gi = kc * cols + o, si = mb * m + r;
-            if (gi < P.view.G && si < P.view.S)
-                v = dense[b * P.view.stride_b + gi * P.view.stride_g + si * P.view.stride_s];
+            const int64_t si = mb * m + r;
+            if (si < P.view.S) {
+                src = dense + b * P.view.stride_b + kc * cols * P.view.stride_g + si * P.view.stride_s;
+                const int64_t left = P.view.G - kc * cols;
+                valid_cols = left < cols ? (int)left : cols;
+            }
         }
-        ((T *)(smem + order_bytes + (size_t)tm * Q.region_bytes))[o * m + r] = v;
+        const int64_t sg = P.view.stride_g;
+#pragma unroll 8
+        for (int o = 0; o < cols; o++) dst[o * m] = o < valid_cols ? src[o * sg] : Zero<T>::v();
     }
     if (team < teams)
         for (int p = tl; p < c; p += L) s_cnt[p] = 0;
@@ -411,8 +416,10 @@ __global__ __launch_bounds__(128) void sparsify_teams_kernel(TeamParams Q)
                     // left-to-right sum over the pattern's positions (ascending), as the reference
                     CT acc = 0;
 #pragma unroll
-                    for (int r = 0; r < 8; r++)
+                    for (int r = 0; r < 8; r++) {
+                        if (r >= m) break;
                         if ((mk[i] >> r) & 1) acc += a[r];
+                    }
                     const SB sb = score_bits(acc) + 1;
                     if (sb >= best_s) {  // ties: larger p wins
                         best_s = sb;
@@ -434,27 +441,46 @@ __global__ __launch_bounds__(128) void sparsify_teams_kernel(TeamParams Q)
         }
     };
     // Largest head among this lane's free columns (ties: larger o wins); s == 0 when none is left.
-    // A lane owns at most 32 columns (the launcher picks L accordingly).
-    auto local_best = [&]() {
-        Key<SB> lb;
-        lb.s = 0;
-        lb.op = 0;
-        SB v[32];
+    // A lane owns at most 32 columns (the launcher picks L accordingly), kept as 4 groups of 8
+    // whose maxima live in registers: a change rescans one group only.
+    SB gs[4] = {0, 0, 0, 0};
+    int go[4] = {0, 0, 0, 0};
+    auto scan_group = [&](int k) {
+        SB v[8];
 #pragma unroll
-        for (int i = 0; i < 32; i++) {
-            const int o = tl + L * i;
+        for (int i = 0; i < 8; i++) {
+            const int o = tl + L * (k * 8 + i);
             v[i] = s_hs[o < cols ? o : tl];
         }
-        SB best_s = 1;
-        int best_o = -1;
+        SB best_s = 0;
+        int best_o = 0;
 #pragma unroll
-        for (int i = 0; i < 32; i++) {
-            const int o = tl + L * i;
-            if (o < cols && v[i] >= best_s) {
+        for (int i = 0; i < 8; i++) {
+            const int o = tl + L * (k * 8 + i);
+            if (o < cols && v[i] != 0 && v[i] >= best_s) {
                 best_s = v[i];
                 best_o = o;
             }
         }
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            if (q == k) {
+                gs[q] = best_s;
+                go[q] = best_o;
+            }
+    };
+    auto local_best = [&]() {
+        Key<SB> lb;
+        lb.s = 0;
+        lb.op = 0;
+        SB best_s = 0;
+        int best_o = -1;
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            if (gs[q] != 0 && gs[q] >= best_s) {
+                best_s = gs[q];
+                best_o = go[q];
+            }
         if (best_o >= 0) {
             lb.s = best_s;
             lb.op = ((uint32_t)best_o << 16) | s_hp[best_o];
@@ -473,6 +499,8 @@ __global__ __launch_bounds__(128) void sparsify_teams_kernel(TeamParams Q)
             s_hs[o] = bs;
             s_hp[o] = (uint16_t)bp;
         }
+#pragma unroll
+        for (int k = 0; k < 4; k++) scan_group(k);
         lb = local_best();
     }
 
@@ -499,6 +527,7 @@ __global__ __launch_bounds__(128) void sparsify_teams_kernel(TeamParams Q)
                     s_hs[o_star] = 0;
                     s_oidx[p_star * g + cntp] = (int16_t)o_star;
                 }
+                scan_group((o_star / L) >> 3);
                 lb = local_best();
             }
             if (!stale) accepted++;
