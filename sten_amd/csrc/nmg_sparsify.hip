@@ -322,6 +322,7 @@ struct TeamParams {
     int region_bytes;                  // LDS bytes of one team
     int t_hs, t_hp, t_cnt, t_oidx;     // offsets inside a team region
     int teams;                         // teams (= tiles) per workgroup
+    uint64_t magic_cols, magic_g;      // ceil(2^32 / cols), ceil(2^32 / g): x / d == (x * magic) >> 32 for x < 2^16
 };
 
 template <typename T, int L>
@@ -537,24 +538,21 @@ __global__ __launch_bounds__(128) void sparsify_teams_kernel(TeamParams Q)
         __builtin_amdgcn_wave_barrier();
     }
 
-    // ---- coalesced store of the workgroup's tiles: val is gathered from the tile data ----
+    // ---- coalesced store of the workgroup's tiles: one thread per slot writes its index and
+    //      gathers its n values from the tile data (divisions by multiplication: e < 2^16) ----
     __syncthreads();
     T *val = (T *)P.val;
-    for (int e = tid; e < teams * cols * n; e += nthr) {
-        const int tm = e / (cols * n), i = e - tm * (cols * n);
+    for (int e = tid; e < teams * cols; e += nthr) {
+        const int tm = (int)(((uint64_t)e * Q.magic_cols) >> 32), slot = e - tm * cols;
         const int64_t t = tile0 + tm;
         if (t >= P.outer) break;
         const unsigned char *reg = smem + order_bytes + (size_t)tm * Q.region_bytes;
-        const int slot = i / n, j = i - slot * n;
         const int o = ((const int16_t *)(reg + Q.t_oidx))[slot];
-        val[t * (int64_t)(cols * n) + i] = ((const T *)reg)[o * m + s_order[(slot / g) * n + j]];
-    }
-    for (int e = tid; e < teams * cols; e += nthr) {
-        const int tm = e / cols, slot = e - tm * cols;
-        const int64_t t = tile0 + tm;
-        if (t >= P.outer) break;
-        P.idx[t * (int64_t)cols + slot] =
-            ((const int16_t *)(smem + order_bytes + (size_t)tm * Q.region_bytes + Q.t_oidx))[slot];
+        const int p = (int)(((uint64_t)slot * Q.magic_g) >> 32);
+        const T *col = (const T *)reg + o * m;
+        const int64_t at = t * (int64_t)cols + slot;
+        P.idx[at] = (int16_t)o;
+        for (int j = 0; j < n; j++) val[at * n + j] = col[s_order[p * n + j]];
     }
 }
 
@@ -590,6 +588,8 @@ template <typename T, int L> static int launch_sparsify_teams(SparsifyParams &P,
     }
     if (lds > 160 * 1024) return NMG_OK;   // too large for this kernel: the caller falls back
     Q.teams = threads / L;
+    Q.magic_cols = (((uint64_t)1 << 32) + cols - 1) / cols;
+    Q.magic_g = (((uint64_t)1 << 32) + P.g - 1) / P.g;
     auto kern = sparsify_teams_kernel<T, L>;
     if (lds > 64 * 1024)
         NMG_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
