@@ -15,7 +15,10 @@ from .impls import GroupedNMSparsifier, install
 from .layout import NMGLayout
 from .native import NmgError
 from .tensor import GroupedNMTensor, spmm
+from . import w4
+from .w4 import SparseMarlinSparsifier, SparseMarlinTensor
 
 install(dispatch)
+w4.install(dispatch)
 
 __all__ = [n for n in dir() if not n.startswith("_")]

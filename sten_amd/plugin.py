@@ -10,7 +10,7 @@ registration of a sparsifier key (sten.py:1096-1100), so existing keys are remov
 """
 import torch
 
-from . import impls
+from . import impls, w4
 from .tensor import GroupedNMTensor
 
 
@@ -29,4 +29,7 @@ def register(sten_module):
     # expose the GPU classes under the names user code already uses
     sten_module.GroupedNMTensor = GroupedNMTensor
     sten_module.GroupedNMSparsifier = impls.GroupedNMSparsifier
-    return impls.install(sten_module)
+    impls.install(sten_module)
+    w4_key = (w4.SparseMarlinSparsifier, torch.Tensor, w4.SparseMarlinTensor)
+    if reg is None or w4_key not in reg:
+        w4.install(sten_module)

@@ -1,0 +1,98 @@
+"""2:4 + int4 decode path: the HIP packing against its numpy restatement (bit-exact), the product
+against the dequantised dense matmul (rel-L2 <= 1e-3, fp16 with fp32 accumulation), and the
+registration pattern of the reference's test (tests/test_sparse_marlin.py:76-133).
+Parity against the reference itself is unpinned: its test asserts nothing."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import w4_oracle as W
+from helpers import rel_l2, seeded, to_np
+
+
+def test_oracle_round_trip_properties():
+    rng = np.random.default_rng(0)
+    w = (rng.standard_normal((40, 256)) * 0.02).astype(np.float16)
+    pos, q, s = W.prune_quantise(w)
+    # exactly two kept per group of 4, increasing positions, the two largest magnitudes
+    assert (pos[:, :, 0] < pos[:, :, 1]).all()
+    a = np.abs(w.astype(np.float32)).reshape(40, 64, 4)
+    kept = np.take_along_axis(a, pos.astype(np.int64), axis=2)
+    assert (np.sort(a, axis=2)[:, :, 2:] == np.sort(kept, axis=2)).all()
+    d = W.dequantise(pos, q, s, 256)
+    # quantisation error of a kept value: half a step of its group, plus the fp16 roundings of the
+    # scale and of the dequantised product
+    step = np.repeat(s.astype(np.float32), 128, axis=1)
+    mask = d != 0
+    wf = w.astype(np.float32)
+    assert (np.abs(d.astype(np.float32) - wf)[mask] <= 0.5 * step[mask] + np.abs(wf)[mask] * 2.0 ** -9).all()
+    assert (q <= 15).all() and (np.abs(q.astype(int) - 8).reshape(40, 2, 64).max(axis=2) == 7).all()
+
+
+def test_oracle_hand_worked_group():
+    # one row, one group of 128: first group of 4 = (1, -7, 3, 7): keep -7 (pos 1) and 7 (pos 3);
+    # the rest zeros -> scale 1, nibbles 1 and 15
+    w = np.zeros((1, 128), dtype=np.float16)
+    w[0, :4] = [1, -7, 3, 7]
+    pos, q, s = W.prune_quantise(w)
+    assert pos[0, 0].tolist() == [1, 3] and q[0, 0].tolist() == [1, 15] and float(s[0, 0]) == 1.0
+    assert pos[0, 1].tolist() == [0, 1] and q[0, 1].tolist() == [8, 8]          # all-zero group: ties
+    d = W.dequantise(pos, q, s, 128)
+    assert d[0, :4].tolist() == [0, -7, 0, 7]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K", [(32, 128), (100, 256), (344, 1024), (64, 4096)])
+def test_hip_packing_is_bit_exact(M, K):
+    import sten_amd as sten
+    print(f"case w4 pack M={M} K={K}", flush=True)
+    w = seeded((M, K), torch.float16, seed=M + K, std=0.02)
+    w[0, :8] = torch.tensor([1, -1, 1, 1, 0, 0, 0, 0], dtype=torch.float16)      # ties and an all-zero group
+    t = sten.SparseMarlinTensor.from_dense(w.to("cuda:0"))
+    pos, q, s = W.prune_quantise(to_np(w))
+    B, meta, sc = W.pack(pos, q, s, M, K)
+    assert np.array_equal(to_np(t.B), B)
+    assert np.array_equal(to_np(t.meta).view(np.uint32), meta)
+    assert np.array_equal(to_np(t.s).view(np.uint16), sc.view(np.uint16))
+    assert np.array_equal(to_np(t.to_dense()).view(np.uint16), W.dequantise(pos, q, s, K).view(np.uint16))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T", [1, 4, 16])
+@pytest.mark.parametrize("M,K", [(100, 256), (1000, 1024), (344, 4096)])
+def test_hip_linear_matches_dequantised_matmul(M, K, T):
+    import sten_amd as sten
+    print(f"case w4 linear M={M} K={K} T={T}", flush=True)
+    w = seeded((M, K), torch.float16, seed=M + K + T, std=0.02)
+    x = seeded((T, K), torch.float16, seed=7)
+    b = seeded((M,), torch.float16, seed=8)
+    t = sten.SparseMarlinTensor.from_dense(w.to("cuda:0"))
+    pos, q, s = W.prune_quantise(to_np(w))
+    wd = W.dequantise(pos, q, s, K)
+    y = t.linear(x.to("cuda:0"), b.to("cuda:0"))
+    assert y.shape == (T, M)
+    assert rel_l2(to_np(y), W.linear(wd, to_np(x), to_np(b))) <= 1e-3
+    y0 = t.linear(x.to("cuda:0"))
+    assert rel_l2(to_np(y0), W.linear(wd, to_np(x))) <= 1e-3
+
+
+@pytest.mark.gpu
+def test_registered_linear_like_the_reference_test():
+    # tests/test_sparse_marlin.py:119-133 sparsifies every MLP weight of a model and runs it; here
+    # a local two-layer MLP stands in for the hub model
+    import sten_amd as sten
+    torch.manual_seed(0)
+    model = torch.nn.Sequential(torch.nn.Linear(256, 384, bias=False), torch.nn.Linear(384, 128)).half().to("cuda:0")
+    x = torch.randn(4, 256, dtype=torch.float16, device="cuda:0")
+    sb = sten.SparsityBuilder()
+    for name in ("0.weight", "1.weight"):
+        sb.set_weight(name, initial_sparsifier=sten.SparseMarlinSparsifier(), out_format=sten.SparseMarlinTensor)
+    sparse = sb.get_sparse_model(model)
+    with torch.no_grad():
+        y = sparse(x)
+        w0 = sparse[0].weight.wrapped_tensor.to_dense()
+        w1 = sparse[1].weight.wrapped_tensor.to_dense()
+        ref = torch.nn.functional.linear(torch.nn.functional.linear(x, w0), w1, model[1].bias)
+    assert rel_l2(to_np(y), to_np(ref)) <= 2e-3
+    with pytest.raises(sten.NmgError):
+        sten.SparseMarlinTensor.from_dense(torch.zeros(8, 100, dtype=torch.float16, device="cuda:0"))
