@@ -46,6 +46,9 @@ WORKLOADS = {
     "c2_grad_x": ("grad_x", 4096, 4096, 2048, 2, 4, 16, "configs[1] shape: dY 2048x4096 x W 4096x4096 fp16 2:4:16, grad_input"),
     "decode_1": ("decode", 4096, 11008, 1, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 1 token"),
     "decode_16": ("decode", 4096, 11008, 16, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 16 tokens"),
+    "c4_b1": ("w4", 11008, 4096, 1, 2, 4, 1, "configs[3]: W 11008x4096 2:4 + int4 (scale per 128) x 1 token"),
+    "c4_b4": ("w4", 11008, 4096, 4, 2, 4, 1, "configs[3]: W 11008x4096 2:4 + int4 (scale per 128) x 4 tokens"),
+    "c4_b16": ("w4", 11008, 4096, 16, 2, 4, 1, "configs[3]: W 11008x4096 2:4 + int4 (scale per 128) x 16 tokens"),
     "sparsify_c2": ("sparsify", 4096, 4096, 0, 2, 4, 16, "configs[1]: sparsify W 4096x4096 fp16 to 2:4:16"),
     "sparsify_c3_2_8": ("sparsify", 8192, 8192, 0, 2, 8, 32, "configs[2]: sparsify W 8192x8192 fp16 to 2:8:32"),
 }
@@ -130,7 +133,16 @@ def main():
     torch.manual_seed(0)
     W = (torch.randn(M, K) * 0.02).half().to(dev)
 
-    if kind == "sparsify":
+    if kind == "w4":
+        w = sten.SparseMarlinTensor.from_dense(W)
+        del W
+        X = torch.randn(N, K).half().to(dev)
+
+        def step():
+            return w.linear(X)
+        # int4 kept values + 2-bit positions + fp16 scales + activations + output
+        algo_bytes = M * K // 4 + M * K // 8 + (K // 128) * M * 2 + N * K * 2 + N * M * 2
+    elif kind == "sparsify":
         def step():
             return sten.GroupedNMTensor.from_dense(W, n, m, sparse_dim=1, group_size=g, group_dim=0)
         w = step()
@@ -194,7 +206,7 @@ def main():
     else:
         achieved = algo_bytes / (kern_ms * 1e-3) / 1e9
         out.update({
-            "metric": "nmg sparsifier GB/s" if kind == "sparsify" else "nmg sparse x dense GEMV-like GB/s",
+            "metric": "nmg sparsifier GB/s" if kind == "sparsify" else "nmg sparse x dense decode GB/s",
             "value": algo_bytes / wall / 1e9, "unit": "GB/s",
             "config": {"workload": desc, "kernel": args.kernel, "kernel_ms": kern_ms,
                        "algorithmic_bytes": algo_bytes},
