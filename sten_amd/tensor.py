@@ -132,6 +132,14 @@ class GroupedNMTensor:
     def clone(self):
         return self.to(copy=True)
 
+    # ---- serialization: the canonical val/idx and the layout; derived operands are rebuilt ----
+    def __getstate__(self):
+        return {"val": self.val, "idx": self.idx, "layout": self.layout, "spmm_opt": dict(self.spmm_opt)}
+
+    def __setstate__(self, state):
+        self.__init__(state["val"], state["idx"], state["layout"])
+        self.spmm_opt = state.get("spmm_opt", {"kernel": "auto"})
+
     # ---- in-place updates that keep the pattern (used by optimizers) ------------------------
     def _other_val(self, other):
         if isinstance(other, GroupedNMTensor):

@@ -338,3 +338,22 @@ def test_densefrag_route_both_directions(dense_variant, dtype, M, K, T, n, m, g)
         assert rel_l2(to_np(y), ref) <= TOL[dtype], sd
         gx = sten.spmm(w, gy.to(DEV), reduce_dim=0, kernel="densefrag")
         assert rel_l2(to_np(gx), to_np(gy).astype(np.float64) @ Wd) <= TOL[dtype], sd
+
+
+def test_serialization_round_trip(tmp_path):
+    # reference: tests/test_serialization.py saves and loads a model with sparse weights
+    import pickle
+    W = seeded((128, 128), torch.float16, seed=11, std=0.5)
+    w = make(W, 2, 4, 16, 1)
+    x = seeded((32, 128), torch.float16, seed=12).to(DEV)
+    y = sten.spmm(w, x, reduce_dim=1)                    # builds the cached operands
+    w2 = pickle.loads(pickle.dumps(w))
+    assert torch.equal(w2.val, w.val) and torch.equal(w2.idx, w.idx) and w2.layout == w.layout
+    assert torch.equal(sten.spmm(w2, x, reduce_dim=1), y)
+    lin = build_sparse_linear(torch.nn.Linear(128, 128).half().to(DEV), 2, 4, 16, 1)
+    path = tmp_path / "model.pt"
+    torch.save(lin, path)
+    lin2 = torch.load(path, weights_only=False)          # a file this test wrote itself
+    assert isinstance(lin2.weight, sten.SparseParameterWrapper)
+    with torch.no_grad():
+        assert torch.equal(lin2(x), lin(x))
