@@ -357,3 +357,55 @@ def test_serialization_round_trip(tmp_path):
     assert isinstance(lin2.weight, sten.SparseParameterWrapper)
     with torch.no_grad():
         assert torch.equal(lin2(x), lin(x))
+
+
+def _check_structure(w, n, m):
+    """Size-independent properties of a compressed weight: every block of m keeps at most n
+    entries, and the dense form reproduces the kept entries."""
+    d = w.to_dense()
+    blocks = d.reshape(d.shape[0], -1, m)
+    assert int((blocks != 0).sum(dim=2).max()) <= n
+    return d
+
+
+@pytest.mark.parametrize("n,m", [(2, 8), (4, 8)])
+def test_full_size_config3_forward(n, m):
+    # BASELINE config 3 at full size (8192 x 8192, group 32, 4096 tokens): structure of the
+    # compressed weight, the product against the dense product of its own dense form, linearity
+    print(f"case full size config 3 {n}:{m}", flush=True)
+    torch.manual_seed(0)
+    W = (torch.randn(8192, 8192) * 0.02).half().to(DEV)
+    X = torch.randn(4096, 8192).half().to(DEV)
+    w = sten.GroupedNMTensor.from_dense(W, n, m, sparse_dim=1, group_size=32, group_dim=0)
+    d = _check_structure(w, n, m)
+    kept = d != 0
+    assert torch.equal(d[kept], W[kept])
+    y = sten.spmm(w, X, reduce_dim=1)
+    ref = torch.nn.functional.linear(X, d).float()
+    assert float((y.float() - ref).norm() / ref.norm()) <= 1e-3
+    y2 = sten.spmm(w, -0.5 * X, reduce_dim=1).float()
+    assert float((y2 + 0.5 * y.float()).norm() / y2.norm()) <= 1e-3
+
+
+def test_full_size_config5_training_step_pieces():
+    # BASELINE config 5 at full size: forward, grad_input (transposed product) and the masked
+    # weight gradient in val layout, each against the dense computation on the dense form
+    print("case full size config 5", flush=True)
+    torch.manual_seed(0)
+    W = (torch.randn(16384, 4096) * 0.02).half().to(DEV)
+    X = torch.randn(4096, 4096).half().to(DEV)
+    dY = torch.randn(4096, 16384).half().to(DEV)
+    w = sten.GroupedNMTensor.from_dense(W, 2, 4, sparse_dim=1, group_size=16, group_dim=0)
+    d = _check_structure(w, 2, 4)
+    y = sten.spmm(w, X, reduce_dim=1).float()
+    ref = torch.nn.functional.linear(X, d).float()
+    assert float((y - ref).norm() / ref.norm()) <= 1e-3
+    gx = sten.spmm(w, dY, reduce_dim=0).float()
+    ref = torch.mm(dY, d).float()
+    assert float((gx - ref).norm() / ref.norm()) <= 1e-3
+    gw_dense = torch.mm(dY.t(), X)                       # dense product; masked by the gather
+    gw = w.clone_layout(gw_dense)
+    assert torch.equal(gw.idx, w.idx)
+    mask = w.clone_layout(torch.ones_like(W)).to_dense() != 0     # kept positions (a kept weight may be 0)
+    back = gw.to_dense()
+    assert torch.equal(back[mask], gw_dense[mask]) and not bool(back[~mask].any())
