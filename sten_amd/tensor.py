@@ -200,10 +200,15 @@ class GroupedNMTensor:
 
     def densefrag(self, reduce_dim):
         """The weight as the A operand of the dense matrix cores, [outputs, reduction] in
-        fragment order, expanded from the rowpack operand into fresh scratch (not cached: it
-        is as large as the dense weight)."""
+        fragment order, expanded from the rowpack operand into fresh scratch.  It is as large as
+        the dense weight, so it is rebuilt per call unless ``spmm_opt["cache_dense"]`` is set
+        (inference on a frozen weight: trades the memory saving for one pass less per call)."""
         lay = self.layout
         lib = native.load()
+        key = (self.val.data_ptr(), self.val._version, self.idx.data_ptr(), reduce_dim)
+        cached = getattr(self, "_densefrag", None)
+        if self.spmm_opt.get("cache_dense") and cached is not None and cached[0] == key:
+            return cached[1]
         pk_val, pk_pat = self.rowpack()
         O, K = lay.dense_shape[1 - reduce_dim], lay.dense_shape[reduce_dim]
         elems = ctypes.c_int64(0)
@@ -214,6 +219,7 @@ class GroupedNMTensor:
             native.check(lib.nmg_densefrag(
                 native.ptr(pk_val), native.ptr(pk_pat), lay.G, lay.S, transpose, native.ptr(df),
                 lay.n, lay.m, native.dtype_code(df.dtype), native.stream_ptr(df.device)))
+        self._densefrag = (key, df) if self.spmm_opt.get("cache_dense") else None
         return df
 
     def dense_operand(self, reduce_dim):

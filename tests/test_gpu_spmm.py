@@ -409,3 +409,15 @@ def test_full_size_config5_training_step_pieces():
     mask = w.clone_layout(torch.ones_like(W)).to_dense() != 0     # kept positions (a kept weight may be 0)
     back = gw.to_dense()
     assert torch.equal(back[mask], gw_dense[mask]) and not bool(back[~mask].any())
+
+
+def test_cached_dense_operand_follows_weight_updates():
+    W = seeded((256, 256), torch.float16, seed=21, std=0.5)
+    w = make(W, 4, 8, 8, 1)
+    w.spmm_opt["cache_dense"] = True
+    x = seeded((64, 256), torch.float16, seed=22).to(DEV)
+    y1 = sten.spmm(w, x, reduce_dim=1)
+    assert torch.equal(sten.spmm(w, x, reduce_dim=1), y1)          # served from the cache
+    w.mul_(2.0)                                                     # in-place update invalidates it
+    y2 = sten.spmm(w, x, reduce_dim=1)
+    assert rel_l2(to_np(y2), 2.0 * to_np(y1).astype(np.float64)) <= 1e-3
