@@ -45,6 +45,8 @@ WORKLOADS = {
     "c5_grad_x": ("grad_x", 16384, 4096, 4096, 2, 4, 16, "configs[4]: dY 4096x16384 x W 16384x4096 fp16 2:4:16, grad_input"),
     "c2_grad_x": ("grad_x", 4096, 4096, 2048, 2, 4, 16, "configs[1] shape: dY 2048x4096 x W 4096x4096 fp16 2:4:16, grad_input"),
     "decode_1": ("decode", 4096, 11008, 1, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 1 token"),
+    "decode_4": ("decode", 4096, 11008, 4, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 4 tokens"),
+    "decode_8": ("decode", 4096, 11008, 8, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 8 tokens"),
     "decode_16": ("decode", 4096, 11008, 16, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 16 tokens"),
     "c4_b1": ("w4", 11008, 4096, 1, 2, 4, 1, "configs[3]: W 11008x4096 2:4 + int4 (scale per 128) x 1 token"),
     "c4_b4": ("w4", 11008, 4096, 4, 2, 4, 1, "configs[3]: W 11008x4096 2:4 + int4 (scale per 128) x 4 tokens"),

@@ -870,6 +870,177 @@ template <typename T, int NW, int UN> static int launch_smfmac_skinny(SmfParams 
     return NMG_OK;
 }
 
+// Decode kernel with staged activations (the default when K % 128 == 0).  In the kernel above a
+// wavefront's activation loads touch 32 bytes of each token row per instruction (two lanes per
+// token); from 8 tokens on the activations weigh as much as the weight in the vector memory
+// path (18.7 us against 12.7 us here at 16 tokens on a 4096 x 11008 weight; 12.0 against 9.9 at
+// one token).  Here a wavefront stages the
+// activations of its next 128 reduction positions in LDS with row-contiguous DMA loads (256 bytes
+// per token and instruction) and reads its fragments from there.  The staging area is private to
+// the wavefront, so no barrier is involved: a chunk's DMA loads are issued before its weight
+// loads, and the counted wait for the chunk covers both.
+// Chunk = 2 k pairs (128 dense positions): ND DMA loads (4 token rows each) + 6 weight loads.
+// One chunk is in flight while the previous one is multiplied.  16-byte pieces of a row are
+// XOR-swizzled with the row number so that the 16 rows of a fragment read hit distinct banks.
+template <typename T, int SK_NW, int ND>
+__global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_decode_staged_kernel(SmfParams P)
+{
+    using S = Smf<T>;
+    constexpr int OPS = ND + 6;
+    constexpr int BUF = 16 * 256;                       // one chunk: 16 token rows x 256 bytes
+    extern __shared__ __align__(16) unsigned char smem[];
+    static_assert(SK_NW * 2 * BUF >= SK_NW * 32 * 17 * 4, "the reduction buffer reuses the staging area");
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int mb = blockIdx.x;
+    const int KP = P.KP;
+    const int j = lane & 31, h = lane >> 5;
+    // an even number of k pairs per wavefront: chunks never straddle two ranges (KP is even)
+    const int per = (((KP + SK_NW - 1) / SK_NW) + 1) & ~1;
+    const int kp_lo = wave * per, kp_hi = min(KP, kp_lo + per);
+    unsigned char *stage = smem + wave * (2 * BUF);
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+
+    const unsigned char *aval = (const unsigned char *)P.fp_val + ((int64_t)mb * KP * 2) * 1024;
+    const unsigned char *aidx = (const unsigned char *)P.fp_idx + ((int64_t)mb * KP) * 256;
+    const uint32_t lane16 = lane * 16, lane4 = lane * 4;
+    // DMA source of lane l in load i: token row 4i + l/16 (clamped: surplus rows repeat the last
+    // token and are never stored), logical 16-byte piece (l%16) ^ row
+    uint32_t x_off[ND];
+#pragma unroll
+    for (int i = 0; i < ND; i++) {
+        const int row = 4 * i + (lane >> 4);
+        const int q = (lane & 15) ^ (row & 15);
+        const int64_t tok = row < P.T ? row : P.T - 1;
+        x_off[i] = (uint32_t)((tok * P.ldx + q * 8) * 2);
+    }
+    // fragment read offsets: lane (token j, half h), k pair kl, k-step ks, piece c
+    int b_off[2][2][2];
+#pragma unroll
+    for (int kl = 0; kl < 2; kl++)
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+            for (int c = 0; c < 2; c++)
+                b_off[kl][ks][c] = (j & 15) * 256 + (((kl * 8 + ks * 4 + 2 * h + c) ^ (j & 15)) << 4);
+
+    struct ASet {
+        u32x4 a[2][2];
+        uint32_t ix[2];
+    };
+    ASet as[2];
+    // Loads of the chunk that starts at k pair kp0 (clamped into the operand when it lies beyond
+    // the wavefront's range: the count of operations stays uniform, the data is zeroed later).
+    auto issue = [&](int kp0, unsigned char *buf, ASet &A) {
+        const int kpc = min(kp0, KP - 2 >= 0 ? KP - 2 : 0);
+        const unsigned char *xb = (const unsigned char *)P.x + (int64_t)kpc * 128;
+#pragma unroll
+        for (int i = 0; i < ND; i++)
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[i]), (lds_ptr_t)(buf + i * 1024), 16, 0, 0);
+#pragma unroll
+        for (int kl = 0; kl < 2; kl++) {
+            const int kp = min(kp0 + kl, KP - 1);
+            const unsigned char *av = aval + (int64_t)kp * 2048;
+            const unsigned char *ai = aidx + (int64_t)kp * 256;
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(A.a[kl][0]) : "v"(lane16), "s"(av) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(A.a[kl][1]) : "v"(lane16), "s"(av) : "memory");
+            asm volatile("global_load_dword %0, %1, %2" : "=v"(A.ix[kl]) : "v"(lane4), "s"(ai) : "memory");
+        }
+    };
+    auto consume = [&](int kp0, const unsigned char *buf, ASet &A) {
+        u32x4 b[2][2][2];
+#pragma unroll
+        for (int kl = 0; kl < 2; kl++)
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                for (int c = 0; c < 2; c++) b[kl][ks][c] = *(const u32x4 *)(buf + b_off[kl][ks][c]);
+#pragma unroll
+        for (int kl = 0; kl < 2; kl++) {
+            // k pairs beyond the wavefront's range (or, when K is not a multiple of 128, beyond the
+            // chunk's real extent) contribute nothing: their weights are replaced by zeros
+            const bool live = kp0 + kl < kp_hi;
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                union {
+                    u32x4 u4;
+                    typename S::A v;
+                } ca;
+                const u32x4 zero4 = {0, 0, 0, 0};
+                ca.u4 = live ? A.a[kl][ks] : zero4;
+                union {
+                    u32x4 u4[2];
+                    typename S::B v;
+                } cb;
+                cb.u4[0] = b[kl][ks][0];
+                cb.u4[1] = b[kl][ks][1];
+                if (ks == 0)
+                    acc = S::template run<0>(ca.v, cb.v, acc, (int)A.ix[kl]);
+                else
+                    acc = S::template run<1>(ca.v, cb.v, acc, (int)A.ix[kl]);
+            }
+        }
+    };
+
+    issue(kp_lo, stage, as[0]);
+    for (int kp0 = kp_lo; kp0 < kp_hi; kp0 += 4) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int kc = kp0 + 2 * u;
+            // (the other buffer was read out before the MFMAs of the previous chunk)
+            issue(kc + 2, stage + ((u + 1) & 1) * BUF, as[(u + 1) & 1]);
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(OPS) : "memory");   // chunk kc has landed
+            __builtin_amdgcn_sched_barrier(0);
+            consume(kc, stage + u * BUF, as[u]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();   // every wavefront is done with its staging area: reuse it for the reduction
+    float(*red)[32][17] = (float(*)[32][17])smem;
+    // D[row = line][col = token]: lane holds token j, lines 8*(r/4) + 4*h + r%4
+    if (j < 16) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) red[wave][(r >> 2) * 8 + h * 4 + (r & 3)][j] = acc[r];
+    }
+    __syncthreads();
+    for (int e = tid; e < 32 * 16; e += 64 * SK_NW) {
+        const int line = e & 31, tok = e >> 5;
+        const int64_t f = (int64_t)mb * 32 + line;
+        if (tok >= P.T || f >= P.M) continue;
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < SK_NW; w++) s += red[w][line][tok];
+        if (P.bias) s += to_f32(((const T *)P.bias)[f]);
+        ((uint16_t *)P.y)[tok * P.ldy + f] = f32_to_bits16(s, (T *)nullptr);
+    }
+}
+
+template <typename T, int NW, int ND> static int launch_smfmac_decode_staged(SmfParams &P, hipStream_t s)
+{
+    dim3 grid((unsigned)((P.M + 31) / 32));
+    const size_t lds = (size_t)NW * 2 * 16 * 256;
+    auto k = spmm_smfmac_decode_staged_kernel<T, NW, ND>;
+    if (lds > 64 * 1024)
+        NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(k, grid, dim3(64 * NW), lds, s, P);
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
+template <typename T, int NW> static int launch_smfmac_decode_staged_nd(SmfParams &P, hipStream_t s)
+{
+    switch ((int)(P.T + 3) / 4) {
+    case 1: return launch_smfmac_decode_staged<T, NW, 1>(P, s);
+    case 2: return launch_smfmac_decode_staged<T, NW, 2>(P, s);
+    case 3: return launch_smfmac_decode_staged<T, NW, 3>(P, s);
+    default: return launch_smfmac_decode_staged<T, NW, 4>(P, s);
+    }
+}
+
 // ------------------------------------------------------------------------------ fragpack
 struct FragpackParams {
     const void *pk_val;   // rowpack values [G, nb, n]
@@ -1054,6 +1225,11 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
         if (P.T > 16) return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
         // few line blocks: many wavefronts per workgroup keep enough loads in flight per CU;
         // many line blocks: small workgroups pack several per CU and balance better
+        // reduction extents that are a multiple of 128: activations staged through LDS
+        if (P.K % 128 == 0 && P.T * P.ldx * 2 < ((int64_t)1 << 31)) {
+            if ((P.M + 31) / 32 >= 256) return launch_smfmac_decode_staged_nd<T, 4>(P, s);
+            return launch_smfmac_decode_staged_nd<T, 16>(P, s);
+        }
         if ((P.M + 31) / 32 >= 256) return launch_smfmac_skinny<T, 4, 4>(P, s);
         return launch_smfmac_skinny<T, 16, 1>(P, s);
     case 4:                                                     // 256 x 128, LDS-DMA ring

@@ -421,3 +421,24 @@ def test_cached_dense_operand_follows_weight_updates():
     w.mul_(2.0)                                                     # in-place update invalidates it
     y2 = sten.spmm(w, x, reduce_dim=1)
     assert rel_l2(to_np(y2), 2.0 * to_np(y1).astype(np.float64)) <= 1e-3
+
+
+@pytest.mark.parametrize("T", [1, 2, 5, 7, 8, 9, 12, 13, 16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,K,n,m,g", [
+    (515, 1024, 2, 4, 16),     # ragged lines, 16 wavefronts per line block
+    (96, 128, 2, 4, 16),       # one chunk of 128 positions: most wavefronts have nothing to do
+    (200, 2432, 1, 4, 8),      # k pairs not a multiple of the wavefront count
+    (64, 192, 2, 4, 16),       # K % 128 != 0: the staging kernel steps aside
+    (8224, 256, 2, 8, 4),      # >= 256 line blocks: 4 wavefronts per workgroup
+])
+def test_decode_kernels_all_token_counts(T, dtype, M, K, n, m, g):
+    print(f"case decode {dtype} M={M} K={K} T={T} {n}:{m}:{g}", flush=True)
+    W = seeded((M, K), dtype, seed=M + K + T, std=0.05)
+    Wd, _ = dense_ref(W, n, m, g, 1)
+    w = make(W, n, m, g, 1)
+    x = seeded((T, K), dtype, seed=6)
+    b = seeded((M,), dtype, seed=7)
+    ref = to_np(x).astype(np.float64) @ Wd.T + to_np(b).astype(np.float64)
+    y = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)
+    assert rel_l2(to_np(y), ref) <= TOL[dtype]
