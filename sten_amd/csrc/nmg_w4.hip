@@ -278,6 +278,148 @@ __global__ __launch_bounds__(64 * NW) void w4_linear_kernel(W4Params P)
     }
 }
 
+// The same product with the activations staged through LDS: a wavefront's direct activation loads
+// touch 32 bytes of a token row per instruction; here the next group's 16 token rows x 256 bytes
+// arrive by row-contiguous DMA loads into a staging area private to the wavefront (no barrier),
+// issued before the group's weight loads so that one counted wait covers both.  One group is in
+// flight while the previous one is multiplied; 16-byte pieces of a row are XOR-swizzled with the
+// row number so that a fragment read hits distinct banks.
+template <int NW, int ND>
+__global__ __launch_bounds__(64 * NW) void w4_linear_staged_kernel(W4Params P)
+{
+    constexpr int OPS = ND + 3;
+    constexpr int BUF = 16 * 256;
+    extern __shared__ __align__(16) unsigned char w4_smem[];
+    static_assert(NW * 2 * BUF >= NW * 32 * 17 * 4, "the reduction buffer reuses the staging area");
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int mb = blockIdx.x;
+    const int KQ = P.KQ;
+    const int j = lane & 31, h = lane >> 5;
+    const int per = (KQ + NW - 1) / NW;
+    const int kq_lo = wave * per, kq_hi = min(KQ, kq_lo + per);
+    unsigned char *stage = w4_smem + wave * (2 * BUF);
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+
+    const unsigned char *bv = (const unsigned char *)P.B + ((int64_t)mb * KQ) * 1024;
+    const unsigned char *mv = (const unsigned char *)P.meta + ((int64_t)mb * KQ) * 512;
+    const unsigned char *sv = (const unsigned char *)P.s + ((int64_t)mb * KQ) * 64;
+    const uint32_t lane16 = lane * 16, lane8 = lane * 8, row2 = j * 2;
+    uint32_t x_off[ND];
+#pragma unroll
+    for (int i = 0; i < ND; i++) {
+        const int row = 4 * i + (lane >> 4);
+        const int q = (lane & 15) ^ (row & 15);
+        const int64_t tok = row < P.T ? row : P.T - 1;   // surplus rows repeat the last token, never stored
+        x_off[i] = (uint32_t)((tok * P.ldx + q * 8) * 2);
+    }
+    int b_off[4][2];
+#pragma unroll
+    for (int ins = 0; ins < 4; ins++)
+#pragma unroll
+        for (int c = 0; c < 2; c++) b_off[ins][c] = (j & 15) * 256 + (((ins * 4 + 2 * h + c) ^ (j & 15)) << 4);
+
+    struct WSet {
+        u32x4 a;
+        uint2 ix;
+        uint32_t s;
+    };
+    WSet ws[2];
+    auto issue = [&](int kq, unsigned char *buf, WSet &W) {
+        const int kc = min(kq, KQ - 1);       // beyond the range: same count of operations, data unused
+        const unsigned char *xb = (const unsigned char *)P.x + (int64_t)kc * 256;
+#pragma unroll
+        for (int i = 0; i < ND; i++)
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[i]), (lds_ptr_t)(buf + i * 1024), 16, 0, 0);
+        const unsigned char *pb = bv + (int64_t)kc * 1024, *pm = mv + (int64_t)kc * 512, *ps = sv + (int64_t)kc * 64;
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(W.a) : "v"(lane16), "s"(pb) : "memory");
+        asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(W.ix) : "v"(lane8), "s"(pm) : "memory");
+        asm volatile("global_load_ushort %0, %1, %2" : "=v"(W.s) : "v"(row2), "s"(ps) : "memory");
+    };
+    auto consume = [&](int kq, const unsigned char *buf, const WSet &W) {
+        u32x4 b[4][2];
+#pragma unroll
+        for (int ins = 0; ins < 4; ins++)
+#pragma unroll
+            for (int c = 0; c < 2; c++) b[ins][c] = *(const u32x4 *)(buf + b_off[ins][c]);
+        const bool live = kq < kq_hi;
+        union {
+            uint16_t u;
+            _Float16 f;
+        } sc;
+        sc.u = live ? (uint16_t)W.s : (uint16_t)0;      // scale 0 silences a group beyond the range
+        const w4_f16x2 s2 = {sc.f, sc.f};
+        const uint32_t words[4] = {W.a.x, W.a.y, W.a.z, W.a.w};
+#pragma unroll
+        for (int ins = 0; ins < 4; ins++) {
+            union {
+                u32x4 u4;
+                w4_f16x8 v;
+            } ca;
+            ca.u4 = w4_dequant(words[ins], s2);
+            union {
+                u32x4 u4[2];
+                w4_f16x16 v;
+            } cb;
+            cb.u4[0] = b[ins][0];
+            cb.u4[1] = b[ins][1];
+            const int ix = (int)(ins < 2 ? W.ix.x : W.ix.y);
+            if (ins & 1)
+                acc = __builtin_amdgcn_smfmac_f32_32x32x32_f16(ca.v, cb.v, acc, ix, 0, 1);
+            else
+                acc = __builtin_amdgcn_smfmac_f32_32x32x32_f16(ca.v, cb.v, acc, ix, 0, 0);
+        }
+    };
+
+    issue(kq_lo, stage, ws[0]);
+    for (int kq0 = kq_lo; kq0 < kq_hi; kq0 += 2) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int kq = kq0 + u;
+            issue(kq + 1, stage + ((u + 1) & 1) * BUF, ws[(u + 1) & 1]);
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(OPS) : "memory");   // group kq has landed
+            __builtin_amdgcn_sched_barrier(0);
+            consume(kq, stage + u * BUF, ws[u]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    float(*red)[32][17] = (float(*)[32][17])w4_smem;
+    if (j < 16) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) red[wave][(r >> 2) * 8 + h * 4 + (r & 3)][j] = acc[r];
+    }
+    __syncthreads();
+    for (int e = tid; e < 32 * 16; e += 64 * NW) {
+        const int line = e & 31, tok = e >> 5;
+        const int64_t f = (int64_t)mb * 32 + line;
+        if (tok >= P.T || f >= P.M) continue;
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; w++) s += red[w][line][tok];
+        if (P.bias) s += __half2float(((const __half *)P.bias)[f]);
+        ((__half *)P.y)[tok * P.ldy + f] = __float2half(s);
+    }
+}
+
+template <int NW, int ND> static void w4_launch_staged(const W4Params &P, hipStream_t s)
+{
+    hipLaunchKernelGGL((w4_linear_staged_kernel<NW, ND>), dim3((unsigned)P.MB), dim3(64 * NW), (size_t)NW * 2 * 16 * 256, s, P);
+}
+template <int NW> static void w4_launch_staged_nd(const W4Params &P, hipStream_t s)
+{
+    switch ((int)(P.T + 3) / 4) {
+    case 1: w4_launch_staged<NW, 1>(P, s); break;
+    case 2: w4_launch_staged<NW, 2>(P, s); break;
+    case 3: w4_launch_staged<NW, 3>(P, s); break;
+    default: w4_launch_staged<NW, 4>(P, s); break;
+    }
+}
+
 template <int NW, int NB, int RB> static void w4_launch(const W4Params &P, hipStream_t s)
 {
     hipLaunchKernelGGL((w4_linear_kernel<NW, NB, RB>), dim3((unsigned)((P.MB + RB - 1) / RB)), dim3(64 * NW), 0, s, P);
@@ -380,10 +522,17 @@ extern "C" int nmg_w4_linear(const void *d_B, const void *d_meta, const void *d_
     P.MB = (int)((M + 31) / 32);
     P.KQ = (int)(K / 128);
     hipStream_t s = (hipStream_t)stream;
-    // One block of 32 rows per workgroup and one group in flight per wavefront measured best on
-    // the 11008 x 4096 weight (8.9 us at 1 token; two row blocks per workgroup: 19 us -- the
-    // kernel lives on the number of workgroups pulling data at once, not on bytes per request).
-    if (P.KQ >= 16)
+    // One block of 32 rows per workgroup measured best on the 11008 x 4096 weight (two row blocks
+    // per workgroup sharing the activation fragments: 19 us against 8.9 -- the kernel lives on the
+    // number of workgroups pulling data at once).  Staged activations and counted waits: 6.6 us at
+    // one token, 7.8 us at 16 (direct loads: 8.8 / 13.2); the direct kernel remains for K = 0 and
+    // activations beyond 2 GiB.
+    if (P.KQ >= 1 && P.T * P.ldx * 2 < ((int64_t)1 << 31)) {
+        if (P.KQ >= 16)
+            w4_launch_staged_nd<8>(P, s);
+        else
+            w4_launch_staged_nd<4>(P, s);
+    } else if (P.KQ >= 16)
         w4_launch<8, 1, 1>(P, s);
     else
         w4_launch<4, 1, 1>(P, s);
