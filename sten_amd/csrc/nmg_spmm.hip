@@ -310,7 +310,7 @@ extern "C" int nmg_spmm(const void *d_pk_val, const void *d_pk_pat, int64_t G, i
     // tiled kernel below keeps serving f32, ragged K, unusual n:m and explicit requests.
     if (kernel == NMG_KERNEL_MFMA && (dtype == NMG_F16 || dtype == NMG_BF16) && T > 16 &&
         dense_pipe_supports(n, m) && P.K % 64 == 0 && P.K >= 64 && (ldx % 8) == 0 && ((uintptr_t)d_x % 16) == 0 &&
-        T * ldx * 2 < ((int64_t)1 << 31) && binom(m, n) <= 256 && !getenv("NMG_SIMPLE_MFMA"))
+        T * ldx * 2 < ((int64_t)1 << 31) && binom(m, n) <= 256)
         return spmm_dense_pipe(d_pk_val, d_pk_pat, P.order, G, S, d_x, ldx, d_y, ldy, d_bias, T,
                                reduce_sparse, n, m, dtype, s);
     switch (dtype) {
