@@ -14,6 +14,7 @@ from .dispatch import (DISPATCH_RAISE, DISPATCH_WARN, DenseTensor, DispatchError
 from .impls import GroupedNMSparsifier, install
 from .layout import NMGLayout
 from .native import NmgError
+from .perfect import PerfectNMTensor, is_correct_nm
 from .tensor import GroupedNMTensor, spmm
 from . import w4
 from .w4 import SparseMarlinSparsifier, SparseMarlinTensor

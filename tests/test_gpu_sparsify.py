@@ -131,3 +131,23 @@ def test_full_size_properties_config2():
     val, idx_o, _ = oracle_sparsify(w[:192], 2, 4, 1, 16, 0)            # first two 96-row chunks
     k = val.shape[0]
     assert np.array_equal(to_np(t.idx[:k]), idx_o) and same_bits(t.val[:k], val)
+
+
+def test_preserved_magnitude_between_random_and_perfect():
+    # tests/test_nmg.py:33-86: shapes (3, a, b) with a, b in {17, 5, 1} in every axis order, 5:12:2;
+    # the grouped tensor is a valid n:m tensor, beats n/m of the magnitude and stays below the
+    # ungrouped ("perfect") n:m tensor
+    torch.manual_seed(123)
+    n, m, g = 5, 12, 2
+    for a, b in itertools.permutations([17, 5, 1], 2):
+        for sparse_dim, group_dim in itertools.permutations(range(3), 2):
+            x = torch.rand(3, a, b, device=DEV)
+            t = sten.GroupedNMTensor.from_dense(x, n, m, sparse_dim=sparse_dim, group_size=g, group_dim=group_dim)
+            d = t.to_dense()
+            assert sten.is_correct_nm(x, d, sparse_dim, n, m)
+            kept = float(d.abs().sum() / x.abs().sum())
+            assert kept > n / m or x.shape[sparse_dim] < m
+            p = sten.PerfectNMTensor.from_dense(x, n=n, m=m, sparse_dim=sparse_dim)
+            pd = p.to_dense()
+            assert pd.shape == x.shape and sten.is_correct_nm(x, pd, sparse_dim, n, m)
+            assert float(pd.abs().sum() / x.abs().sum()) >= kept - 1e-5
