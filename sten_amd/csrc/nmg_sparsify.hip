@@ -18,6 +18,8 @@
 // contiguous one, so the cooperative tile load is coalesced across them.
 #include "nmg_common.h"
 
+#include <algorithm>
+
 namespace nmg {
 
 template <typename T> struct ScoreOf { using type = float; using bits = uint32_t; };
@@ -777,6 +779,127 @@ extern "C" int nmg_sparsify(const void *d_dense, const nmg_view *view, void *d_v
 
 template <template <typename> class K> struct Launch;
 
+// Tiled forms of the two kernels above for views whose sparse dim is contiguous (the layout of
+// a weight with n:m blocks along its rows' direction).  There a tile is c*g lines x m positions:
+// one slot's m values are a few bytes of a line, so the slot-per-thread kernels touch every cache
+// line of the dense tensor many times.  Here a workgroup takes NT tiles that are neighbours along
+// the sparse dim -- a region of c*g lines x NT*m contiguous positions -- and moves it through
+// LDS: rows of the region go to / come from global memory as contiguous segments, val / idx are
+// contiguous for the NT tiles anyway.
+struct TiledParams {
+    ScatterParams sp;
+    int nt;                      // tiles per workgroup
+    int pitch;                   // elements per region row in LDS
+    int groups_per_chunk;        // workgroups along the sparse dim
+    uint64_t magic_cols, magic_g;
+};
+
+template <typename T, bool GATHER>
+__global__ __launch_bounds__(256) void scatter_tiled_kernel(TiledParams Q)
+{
+    const ScatterParams &P = Q.sp;
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *tile = (T *)smem;
+    const int tid = threadIdx.x;
+    const int n = P.n, m = P.m, cols = P.cols, nt = Q.nt, pitch = Q.pitch;
+    // workgroup -> (batch, group-dim chunk, first block)
+    const int64_t wg = blockIdx.x;
+    const int64_t chunk_id = wg / Q.groups_per_chunk;
+    const int64_t mb0 = (wg - chunk_id * Q.groups_per_chunk) * nt;
+    const int64_t b = chunk_id / P.view.num_chunks, kc = chunk_id - b * P.view.num_chunks;
+    const int64_t t0 = (b * P.view.num_chunks + kc) * P.view.num_blocks + mb0;
+    const int tiles = (int)min((int64_t)nt, P.view.num_blocks - mb0);
+    const int64_t g0 = kc * cols, s0 = mb0 * m;
+    const int width = tiles * m;                       // positions of the region
+    const int rows = (int)min((int64_t)cols, P.view.G - g0);
+    const int valid_w = (int)max((int64_t)0, min((int64_t)width, P.view.S - s0));
+    T *dense = (T *)P.dense + b * P.view.stride_b + g0 * P.view.stride_g + s0;
+    constexpr int V = 16 / sizeof(T);
+    const bool vec = (P.view.stride_g % V) == 0 && (s0 % V) == 0 && (P.view.stride_b % V) == 0 &&
+                     ((uintptr_t)P.dense % 16) == 0 && (pitch % V) == 0;
+    const int wv = (width + V - 1) / V;
+
+    if (GATHER) {
+        // region -> LDS (zeros beyond G / S)
+        for (int i = tid; i < cols * wv; i += 256) {
+            const int r = i / wv, cc = (i - r * wv) * V;
+            T *dst = tile + r * pitch + cc;
+            const T *src = dense + (int64_t)r * P.view.stride_g + cc;
+            if (vec && r < rows && cc + V <= valid_w) {
+                *(uint4 *)dst = *(const uint4 *)src;
+            } else {
+                for (int e = 0; e < V && cc + e < pitch; e++)
+                    dst[e] = (r < rows && cc + e < valid_w) ? src[e] : Zero<T>::v();
+            }
+        }
+    } else {
+        const uint4 z = {0, 0, 0, 0};
+        for (int i = tid; i < cols * pitch * (int)sizeof(T) / 16; i += 256) ((uint4 *)tile)[i] = z;
+    }
+    __syncthreads();
+    // slots of the NT tiles: contiguous in val / idx
+    for (int e = tid; e < tiles * cols; e += 256) {
+        const int tm = (int)(((uint64_t)e * Q.magic_cols) >> 32), slot = e - tm * cols;
+        const int p = (int)(((uint64_t)slot * Q.magic_g) >> 32);
+        const int64_t at = (t0 + tm) * (int64_t)cols + slot;
+        const int o = P.idx[at];
+        T *v = (T *)P.val + at * n;
+        if (GATHER) {
+            for (int j = 0; j < n; j++)
+                v[j] = (o >= 0 && o < cols) ? tile[o * pitch + tm * m + P.order[p * n + j]] : Zero<T>::v();
+        } else if (o >= 0 && o < cols) {
+            for (int j = 0; j < n; j++) tile[o * pitch + tm * m + P.order[p * n + j]] = v[j];
+        }
+    }
+    if (GATHER) return;
+    __syncthreads();
+    // LDS -> region
+    for (int i = tid; i < rows * wv; i += 256) {
+        const int r = i / wv, cc = (i - r * wv) * V;
+        if (cc >= valid_w) continue;
+        const T *src = tile + r * pitch + cc;
+        T *dst = dense + (int64_t)r * P.view.stride_g + cc;
+        if (vec && cc + V <= valid_w) {
+            *(uint4 *)dst = *(const uint4 *)src;
+        } else {
+            for (int e = 0; e < V && cc + e < valid_w; e++) dst[e] = src[e];
+        }
+    }
+}
+
+// Launches the tiled kernel when it applies; *done tells whether it did.
+template <typename T>
+static int launch_scatter_tiled(bool gather, ScatterParams &P, hipStream_t s, bool *done)
+{
+    *done = false;
+    if (P.view.stride_s != 1 || P.view.num_blocks < 8) return NMG_OK;
+    // as many tiles per workgroup as 64 KiB of LDS hold, at most 64, at least 8
+    const int64_t per_tile = (int64_t)P.cols * P.m * (int64_t)sizeof(T);
+    int nt = (int)std::min<int64_t>(64, (60 * 1024) / per_tile);
+    if (nt < 8) return NMG_OK;
+    nt = (int)std::min<int64_t>(nt, P.view.num_blocks);
+    TiledParams Q{};
+    Q.sp = P;
+    Q.nt = nt;
+    const int V = 16 / (int)sizeof(T);
+    Q.pitch = ((nt * P.m + V - 1) / V) * V + V;         // 16-byte rows, one vector of padding
+    Q.groups_per_chunk = (int)((P.view.num_blocks + nt - 1) / nt);
+    Q.magic_cols = (((uint64_t)1 << 32) + P.cols - 1) / P.cols;
+    Q.magic_g = (((uint64_t)1 << 32) + P.g - 1) / P.g;
+    const size_t lds = (size_t)P.cols * Q.pitch * sizeof(T);
+    if (lds > 160 * 1024 || (int64_t)nt * P.cols >= 65536) return NMG_OK;
+    const int64_t chunks = P.outer / P.view.num_blocks;   // batches x group-dim chunks
+    const int64_t grid = chunks * Q.groups_per_chunk;
+    if (grid > 0x7fffffffLL) return NMG_OK;
+    auto kern = gather ? scatter_tiled_kernel<T, true> : scatter_tiled_kernel<T, false>;
+    if (lds > 64 * 1024)
+        NMG_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, s, Q);
+    NMG_HIP_TRY(hipGetLastError());
+    *done = true;
+    return NMG_OK;
+}
+
 static int launch_scatter(bool gather, const void *dense, const nmg_view *view, const void *val,
                           const int16_t *idx, int n, int m, int g, int dtype, void *stream)
 {
@@ -801,6 +924,17 @@ static int launch_scatter(bool gather, const void *dense, const nmg_view *view, 
     const int64_t grid = (total + bs - 1) / bs;
     NMG_REQUIRE(grid <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "too many slots");
     hipStream_t s = (hipStream_t)stream;
+    {
+        bool done = false;
+        int rc = NMG_OK;
+        switch (dtype) {
+        case NMG_F32: rc = launch_scatter_tiled<float>(gather, P, s, &done); break;
+        case NMG_F16: rc = launch_scatter_tiled<__half>(gather, P, s, &done); break;
+        case NMG_BF16: rc = launch_scatter_tiled<__hip_bfloat16>(gather, P, s, &done); break;
+        case NMG_F64: rc = launch_scatter_tiled<double>(gather, P, s, &done); break;
+        }
+        if (rc != NMG_OK || done) return rc;
+    }
 #define NMG_LAUNCH(T)                                                                         \
     do {                                                                                      \
         if (gather)                                                                           \
