@@ -327,7 +327,7 @@ struct TeamParams {
     uint64_t magic_cols, magic_g;      // ceil(2^32 / cols), ceil(2^32 / g): x / d == (x * magic) >> 32 for x < 2^16
 };
 
-template <typename T, int L>
+template <typename T, int L, bool SMALLC>
 __global__ __launch_bounds__(128) void sparsify_teams_kernel(TeamParams Q)
 {
     using CT = typename ScoreOf<T>::type;
@@ -394,6 +394,18 @@ __global__ __launch_bounds__(128) void sparsify_teams_kernel(TeamParams Q)
 
     const bool live = team < teams && tile0 + team < P.outer;
 
+    // SMALLC (at most 8 patterns, m <= 8, g <= 255): the pattern masks and the pattern counters
+    // (8 bits each, packed) stay in registers of every lane of the team -- all lanes see every
+    // accepted (column, pattern) -- so neither the staleness test nor a repair waits for LDS
+    // beyond the read of the column itself.
+    int mk_r[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    uint64_t cnt64 = 0;
+    if (SMALLC) {
+#pragma unroll
+        for (int p = 0; p < 8; p++) mk_r[p] = p < c ? (int)s_mask[p] : 0;
+    }
+    auto cnt_of = [&](int p) { return (int)((cnt64 >> (8 * p)) & 0xFF); };
+
     // Best key of column o over the patterns that still have room: score bits + 1 and pattern.
     // LDS reads are issued in batches of independent loads (the column first, then 8 patterns'
     // masks and counters at a time): the loop is latency-bound, not throughput-bound.
@@ -401,6 +413,27 @@ __global__ __launch_bounds__(128) void sparsify_teams_kernel(TeamParams Q)
         best_p = 0;
         best_s = 0;
         const T *col = s_d + o * m;
+        if (SMALLC) {
+            CT a[8];
+#pragma unroll
+            for (int r = 0; r < 8; r++) a[r] = score_of(col[r < m ? r : 0]);
+#pragma unroll
+            for (int p = 0; p < 8; p++) {
+                if (p >= c || cnt_of(p) >= g) continue;
+                CT acc = 0;
+#pragma unroll
+                for (int r = 0; r < 8; r++) {
+                    if (r >= m) break;
+                    if ((mk_r[p] >> r) & 1) acc += a[r];
+                }
+                const SB sb = score_bits(acc) + 1;
+                if (sb >= best_s) {
+                    best_s = sb;
+                    best_p = p;
+                }
+            }
+            return;
+        }
         if (m <= 8) {
             CT a[8];
 #pragma unroll
@@ -447,29 +480,38 @@ __global__ __launch_bounds__(128) void sparsify_teams_kernel(TeamParams Q)
     // A lane owns at most 32 columns (the launcher picks L accordingly), kept as 4 groups of 8
     // whose maxima live in registers: a change rescans one group only.
     SB gs[4] = {0, 0, 0, 0};
-    int go[4] = {0, 0, 0, 0};
+    int go[4] = {0, 0, 0, 0};   // column << 16 | pattern of the group's best head
     auto scan_group = [&](int k) {
         SB v[8];
+        int hp[8];
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             const int o = tl + L * (k * 8 + i);
             v[i] = s_hs[o < cols ? o : tl];
+            hp[i] = s_hp[o < cols ? o : tl];
         }
-        SB best_s = 0;
-        int best_o = 0;
+        // pairwise (tree) reduction; on equal scores the larger column, i.e. the later entry, wins
+        SB bs[8];
+        int bo[8];
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             const int o = tl + L * (k * 8 + i);
-            if (o < cols && v[i] != 0 && v[i] >= best_s) {
-                best_s = v[i];
-                best_o = o;
-            }
+            bs[i] = o < cols ? v[i] : 0;
+            bo[i] = (o << 16) | hp[i];
         }
+#pragma unroll
+        for (int w = 1; w < 8; w <<= 1)
+#pragma unroll
+            for (int i = 0; i < 8; i += 2 * w)
+                if (bs[i + w] >= bs[i] && bs[i + w] != 0) {
+                    bs[i] = bs[i + w];
+                    bo[i] = bo[i + w];
+                }
 #pragma unroll
         for (int q = 0; q < 4; q++)
             if (q == k) {
-                gs[q] = best_s;
-                go[q] = best_o;
+                gs[q] = bs[0];
+                go[q] = bo[0];
             }
     };
     auto local_best = [&]() {
@@ -477,17 +519,15 @@ __global__ __launch_bounds__(128) void sparsify_teams_kernel(TeamParams Q)
         lb.s = 0;
         lb.op = 0;
         SB best_s = 0;
-        int best_o = -1;
+        int best_op = 0;
 #pragma unroll
         for (int q = 0; q < 4; q++)
             if (gs[q] != 0 && gs[q] >= best_s) {
                 best_s = gs[q];
-                best_o = go[q];
+                best_op = go[q];
             }
-        if (best_o >= 0) {
-            lb.s = best_s;
-            lb.op = ((uint32_t)best_o << 16) | s_hp[best_o];
-        }
+        lb.s = best_s;
+        lb.op = best_s != 0 ? (uint32_t)best_op : 0u;
         return lb;
     };
 
@@ -516,8 +556,9 @@ __global__ __launch_bounds__(128) void sparsify_teams_kernel(TeamParams Q)
             // ---- team arg-max ----
             const Key<SB> b = team_max<L>(lb);
             const int o_star = (int)(b.op >> 16), p_star = (int)(b.op & 0xFFFFu);
-            const int cntp = s_cnt[p_star];
+            const int cntp = SMALLC ? cnt_of(p_star) : (int)s_cnt[p_star];
             const bool stale = cntp >= g;
+            if (SMALLC && !stale) cnt64 += (uint64_t)1 << (8 * p_star);
             if (o_star % L == tl) {
                 if (stale) {
                     SB bs;
@@ -526,7 +567,7 @@ __global__ __launch_bounds__(128) void sparsify_teams_kernel(TeamParams Q)
                     s_hs[o_star] = bs;
                     s_hp[o_star] = (uint16_t)bp;
                 } else {
-                    s_cnt[p_star] = (int16_t)(cntp + 1);
+                    if (!SMALLC) s_cnt[p_star] = (int16_t)(cntp + 1);
                     s_hs[o_star] = 0;
                     s_oidx[p_star * g + cntp] = (int16_t)o_star;
                 }
@@ -592,7 +633,8 @@ template <typename T, int L> static int launch_sparsify_teams(SparsifyParams &P,
     Q.teams = threads / L;
     Q.magic_cols = (((uint64_t)1 << 32) + cols - 1) / cols;
     Q.magic_g = (((uint64_t)1 << 32) + P.g - 1) / P.g;
-    auto kern = sparsify_teams_kernel<T, L>;
+    const bool smallc = c <= 8 && m <= 8 && P.g <= 255;
+    auto kern = smallc ? sparsify_teams_kernel<T, L, true> : sparsify_teams_kernel<T, L, false>;
     if (lds > 64 * 1024)
         NMG_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                         (int)lds));
