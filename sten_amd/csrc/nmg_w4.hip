@@ -1,4 +1,4 @@
-// Decode-shape linear layer on a 2:4-pruned, int4-quantised weight (BASELINE's "sparse-marlin"
+// Decode-shape linear layer on a 2:4-pruned, int4-quantised weight (the benchmark's "sparse-marlin"
 // configuration: Llama-like MLP weight, 2:4 along K, symmetric int4 with one fp16 scale per 128
 // dense positions of a row, few tokens).  Memory-bound: 0.39 bytes per dense weight element are
 // streamed once, dequantised in registers and multiplied on the sparse matrix cores

@@ -1,4 +1,4 @@
-"""2:4-pruned, int4-quantised weight for decode-shape linear layers (BASELINE's "sparse-marlin"
+"""2:4-pruned, int4-quantised weight for decode-shape linear layers (the benchmark's "sparse-marlin"
 configuration).  Mirrors the custom format of the reference's test, which wraps an external
 library: ``SparseMarlinSparsifier`` / ``SparseMarlinTensor`` with fields ``B`` (packed values),
 ``s`` (scales) and ``meta`` (positions), registered for ``F.linear``
