@@ -43,6 +43,7 @@ WORKLOADS = {
     "c3_4_8": ("fwd", 8192, 8192, 4096, 4, 8, 32, "configs[2]: W 8192x8192 fp16 4:8:32 x 4096 tokens, forward"),
     "c5_fwd": ("fwd", 16384, 4096, 4096, 2, 4, 16, "configs[4]: W 16384x4096 fp16 2:4:16 x 4096 tokens, forward"),
     "c5_grad_x": ("grad_x", 16384, 4096, 4096, 2, 4, 16, "configs[4]: dY 4096x16384 x W 16384x4096 fp16 2:4:16, grad_input"),
+    "c5_step": ("step", 16384, 4096, 4096, 2, 4, 16, "configs[4]: training step of a sparse linear 4096 -> 16384, 4096 tokens: forward, grad_input, masked grad_weight in val layout"),
     "c2_grad_x": ("grad_x", 4096, 4096, 2048, 2, 4, 16, "configs[1] shape: dY 2048x4096 x W 4096x4096 fp16 2:4:16, grad_input"),
     "decode_1": ("decode", 4096, 11008, 1, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 1 token"),
     "decode_4": ("decode", 4096, 11008, 4, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 4 tokens"),
@@ -135,7 +136,26 @@ def main():
     torch.manual_seed(0)
     W = (torch.randn(M, K) * 0.02).half().to(dev)
 
-    if kind == "w4":
+    if kind == "step":
+        # the registered F.linear through the dispatch layer, compressed weight gradient
+        lin = torch.nn.Linear(K, M, bias=False).half().to(dev)
+        with torch.no_grad():
+            lin.weight.copy_(W)
+        del W
+        sb = sten.SparsityBuilder()
+        sb.set_weight("weight", initial_sparsifier=sten.GroupedNMSparsifier(n, m, g, sparse_dim=1, group_dim=0),
+                      out_format=sten.GroupedNMTensor)
+        sb.set_weight_grad("weight", tmp_format=sten.GroupedNMTensor, out_format=sten.GroupedNMTensor)
+        slin = sb.get_sparse_model(lin)
+        X = torch.randn(N, K, dtype=torch.float16, device=dev, requires_grad=True)
+        dY = torch.randn(N, M, dtype=torch.float16, device=dev)
+
+        def step():
+            slin.weight.grad = None
+            X.grad = None
+            slin(X).backward(dY)
+        algo_bytes = 0
+    elif kind == "w4":
         w = sten.SparseMarlinTensor.from_dense(W)
         del W
         X = torch.randn(N, K).half().to(dev)
@@ -191,8 +211,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
     }
-    if kind in ("fwd", "grad_x"):
-        dense_flops = 2.0 * M * K * N
+    if kind in ("fwd", "grad_x", "step"):
+        dense_flops = 2.0 * M * K * N * (3 if kind == "step" else 1)
         eff_flops = dense_flops * n / m
         achieved = eff_flops / (kern_ms * 1e-3) / 1e12
         out.update({
