@@ -190,6 +190,29 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
             __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[i]),
                                              (lds_ptr_t)(base + (wave * XL + i) * 1024), 16, 0, 0);
     };
+    // load number i (0 .. OPS-1) of K step kp: first the XL activation DMA loads, then the
+    // 4 * FB weight fragments
+    auto issue_one = [&](int kp, WSet &w, int i) {
+        if (kp >= KP) kp = KP - 1;
+        if (i < XL) {
+            unsigned char *base = smem + (kp & (DD_NS - 1)) * STAGE;
+            const unsigned char *xb = x_base + (int64_t)kp * 128;
+#pragma unroll
+            for (int q = 0; q < XL; q++)
+                if (q == i)
+                    __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[q]),
+                                                     (lds_ptr_t)(base + (wave * XL + q) * 1024), 16, 0, 0);
+        } else {
+#pragma unroll
+            for (int fb = 0; fb < FB; fb++)
+#pragma unroll
+                for (int k16 = 0; k16 < 4; k16++)
+                    if (XL + fb * 4 + k16 == i) {
+                        const unsigned char *av = av_base[fb] + (int64_t)kp * 4096 + k16 * 1024;
+                        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(w.a[fb][k16]) : "v"(lane16), "s"(av) : "memory");
+                    }
+        }
+    };
     auto issue_a = [&](int kp, WSet &w) {
         if (kp >= KP) kp = KP - 1;
 #pragma unroll
@@ -289,6 +312,10 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
                 mma(ws[u], fr[PH % 2], ph_tag, 0, 2);
                 __builtin_amdgcn_sched_barrier(0);
                 if (PH == NP - 1) {
+#pragma unroll
+                    for (int i = 0; i < OPS / NP; i++)
+                        issue_one(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)], PH * (OPS / NP) + i);
+                    __builtin_amdgcn_sched_barrier(0);
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // fragments of step kp are in registers
                     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DD_D - 1) * OPS) : "memory");  // my share of kp+1 landed
                     asm volatile("s_barrier" ::: "memory");              // ... and everybody else's
@@ -297,9 +324,24 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
                 } else {
                     read_b(fr[(PH + 1) % 2], base, PH + 1);
                 }
-                if (PH == 0) issue_x(kp + DD_D);
-                if (PH == 1) issue_a(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)]);
-                mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
+                // The step's OPS loads are dealt out evenly over its phases, one at a time between
+                // MFMAs: a burst would find the CU's vector memory path busy (16 clocks per 1 KiB
+                // instruction, shared by the four wavefronts) and stall with its MFMAs unissued.
+                // (In the last phase the loads come before the counted wait, which assumes them.)
+                constexpr int LPP = OPS / NP;               // loads per phase
+                static_assert(OPS % NP == 0 && LPP <= NM - 2, "loads spread evenly over the phases");
+                if (PH != NP - 1) {
+#pragma unroll
+                    for (int i = 0; i < LPP; i++) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        issue_one(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)], PH * LPP + i);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma(ws[u], fr[PH % 2], ph_tag, 2 + i, 3 + i);
+                    }
+                    mma(ws[u], fr[PH % 2], ph_tag, 2 + LPP, NM);
+                } else {
+                    mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             };
             phase(std::integral_constant<int, 0>{});
