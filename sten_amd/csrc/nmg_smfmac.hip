@@ -573,32 +573,42 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
         uint32_t ix[FB];
     };
     WSet ws[DR_D + 1];
-    // Steps beyond the last repeat it: the operation count stays uniform, the data is unused.
-    auto issue_x = [&](int kp) {
+    // Load number i (0 .. OPS-1) of K step kp: first the XL activation DMA loads, then per
+    // feature block two weight fragments and the index word.  Steps beyond the last repeat it:
+    // the operation count stays uniform, the data is unused.
+    auto issue_one = [&](int kp, WSet &w, int i) {
         if (kp >= KP) kp = KP - 1;
-        unsigned char *base = smem + (kp & (DR_NS - 1)) * STAGE;
-        const unsigned char *xb = x_base + (int64_t)kp * 128;
+        if (i < XL) {
+            unsigned char *base = smem + (kp & (DR_NS - 1)) * STAGE;
+            const unsigned char *xb = x_base + (int64_t)kp * 128;
 #pragma unroll
-        for (int i = 0; i < XL; i++)
-            __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[i]),
-                                             (lds_ptr_t)(base + (wave * XL + i) * 1024), 16, 0, 0);
-    };
-    auto issue_a = [&](int kp, WSet &w) {
-        if (kp >= KP) kp = KP - 1;
-#pragma unroll
-        for (int fb = 0; fb < FB; fb++) {
+            for (int q = 0; q < XL; q++)
+                if (q == i)
+                    __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[q]),
+                                                     (lds_ptr_t)(base + (wave * XL + q) * 1024), 16, 0, 0);
+        } else {
             // Written as instructions so that their completion is tracked by the explicit vmcnt
             // waits below and by nothing else (left to itself the compiler waits for vmcnt(0) at
             // the loop head, which empties the pipeline every K step), and with accumulation
             // registers as targets: the ring does not fit beside the accumulators in the 256
             // architectural registers, and a compiler-made copy of a register whose load is
             // still in flight would copy stale data.
-            const unsigned char *av = av_base[fb] + (int64_t)kp * 2048;
-            const unsigned char *ai = ai_base[fb] + (int64_t)kp * 256;
-            asm volatile("global_load_dwordx4 %0, %1, %2" : "=a"(w.a[fb][0]) : "v"(lane16), "s"(av) : "memory");
-            asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=a"(w.a[fb][1]) : "v"(lane16), "s"(av) : "memory");
-            asm volatile("global_load_dword %0, %1, %2" : "=v"(w.ix[fb]) : "v"(lane4), "s"(ai) : "memory");
+#pragma unroll
+            for (int fb = 0; fb < FB; fb++) {
+                const unsigned char *av = av_base[fb] + (int64_t)kp * 2048;
+                const unsigned char *ai = ai_base[fb] + (int64_t)kp * 256;
+                if (XL + fb * 3 == i)
+                    asm volatile("global_load_dwordx4 %0, %1, %2" : "=a"(w.a[fb][0]) : "v"(lane16), "s"(av) : "memory");
+                if (XL + fb * 3 + 1 == i)
+                    asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=a"(w.a[fb][1]) : "v"(lane16), "s"(av) : "memory");
+                if (XL + fb * 3 + 2 == i)
+                    asm volatile("global_load_dword %0, %1, %2" : "=v"(w.ix[fb]) : "v"(lane4), "s"(ai) : "memory");
+            }
         }
+    };
+    auto issue_step = [&](int kp, WSet &w) {
+#pragma unroll
+        for (int i = 0; i < OPS; i++) issue_one(kp, w, i);
     };
 
     f32x16 acc[FB][TB];
@@ -668,8 +678,7 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
     // prologue: steps 0 .. DR_D-1 in flight, then wait for step 0
 #pragma unroll
     for (int st = 0; st < DR_D; st++) {
-        issue_x(st);
-        issue_a(st, ws[st]);
+        issue_step(st, ws[st]);
     }
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DR_D - 1) * OPS) : "memory");
     asm volatile("s_barrier" ::: "memory");
@@ -683,7 +692,7 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
             const unsigned char *base = smem + (kp & (DR_NS - 1)) * STAGE;
             const unsigned char *next = smem + ((kp + 1) & (DR_NS - 1)) * STAGE;
             // One phase: two MFMAs; the LDS reads of the next phase into the other fragment set;
-            // in the first phases the loads of step kp+DR_D; the rest of the MFMAs.  Before the
+            // its share of the loads of step kp+DR_D between the rest of the MFMAs.  Before the
             // reads of the last phase, which fetch from the next stage, the barrier.  The
             // instruction statements fence the scheduler, so this is also the issue order.
             auto phase = [&](auto ph_tag) {
@@ -691,6 +700,10 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
                 mma(ws[u], fr[PH % 2], ph_tag, 0, 2);
                 __builtin_amdgcn_sched_barrier(0);
                 if (PH == NP - 1) {
+#pragma unroll
+                    for (int i = PH * OPS / NP; i < OPS; i++)
+                        issue_one(kp + DR_D, ws[(u + DR_D) % (DR_D + 1)], i);
+                    __builtin_amdgcn_sched_barrier(0);
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // fragments of step kp are in registers
                     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DR_D - 1) * OPS) : "memory");  // my share of kp+1 landed
                     asm volatile("s_barrier" ::: "memory");              // ... and everybody else's
@@ -699,18 +712,21 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
                 } else {
                     read_b(fr[(PH + 1) % 2], base, PH + 1);
                 }
-                if (PH == 0) {
-                    issue_x(kp + DR_D);
-                    if (NP == 2) {
-                        mma(ws[u], fr[PH % 2], ph_tag, 2, 4);
-                        issue_a(kp + DR_D, ws[(u + DR_D) % (DR_D + 1)]);
-                        mma(ws[u], fr[PH % 2], ph_tag, 4, NM);
-                    } else {
-                        mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
+                // The step's OPS loads are dealt out over its phases, one at a time between MFMAs
+                // (a burst finds the CU's vector memory path busy and stalls with its MFMAs
+                // unissued: 5 % on the 256 x 128 tile); in the last phase they come before the
+                // counted wait, which assumes them.
+                constexpr int L0 = PH * OPS / NP, L1 = (PH + 1) * OPS / NP;
+                static_assert(L1 - L0 <= NM - 2, "more loads than MFMAs to put them between");
+                if (PH != NP - 1) {
+#pragma unroll
+                    for (int i = L0; i < L1; i++) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        issue_one(kp + DR_D, ws[(u + DR_D) % (DR_D + 1)], i);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma(ws[u], fr[PH % 2], ph_tag, 2 + i - L0, 3 + i - L0);
                     }
-                } else if (PH == 1 && NP > 2) {
-                    issue_a(kp + DR_D, ws[(u + DR_D) % (DR_D + 1)]);
-                    mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
+                    mma(ws[u], fr[PH % 2], ph_tag, 2 + L1 - L0, NM);
                 } else {
                     mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
 #pragma unroll
@@ -1237,11 +1253,9 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
             return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
         return launch_smfmac_pipe<T>(P, s);
     case 6:                                                     // 256 x 128, weights straight to registers
-    case 7:                                                     // same, wavefronts 2 x 2 (shared weight fetches)
     case 8:                                                     // 256 x 256
         if (P.K % 64 != 0 || P.T * P.ldx * 2 >= (int64_t)1 << 31)
             return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
-        if (variant == 7) return launch_smfmac_direct<T, 4, 2, 2, 2, 1>(P, s);
         if (variant == 8) return launch_smfmac_direct<T, 2, 8, 4, 1, 2>(P, s);
         return launch_smfmac_direct<T, 2, 4, 4, 1, 1>(P, s);
     }
@@ -1255,7 +1269,7 @@ extern "C" int nmg_spmm_smfmac(const void *d_fp_val, const void *d_fp_idx, int64
     NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED,
                 "the sparse matrix cores take f16/bf16 only");
     NMG_REQUIRE(M >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
-    NMG_REQUIRE(variant >= -1 && variant <= 8, NMG_ERR_ARG, "unknown tile variant %d", variant);
+    NMG_REQUIRE(variant >= -1 && variant <= 8 && variant != 7, NMG_ERR_ARG, "unknown tile variant %d", variant);
     NMG_REQUIRE(ldx >= K && ldy >= M, NMG_ERR_ARG, "leading dimension smaller than row length");
     NMG_REQUIRE((K % 8) == 0 && (ldx % 8) == 0 && ((uintptr_t)d_x % 16) == 0, NMG_ERR_UNSUPPORTED,
                 "activations must be 16-byte aligned with K and ldx multiples of 8");
