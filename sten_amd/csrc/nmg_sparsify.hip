@@ -11,7 +11,9 @@
 // largest key among {(o, p): o free, p not full}.  Every free column keeps its "head" = its best
 // key over the patterns that still have room; one step = arg-max of the heads over the free
 // columns, accept it, and if that filled the pattern, recompute the heads that pointed to it.
-// A step is a wavefront (or workgroup) max-reduction; a tile needs c*g steps.
+// A step is a wavefront (or workgroup) max-reduction; a tile needs c*g steps.  The kernels
+// further down batch these steps: the lane teams run many small tiles per wavefront, and the
+// rounds accept in one pass everything the walk accepts before the next pattern fills.
 //
 // Work split: a "team" of TW wavefronts owns one tile; a workgroup holds NT teams that work on
 // NT consecutive tiles, which are adjacent in memory along the sparse dim when that dim is the
@@ -646,12 +648,475 @@ template <typename T, int L> static int launch_sparsify_teams(SparsifyParams &P,
     return NMG_OK;
 }
 
+// ------------------------------------------------------------- rounds: batched acceptance
+// The sorted walk accepts, between two moments at which a pattern fills up, exactly the heads of
+// the free columns whose key is at least the key at which the next pattern fills: until then no
+// pattern is full, so every column met in the walk is accepted by the first pattern it asks for
+// (its head).  One *round* therefore does in parallel what the step-by-step formulation does in
+// up to c*g steps:
+//   1. every free column proposes to its head pattern (best key over the patterns with room);
+//   2. the proposals are grouped by pattern (counting sort) and every proposal gets its rank
+//      inside its pattern's group in descending key order;
+//   3. a pattern with more proposals than room fills at the key of its proposal of rank room-1;
+//      t = the largest such key over the patterns (0 when no pattern overflows);
+//   4. every proposal with key >= t is accepted into slot p*g + used[p] + rank: inside a pattern
+//      the walk hands out slots in descending key order, and the keys accepted later are smaller;
+//   5. the columns whose head pattern is now full compute a new head.
+// Every round fills at least one pattern or ends the tile, so a tile takes at most c rounds.
+//
+// A tile belongs to NT threads: one wavefront (four tiles per workgroup, wavefront-level
+// synchronisation only) or a whole workgroup.  The free columns live in a compact list that
+// every round rewrites, so a round costs as many wavefront passes as the columns that are still
+// free need, not as the tile has.  For scores of 32 bits (every type but double) and m <= 8; a
+// key is one 64-bit word: (score bits + 1) << 32 | column << 16 | pattern.
+struct RoundParams {
+    SparsifyParams sp;
+    int region_bytes;                          // LDS bytes of one tile
+    int r_gk, r_fk, r_oidx, r_work, r_int;     // offsets inside a tile region
+    int tiles;                                 // tiles per workgroup
+    int cpad_log2;                             // log2 of the power of two >= c
+    uint64_t magic_cols, magic_g;
+};
+
+template <int NT> __device__ __forceinline__ void tile_sync()
+{
+    if (NT == 64) {
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    } else {
+        __syncthreads();
+    }
+}
+
+// Inclusive prefix sum over the 64 lanes of a wavefront with DPP moves: shifts by 1, 2, 4, 8
+// inside the rows of 16 lanes, then lane 15 of rows 0 and 2 is added to rows 1 and 3, then lane
+// 31 to rows 2 and 3.
+template <int CTRL, int ROWS> __device__ __forceinline__ int dpp_move0(int v)
+{
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, ROWS, 0xF, CTRL < 0x140);
+}
+__device__ __forceinline__ int wave_prefix_sum(int v)
+{
+    v += dpp_move0<0x111, 0xF>(v);   // row_shr:1
+    v += dpp_move0<0x112, 0xF>(v);   // row_shr:2
+    v += dpp_move0<0x114, 0xF>(v);   // row_shr:4
+    v += dpp_move0<0x118, 0xF>(v);   // row_shr:8
+    v += dpp_move0<0x142, 0xA>(v);   // row_bcast:15 into rows 1 and 3
+    v += dpp_move0<0x143, 0xC>(v);   // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+template <typename T, int NT, int CPT>
+__global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(RoundParams Q)
+{
+    const SparsifyParams &P = Q.sp;
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int n = P.n, m = P.m, g = P.g, c = P.c, cols = P.cols;
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    const int tile = tid / NT, tt = tid % NT;
+    const int tiles = Q.tiles;
+
+    // LDS: [order table][pattern masks][tile regions]
+    int8_t *s_order = (int8_t *)smem;
+    uint8_t *s_mask = (uint8_t *)(smem + ((c * n + 15) & ~15));
+    const int order_bytes = ((c * n + 15) & ~15) + ((c + 15) & ~15);
+    unsigned char *region = smem + order_bytes + (size_t)tile * Q.region_bytes;
+    T *s_d = (T *)region;
+    uint64_t *s_gk = (uint64_t *)(region + Q.r_gk);     // proposals grouped by pattern: key >> 16
+    uint64_t *s_fk = (uint64_t *)(region + Q.r_fk);     // free columns: key of the head
+    int16_t *s_oidx = (int16_t *)(region + Q.r_oidx);
+    uint16_t *s_work = (uint16_t *)(region + Q.r_work); // columns waiting for a new head
+    int *s_dem = (int *)(region + Q.r_int);             // proposals per pattern in this round
+    int *s_start = s_dem + c;                           // first entry of the pattern's group
+    int *s_used = s_start + c;                          // slots taken
+    int *s_new = s_used + c;                            // slots taken in this round
+    int *s_cnt = s_new + c;                             // free columns: list of this round, of the next
+    int *s_nwork = s_cnt + 2;
+    int *s_props = s_nwork + 1;                         // proposals of this round
+    uint64_t *s_fill = (uint64_t *)(s_dem + 4 * c + 4);   // largest fill key of the round
+
+    for (int i = tid; i < c * n; i += nthr) s_order[i] = P.order[i];
+    for (int p = tid; p < c; p += nthr) {
+        int mk = 0;
+        for (int j = 0; j < n; j++) mk |= 1 << P.order[p * n + j];
+        s_mask[p] = (uint8_t)mk;
+    }
+
+    // ---- cooperative load of the workgroup's tiles (zero beyond G / S) ----
+    // Last tiles first: the tiles of the last chunk of the group dim are padded with zero
+    // columns, whose equal keys make them the most expensive ones; they should not be the tail.
+    const int64_t tile0 = ((int64_t)gridDim.x - 1 - blockIdx.x) * tiles;
+    const T *dense = (const T *)P.dense;
+    const int64_t tiles_per_b = P.view.num_chunks * P.view.num_blocks;
+    if (P.view.stride_g == 1) {
+        // the columns are contiguous: consecutive threads walk them
+        for (int line = 0; line < tiles * m; line++) {
+            const int tm = line / m, r = line - tm * m;
+            const int64_t t = tile0 + tm;
+            T *dst = (T *)(smem + order_bytes + (size_t)tm * Q.region_bytes) + r;
+            const T *src = nullptr;
+            int valid_cols = 0;
+            if (t < P.outer) {
+                const int64_t b = t / tiles_per_b;
+                const int64_t rem = t - b * tiles_per_b;
+                const int64_t kc = rem / P.view.num_blocks;
+                const int64_t mb = rem - kc * P.view.num_blocks;
+                const int64_t si = mb * m + r;
+                if (si < P.view.S) {
+                    src = dense + b * P.view.stride_b + kc * cols + si * P.view.stride_s;
+                    const int64_t left = P.view.G - kc * cols;
+                    valid_cols = left < cols ? (int)left : cols;
+                }
+            }
+            for (int o = tid; o < cols; o += nthr) dst[o * m] = o < valid_cols ? src[o] : Zero<T>::v();
+        }
+    } else {
+        // consecutive threads take the m values of a column, then the same column of the next
+        // tile (adjacent along the sparse dim); a thread keeps its (tile, position) pair and walks
+        // the columns, so the 64-bit index arithmetic is done once
+        const int per = tiles * m, walkers = nthr / per;
+        if (tid < walkers * per) {
+            const int o0 = tid / per, rest = tid - o0 * per;
+            const int tm = rest / m, r = rest - tm * m;
+            const int64_t t = tile0 + tm;
+            T *dst = (T *)(smem + order_bytes + (size_t)tm * Q.region_bytes) + r;
+            const T *src = nullptr;
+            int valid_cols = 0;
+            if (t < P.outer) {
+                const int64_t b = t / tiles_per_b;
+                const int64_t rem = t - b * tiles_per_b;
+                const int64_t kc = rem / P.view.num_blocks;
+                const int64_t mb = rem - kc * P.view.num_blocks;
+                const int64_t si = mb * m + r;
+                if (si < P.view.S) {
+                    src = dense + b * P.view.stride_b + kc * cols * P.view.stride_g + si * P.view.stride_s;
+                    const int64_t left = P.view.G - kc * cols;
+                    valid_cols = left < cols ? (int)left : cols;
+                }
+            }
+            const int64_t sg = P.view.stride_g;
+#pragma unroll 4
+            for (int o = o0; o < cols; o += walkers) dst[o * m] = o < valid_cols ? src[o * sg] : Zero<T>::v();
+        }
+    }
+    if (tile < tiles)
+        for (int p = tt; p < 4 * c + 6; p += NT) s_dem[p] = 0;   // counters and the fill key
+    __syncthreads();
+
+    const bool live = tile < tiles && tile0 + tile < P.outer;
+    // Real columns of this tile; the rest (beyond the end of the group dim) is zero padding.
+    int real_cols = cols;
+    if (live) {
+        const int64_t rem = (tile0 + tile) % tiles_per_b;
+        const int64_t left = P.view.G - rem / P.view.num_blocks * cols;
+        if (left < cols) real_cols = (int)left;
+    }
+
+    // Score of column o for the pattern with position mask mk: the sum runs over the pattern's
+    // positions in ascending order, in single precision, as the reference's.
+    auto load_col = [&](int o, float (&a)[8]) {
+        const T *col = s_d + o * m;
+#pragma unroll
+        for (int r = 0; r < 8; r++) a[r] = score_of(col[r < m ? r : 0]);
+    };
+    auto score = [&](const float (&a)[8], int mk) {
+        float acc = 0;
+#pragma unroll
+        for (int r = 0; r < 8; r++)
+            if ((mk >> r) & 1) acc += a[r];
+        return acc;
+    };
+
+    if (live) {
+        // heads of all columns: every pattern has room; on equal scores the larger pattern wins
+        for (int o = tt; o < real_cols; o += NT) {
+            float a[8];
+            load_col(o, a);
+            uint32_t best_s = 0;
+            int best_p = 0;
+#pragma unroll 4
+            for (int p = 0; p < c; p++) {
+                const uint32_t sb = score_bits(score(a, s_mask[p])) + 1;
+                if (sb >= best_s) {
+                    best_s = sb;
+                    best_p = p;
+                }
+            }
+            s_fk[o] = ((uint64_t)best_s << 32) | ((uint32_t)o << 16) | (uint32_t)best_p;
+        }
+        if (tt == 0) s_cnt[0] = real_cols;
+        tile_sync<NT>();
+
+        // Zero padding: the padded columns have score 0 for every pattern and the largest column
+        // numbers of the tile, so the walk meets them after every key with a positive score and
+        // before every other key with score 0, in descending column order, and each takes the
+        // largest pattern with room.  They never enter the list: the rounds first run on the
+        // positive keys alone (hold = true: a column whose head has score 0 waits), then the
+        // padded columns are placed in closed form, then the rounds go on with what is left.
+        bool hold = real_cols < cols;
+        for (int round = 0; round <= 2 * c + 2; round++) {
+            const int q = round & 1;
+            const int nfree = s_cnt[q];
+            if (nfree == 0 && !hold) break;
+            const int ns = (nfree + NT - 1) / NT;   // list entries per thread in this round
+            uint64_t key[CPT];   // key of the head; 0 = no entry, or placed
+            int pos[CPT];        // place inside the pattern's group, then rank
+            uint32_t waiting = 0;   // entries held back in this round
+            // 1. proposals per pattern; the returned count is the place inside the group
+#pragma unroll
+            for (int i = 0; i < CPT; i++) {
+                key[i] = 0;
+                pos[i] = 0;
+                if (i < ns && tt + NT * i < nfree) {
+                    key[i] = s_fk[tt + NT * i];
+                    if (hold && (key[i] >> 32) == 1) waiting |= 1u << i;
+                    else pos[i] = atomicAdd(&s_dem[(int)(key[i] & 0xFFFFu)], 1);
+                }
+            }
+            tile_sync<NT>();
+            // 2. group offsets: exclusive prefix sum of the demands (first wavefront of the tile;
+            //    c <= 128, two patterns per lane)
+            if (tt < 64) {
+                const int p0 = 2 * tt, p1 = 2 * tt + 1;
+                const int d0 = p0 < c ? s_dem[p0] : 0, d1 = p1 < c ? s_dem[p1] : 0;
+                const int excl = wave_prefix_sum(d0 + d1) - (d0 + d1);
+                if (p0 < c) {
+                    s_start[p0] = excl;
+                    s_new[p0] = 0;
+                }
+                if (p1 < c) {
+                    s_start[p1] = excl + d0;
+                    s_new[p1] = 0;
+                }
+                if (tt == 0) {
+                    s_cnt[q ^ 1] = 0;   // the list of the next round starts empty
+                    *s_fill = 0;
+                }
+                if (tt == 63) *s_props = excl + d0 + d1;   // proposals of this round
+            }
+            tile_sync<NT>();
+            bool regular = true;
+            if (hold && *s_props == 0) {
+                // No positive key is left.  Padded column number k from the top (column
+                // cols-1-k) goes to the pattern p with top(p) <= k < top(p) + room(p), where
+                // top(p) = room of the patterns above p.  Lane l of the first wavefront takes the
+                // patterns c-1-2l and c-2-2l.
+                if (tt < 64) {
+                    const int p0 = c - 1 - 2 * tt, p1 = c - 2 - 2 * tt;
+                    const int r0 = p0 >= 0 ? g - s_used[p0] : 0, r1 = p1 >= 0 ? g - s_used[p1] : 0;
+                    const int excl = wave_prefix_sum(r0 + r1) - (r0 + r1);
+                    if (p0 >= 0) s_start[p0] = excl;
+                    if (p1 >= 0) s_start[p1] = excl + r0;
+                }
+                tile_sync<NT>();
+                const int npad = cols - real_cols;
+                for (int e = tt; e < (npad > 0 ? c : 0); e += NT) {
+                    // pattern e takes the padded columns [top, top + room) that exist
+                    const int top = s_start[e], room = g - s_used[e];
+                    const int take = npad - top < room ? (npad - top > 0 ? npad - top : 0) : room;
+                    s_new[e] = take;
+                }
+                for (int k = tt; k < npad; k += NT) {
+                    // top() grows as p falls: the pattern is the smallest p with top(p) <= k
+                    // (then k < top(p-1) = top(p) + room(p), and the total room covers k at p = 0)
+                    int lo = 0, hi = c - 1;
+                    while (lo < hi) {
+                        const int mid = (lo + hi) >> 1;
+                        if (s_start[mid] <= k) hi = mid;
+                        else lo = mid + 1;
+                    }
+                    s_oidx[lo * g + s_used[lo] + (k - s_start[lo])] = (int16_t)(cols - 1 - k);
+                }
+                tile_sync<NT>();
+                for (int p = tt; p < c; p += NT) s_used[p] += s_new[p];
+                // the held entries may now point to a full pattern: all of them take a new head
+                if (tt == 0) {
+                    s_cnt[q ^ 1] = 0;
+                    *s_nwork = 0;
+                }
+                tile_sync<NT>();
+#pragma unroll
+                for (int i = 0; i < CPT; i++)
+                    if ((waiting >> i) & 1) {
+                        const int w = atomicAdd(s_nwork, 1);
+                        s_work[w] = (uint16_t)((key[i] >> 16) & 0xFFFFu);
+                        s_gk[w] = 0;
+                    }
+                hold = false;
+                regular = false;
+                tile_sync<NT>();
+            }
+            if (regular) {
+                // 3. grouped list: (score bits + 1) << 16 | column
+#pragma unroll
+                for (int i = 0; i < CPT; i++)
+                    if (i < ns && key[i] != 0 && !((waiting >> i) & 1)) s_gk[s_start[(int)(key[i] & 0xFFFFu)] + pos[i]] = key[i] >> 16;
+                tile_sync<NT>();
+                // 4. rank inside the group (keys differ in the column at least); the proposal at
+                //    which an overflowing pattern fills publishes its key
+#pragma unroll
+                for (int i = 0; i < CPT; i++)
+                    if (i < ns && key[i] != 0 && !((waiting >> i) & 1)) {
+                        const int p = (int)(key[i] & 0xFFFFu);
+                        const uint64_t mine = key[i] >> 16;
+                        const int seg = s_start[p], d = s_dem[p];
+                        const int room = g - s_used[p];
+                        // Eight entries are in flight at a time (the loop is bound by the LDS round
+                        // trip).  A proposal that has seen `room` larger keys cannot be accepted in
+                        // this round -- its pattern fills above it -- and stops counting.  The group
+                        // is read from its end: equal scores (zero padding) are ordered by column,
+                        // and the later entries tend to be the larger columns.
+                        int r = 0;
+                        for (int j0 = 0; j0 < d && r < room; j0 += 8) {
+                            uint64_t e[8];
+#pragma unroll
+                            for (int u = 0; u < 8; u++) e[u] = s_gk[seg + d - 1 - (j0 + u < d ? j0 + u : d - 1)];
+#pragma unroll
+                            for (int u = 0; u < 8; u++) r += (j0 + u < d && e[u] > mine) ? 1 : 0;
+                        }
+                        pos[i] = r;
+                        if (d > room && r == room - 1) atomicMax((unsigned long long *)s_fill, (unsigned long long)key[i]);
+                    }
+                tile_sync<NT>();
+                // 5. accept what lies at or above the largest fill key (0: no pattern overflows)
+                const uint64_t fill = *s_fill;
+#pragma unroll
+                for (int i = 0; i < CPT; i++)
+                    if (i < ns && key[i] != 0 && !((waiting >> i) & 1) && key[i] >= fill) {
+                        const int p = (int)(key[i] & 0xFFFFu);
+                        s_oidx[p * g + s_used[p] + pos[i]] = (int16_t)((key[i] >> 16) & 0xFFFFu);
+                        atomicAdd(&s_new[p], 1);
+                        key[i] = 0;
+                    }
+                tile_sync<NT>();
+                // 6. counters
+                for (int p = tt; p < c; p += NT) {
+                    s_used[p] += s_new[p];
+                    s_dem[p] = 0;
+                }
+                tile_sync<NT>();
+                // 7. the columns that stay free go to the next round's list; those whose pattern
+                //    has filled need a new head first
+#pragma unroll
+                for (int i = 0; i < CPT; i++)
+                    if (i < ns && key[i] != 0) {
+                        if (s_used[(int)(key[i] & 0xFFFFu)] >= g) {
+                            const int w = atomicAdd(s_nwork, 1);
+                            s_work[w] = (uint16_t)((key[i] >> 16) & 0xFFFFu);
+                            s_gk[w] = 0;
+                        } else {
+                            s_fk[atomicAdd(&s_cnt[q ^ 1], 1)] = key[i];
+                        }
+                    }
+                tile_sync<NT>();
+            }
+            // 8. new heads, one thread per (column, pattern): these columns are few and a loop
+            //    over the patterns is a chain of LDS round trips; the best key of a column is
+            //    gathered with an LDS maximum (the grouped list, free between two rounds, holds it)
+            const int nwork = *s_nwork;
+            if (nwork > 0) {
+                const int cl = Q.cpad_log2;
+                for (int e = tt; e < (nwork << cl); e += NT) {
+                    const int w = e >> cl, p = e & ((1 << cl) - 1);
+                    if (p < c && s_used[p] < g) {
+                        float a[8];
+                        load_col(s_work[w], a);
+                        const uint32_t sb = score_bits(score(a, s_mask[p])) + 1;
+                        atomicMax((unsigned long long *)&s_gk[w], ((unsigned long long)sb << 32) | (unsigned)p);
+                    }
+                }
+                tile_sync<NT>();
+                for (int w = tt; w < nwork; w += NT)
+                    s_fk[atomicAdd(&s_cnt[q ^ 1], 1)] = s_gk[w] | ((uint64_t)s_work[w] << 16);
+                if (tt == 0) *s_nwork = 0;
+                tile_sync<NT>();
+            }
+        }
+    }
+
+    // ---- coalesced store of the workgroup's tiles: one thread per slot writes its index and
+    //      gathers its n values from the tile data ----
+    __syncthreads();
+    T *val = (T *)P.val;
+    for (int e = tid; e < tiles * cols; e += nthr) {
+        const int tm = (int)(((uint64_t)e * Q.magic_cols) >> 32), slot = e - tm * cols;
+        const int64_t t = tile0 + tm;
+        if (t >= P.outer) continue;
+        const unsigned char *reg = smem + order_bytes + (size_t)tm * Q.region_bytes;
+        const int o = ((const int16_t *)(reg + Q.r_oidx))[slot];
+        const int p = (int)(((uint64_t)slot * Q.magic_g) >> 32);
+        const T *col = (const T *)reg + o * m;
+        const int64_t at = t * (int64_t)cols + slot;
+        P.idx[at] = (int16_t)o;
+        for (int j = 0; j < n; j++) val[at * n + j] = col[s_order[p * n + j]];
+    }
+}
+
+template <typename T, int NT, int CPT>
+static int launch_sparsify_rounds(SparsifyParams &P, hipStream_t stream, bool *done)
+{
+    *done = false;
+    if (sizeof(typename ScoreOf<T>::bits) != 4) return NMG_OK;
+    RoundParams Q{};
+    Q.sp = P;
+    const int cols = P.cols, m = P.m, c = P.c, n = P.n;
+    if (m > 8 || c > 128 || n < 1 || cols > NT * CPT) return NMG_OK;
+    Q.tiles = NT == 64 ? 4 : 1;
+    if ((int64_t)Q.tiles * cols >= 65536) return NMG_OK;   // the magic divisions hold below 2^16
+    int off = align_up(cols * m * (int)sizeof(T), 8);
+    Q.r_gk = off;
+    off += cols * 8;
+    Q.r_fk = off;
+    off += cols * 8;
+    Q.r_oidx = off;
+    off = align_up(off + cols * 2, 4);
+    Q.r_work = off;
+    off = align_up(off + cols * 2, 8);
+    Q.r_int = off;
+    off = align_up(off + (4 * c + 6) * 4, 8);
+    Q.region_bytes = off;
+    const int threads = NT == 64 ? 256 : NT;
+    const size_t order_bytes = (size_t)align_up(c * n, 16) + (size_t)align_up(c, 16);
+    const size_t lds = order_bytes + (size_t)Q.tiles * Q.region_bytes;
+    if (lds > 160 * 1024) return NMG_OK;   // too large for this kernel: the caller falls back
+    Q.cpad_log2 = 0;
+    while ((1 << Q.cpad_log2) < c) Q.cpad_log2++;
+    Q.magic_cols = (((uint64_t)1 << 32) + cols - 1) / cols;
+    Q.magic_g = (((uint64_t)1 << 32) + P.g - 1) / P.g;
+    auto kern = sparsify_rounds_kernel<T, NT, CPT>;
+    if (lds > 64 * 1024)
+        NMG_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)lds));
+    const int64_t grid = (P.outer + Q.tiles - 1) / Q.tiles;
+    NMG_REQUIRE(grid <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "too many tiles (%lld)", (long long)grid);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(threads), lds, stream, Q);
+    NMG_HIP_TRY(hipGetLastError());
+    *done = true;
+    return NMG_OK;
+}
+
 template <typename T> static int dispatch_sparsify(SparsifyParams &P, hipStream_t stream)
 {
-    // Small tiles: one wavefront per tile, four tiles per workgroup.  Larger tiles: four
-    // wavefronts per tile -- more of them lose to the two workgroup barriers of every step
-    // (measured on 896-column tiles: 1 / 2 / 4 / 8 / 16 wavefronts -> 17.6 / 12.6 / 10.9 / 21.1 / 69 ms
-    // for an 8192 x 8192 weight).
+    // Tiles of more than 32 columns: batched rounds, with as many threads per tile as its first
+    // round keeps busy (measured on 4096 x 4096 fp16, 2:4 with g = 8 / 16 / 32 / 64: 305 / 208 /
+    // 155 / 200 us against 407 / 402 / 742 / 1204 us for the lane teams below; 8192 x 8192,
+    // 2:8:32 and 4:8:32: 1.06 and 3.2 ms against 10.9 and 56 ms for the step-by-step kernel).
+    // Smaller tiles would leave most of a wavefront idle: they stay with the lane teams.
+    if (P.cols > 32 && P.n > 0) {
+        bool done = false;
+        int rc;
+        if (P.cols <= 256) rc = launch_sparsify_rounds<T, 64, 4>(P, stream, &done);
+        else if (P.cols <= 512) rc = launch_sparsify_rounds<T, 128, 4>(P, stream, &done);
+        else if (P.cols <= 1024) rc = launch_sparsify_rounds<T, 256, 4>(P, stream, &done);
+        else rc = launch_sparsify_rounds<T, 1024, 4>(P, stream, &done);
+        if (rc != NMG_OK || done) return rc;
+    }
+    // What the rounds do not take (tiles of at most 32 columns, double, m > 8, more than 128
+    // patterns) goes step by step: lane teams for tiles of up to 512 columns, else one
+    // wavefront per tile (four tiles per workgroup) or four wavefronts per tile -- more of them
+    // lose to the two workgroup barriers of every step (measured on 896-column tiles: 1 / 2 / 4 /
+    // 8 / 16 wavefronts -> 17.6 / 12.6 / 10.9 / 21.1 / 69 ms for an 8192 x 8192 weight).
     if (P.cols <= 512 && P.n > 0) {
         // lane teams: about 16 to 32 columns per lane
         bool done = false;

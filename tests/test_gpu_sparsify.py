@@ -73,6 +73,36 @@ def test_ties_and_zeros():
     check_parity(w.half(), 1, 4, 0, 8, 1)
 
 
+@pytest.mark.parametrize("n,m,g,rows", [
+    (2, 4, 16, 96 * 2 + 40),     # one wavefront per tile; 56 padded columns in the last chunk
+    (2, 4, 64, 384 + 7),         # 384 columns: two wavefronts per tile, 377 padded columns
+    (2, 8, 32, 896 + 130),       # four wavefronts per tile, 766 padded columns
+    (4, 8, 32, 2240 + 33),       # sixteen wavefronts per tile
+    (1, 8, 8, 64 * 3 + 1),       # a single real column beside 63 padded ones
+])
+def test_zero_columns_beside_zero_padding(n, m, g, rows):
+    # Zero padding is placed in closed form after the keys with a positive score; real columns
+    # that are zero, wholly or in the positions of some patterns, tie with it and must come out
+    # as in the sorted walk: before it when their score is positive, after it when it is zero.
+    gen = torch.Generator().manual_seed(rows)
+    w = torch.randn(rows, 5 * m, generator=gen) * 0.02
+    w[torch.rand(rows, generator=gen) < 0.3] = 0                      # whole columns of every tile
+    w[torch.rand(rows, 5 * m, generator=gen) < 0.4] = 0               # scattered zeros
+    w[:, m:2 * m] = torch.randint(-1, 2, (rows, m), generator=gen).float() * 0.5   # three magnitudes
+    w[:, 2 * m:3 * m] = 0                                             # a block column of zero tiles
+    check_parity(w.half(), n, m, 1, g, 0)
+    check_parity(w.t().contiguous(), n, m, 0, g, 1)
+
+
+def test_resparsifying_a_pruned_weight():
+    # half of the entries are exact zeros already, so most patterns of a column tie at its best score
+    w = seeded((500, 256), torch.float16, seed=21, std=0.02)
+    t = sten.GroupedNMTensor.from_dense(w.to(DEV), 2, 4, 1, 16, 0)
+    check_parity(t.to_dense().cpu(), 2, 4, 1, 32, 0)
+    check_parity(t.to_dense().cpu(), 1, 4, 1, 16, 0)
+    check_parity(t.to_dense().cpu(), 2, 8, 1, 8, 0)
+
+
 def test_reference_test_shapes_5_12_2():
     # tests/test_nmg.py:33-86: shapes (3,a,b), a,b in {17,5,1}, all axis orders, 5:12:2
     torch.manual_seed(123)
