@@ -823,27 +823,47 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
     auto score = [&](const float (&a)[8], int mk) {
         float acc = 0;
 #pragma unroll
-        for (int r = 0; r < 8; r++)
+        for (int r = 0; r < 8; r++) {
+            if (r >= m) break;
             if ((mk >> r) & 1) acc += a[r];
+        }
         return acc;
     };
 
     if (live) {
-        // heads of all columns: every pattern has room; on equal scores the larger pattern wins
-        for (int o = tt; o < real_cols; o += NT) {
-            float a[8];
-            load_col(o, a);
-            uint32_t best_s = 0;
-            int best_p = 0;
-#pragma unroll 4
-            for (int p = 0; p < c; p++) {
-                const uint32_t sb = score_bits(score(a, s_mask[p])) + 1;
-                if (sb >= best_s) {
-                    best_s = sb;
-                    best_p = p;
-                }
+        // heads of all columns: every pattern has room; on equal scores the larger pattern wins.
+        // The patterns are the outer loop: a pattern's mask is fetched once for the thread's
+        // columns and made a scalar, so its positions are picked without lane selects.
+        {
+            float a[CPT][8];
+            uint32_t bs[CPT];
+            int bp[CPT];
+            const int ns0 = (real_cols + NT - 1) / NT;
+#pragma unroll
+            for (int i = 0; i < CPT; i++) {
+                bs[i] = 0;
+                bp[i] = 0;
+                if (i < ns0) load_col(tt + NT * i < real_cols ? tt + NT * i : 0, a[i]);
             }
-            s_fk[o] = ((uint64_t)best_s << 32) | ((uint32_t)o << 16) | (uint32_t)best_p;
+#pragma unroll 2
+            for (int p = 0; p < c; p++) {
+                const int mk = __builtin_amdgcn_readfirstlane((int)s_mask[p]);
+#pragma unroll
+                for (int i = 0; i < CPT; i++)
+                    if (i < ns0) {
+                        const uint32_t sb = score_bits(score(a[i], mk)) + 1;
+                        if (sb >= bs[i]) {
+                            bs[i] = sb;
+                            bp[i] = p;
+                        }
+                    }
+            }
+#pragma unroll
+            for (int i = 0; i < CPT; i++) {
+                const int o = tt + NT * i;
+                if (i < ns0 && o < real_cols)
+                    s_fk[o] = ((uint64_t)bs[i] << 32) | ((uint32_t)o << 16) | (uint32_t)bp[i];
+            }
         }
         if (tt == 0) s_cnt[0] = real_cols;
         tile_sync<NT>();
@@ -1106,7 +1126,8 @@ template <typename T> static int dispatch_sparsify(SparsifyParams &P, hipStream_
     if (P.cols > 32 && P.n > 0) {
         bool done = false;
         int rc;
-        if (P.cols <= 256) rc = launch_sparsify_rounds<T, 64, 4>(P, stream, &done);
+        if (P.cols <= 128) rc = launch_sparsify_rounds<T, 64, 2>(P, stream, &done);
+        else if (P.cols <= 256) rc = launch_sparsify_rounds<T, 64, 4>(P, stream, &done);
         else if (P.cols <= 512) rc = launch_sparsify_rounds<T, 128, 4>(P, stream, &done);
         else if (P.cols <= 1024) rc = launch_sparsify_rounds<T, 256, 4>(P, stream, &done);
         else rc = launch_sparsify_rounds<T, 1024, 4>(P, stream, &done);
