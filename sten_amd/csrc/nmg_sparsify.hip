@@ -876,10 +876,15 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
         // padded columns are placed in closed form, then the rounds go on with what is left.
         bool hold = real_cols < cols;
         for (int round = 0; round <= 2 * c + 2; round++) {
+            // The free columns of this round: the list of the columns whose head stayed valid,
+            // then the columns that were given a new head at the end of the last round.
             const int q = round & 1;
-            const int nfree = s_cnt[q];
+            const int nlist = s_cnt[q], nredo = *s_nwork;
+            const int nfree = nlist + nredo;
             if (nfree == 0 && !hold) break;
-            const int ns = (nfree + NT - 1) / NT;   // list entries per thread in this round
+            // entries per thread in this round; a wavefront beyond the end of the list has none
+            // and only keeps the barriers
+            const int ns = (tt & ~63) < nfree ? (nfree + NT - 1) / NT : 0;
             uint64_t key[CPT];   // key of the head; 0 = no entry, or placed
             int pos[CPT];        // place inside the pattern's group, then rank
             uint32_t waiting = 0;   // entries held back in this round
@@ -888,35 +893,38 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
             for (int i = 0; i < CPT; i++) {
                 key[i] = 0;
                 pos[i] = 0;
-                if (i < ns && tt + NT * i < nfree) {
-                    key[i] = s_fk[tt + NT * i];
+                const int e = tt + NT * i;
+                if (i < ns && e < nfree) {
+                    key[i] = e < nlist ? s_fk[e] : (s_gk[e - nlist] | ((uint64_t)s_work[e - nlist] << 16));
                     if (hold && (key[i] >> 32) == 1) waiting |= 1u << i;
                     else pos[i] = atomicAdd(&s_dem[(int)(key[i] & 0xFFFFu)], 1);
                 }
             }
             tile_sync<NT>();
-            // 2. group offsets: exclusive prefix sum of the demands (first wavefront of the tile;
-            //    c <= 128, two patterns per lane)
+            // 2. the slots taken in the last round are booked; group offsets: exclusive prefix sum
+            //    of the demands (first wavefront of the tile; c <= 128, two patterns per lane)
             if (tt < 64) {
                 const int p0 = 2 * tt, p1 = 2 * tt + 1;
                 const int d0 = p0 < c ? s_dem[p0] : 0, d1 = p1 < c ? s_dem[p1] : 0;
                 const int excl = wave_prefix_sum(d0 + d1) - (d0 + d1);
                 if (p0 < c) {
                     s_start[p0] = excl;
+                    s_used[p0] += s_new[p0];
                     s_new[p0] = 0;
                 }
                 if (p1 < c) {
                     s_start[p1] = excl + d0;
+                    s_used[p1] += s_new[p1];
                     s_new[p1] = 0;
                 }
                 if (tt == 0) {
                     s_cnt[q ^ 1] = 0;   // the list of the next round starts empty
+                    *s_nwork = 0;
                     *s_fill = 0;
                 }
                 if (tt == 63) *s_props = excl + d0 + d1;   // proposals of this round
             }
             tile_sync<NT>();
-            bool regular = true;
             if (hold && *s_props == 0) {
                 // No positive key is left.  Padded column number k from the top (column
                 // cols-1-k) goes to the pattern p with top(p) <= k < top(p) + room(p), where
@@ -931,12 +939,6 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
                 }
                 tile_sync<NT>();
                 const int npad = cols - real_cols;
-                for (int e = tt; e < (npad > 0 ? c : 0); e += NT) {
-                    // pattern e takes the padded columns [top, top + room) that exist
-                    const int top = s_start[e], room = g - s_used[e];
-                    const int take = npad - top < room ? (npad - top > 0 ? npad - top : 0) : room;
-                    s_new[e] = take;
-                }
                 for (int k = tt; k < npad; k += NT) {
                     // top() grows as p falls: the pattern is the smallest p with top(p) <= k
                     // (then k < top(p-1) = top(p) + room(p), and the total room covers k at p = 0)
@@ -949,13 +951,12 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
                     s_oidx[lo * g + s_used[lo] + (k - s_start[lo])] = (int16_t)(cols - 1 - k);
                 }
                 tile_sync<NT>();
-                for (int p = tt; p < c; p += NT) s_used[p] += s_new[p];
-                // the held entries may now point to a full pattern: all of them take a new head
-                if (tt == 0) {
-                    s_cnt[q ^ 1] = 0;
-                    *s_nwork = 0;
+                for (int p = tt; p < c; p += NT) {
+                    // pattern p has taken the padded columns [top, top + room) that exist
+                    const int top = s_start[p], room = g - s_used[p];
+                    s_used[p] += npad - top < room ? (npad - top > 0 ? npad - top : 0) : room;
                 }
-                tile_sync<NT>();
+                // the held entries may now point to a full pattern: all of them take a new head
 #pragma unroll
                 for (int i = 0; i < CPT; i++)
                     if ((waiting >> i) & 1) {
@@ -964,14 +965,13 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
                         s_gk[w] = 0;
                     }
                 hold = false;
-                regular = false;
                 tile_sync<NT>();
-            }
-            if (regular) {
+            } else {
                 // 3. grouped list: (score bits + 1) << 16 | column
 #pragma unroll
                 for (int i = 0; i < CPT; i++)
-                    if (i < ns && key[i] != 0 && !((waiting >> i) & 1)) s_gk[s_start[(int)(key[i] & 0xFFFFu)] + pos[i]] = key[i] >> 16;
+                    if (i < ns && key[i] != 0 && !((waiting >> i) & 1))
+                        s_gk[s_start[(int)(key[i] & 0xFFFFu)] + pos[i]] = key[i] >> 16;
                 tile_sync<NT>();
                 // 4. rank inside the group (keys differ in the column at least); the proposal at
                 //    which an overflowing pattern fills publishes its key
@@ -984,14 +984,12 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
                         const int room = g - s_used[p];
                         // Eight entries are in flight at a time (the loop is bound by the LDS round
                         // trip).  A proposal that has seen `room` larger keys cannot be accepted in
-                        // this round -- its pattern fills above it -- and stops counting.  The group
-                        // is read from its end: equal scores (zero padding) are ordered by column,
-                        // and the later entries tend to be the larger columns.
+                        // this round -- its pattern fills above it -- and stops counting.
                         int r = 0;
                         for (int j0 = 0; j0 < d && r < room; j0 += 8) {
                             uint64_t e[8];
 #pragma unroll
-                            for (int u = 0; u < 8; u++) e[u] = s_gk[seg + d - 1 - (j0 + u < d ? j0 + u : d - 1)];
+                            for (int u = 0; u < 8; u++) e[u] = s_gk[seg + (j0 + u < d ? j0 + u : d - 1)];
 #pragma unroll
                             for (int u = 0; u < 8; u++) r += (j0 + u < d && e[u] > mine) ? 1 : 0;
                         }
@@ -999,29 +997,20 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
                         if (d > room && r == room - 1) atomicMax((unsigned long long *)s_fill, (unsigned long long)key[i]);
                     }
                 tile_sync<NT>();
-                // 5. accept what lies at or above the largest fill key (0: no pattern overflows)
+                // 5. What lies at or above the largest fill key (0: no pattern overflows) is
+                //    accepted.  The pattern of that key is the one pattern that this round leaves
+                //    without room while proposals to it remain: of the columns that stay free,
+                //    those need a new head, the others go to the next round's list as they are.
                 const uint64_t fill = *s_fill;
-#pragma unroll
-                for (int i = 0; i < CPT; i++)
-                    if (i < ns && key[i] != 0 && !((waiting >> i) & 1) && key[i] >= fill) {
-                        const int p = (int)(key[i] & 0xFFFFu);
-                        s_oidx[p * g + s_used[p] + pos[i]] = (int16_t)((key[i] >> 16) & 0xFFFFu);
-                        atomicAdd(&s_new[p], 1);
-                        key[i] = 0;
-                    }
-                tile_sync<NT>();
-                // 6. counters
-                for (int p = tt; p < c; p += NT) {
-                    s_used[p] += s_new[p];
-                    s_dem[p] = 0;
-                }
-                tile_sync<NT>();
-                // 7. the columns that stay free go to the next round's list; those whose pattern
-                //    has filled need a new head first
+                const int filled = fill != 0 ? (int)(fill & 0xFFFFu) : -1;
 #pragma unroll
                 for (int i = 0; i < CPT; i++)
                     if (i < ns && key[i] != 0) {
-                        if (s_used[(int)(key[i] & 0xFFFFu)] >= g) {
+                        const int p = (int)(key[i] & 0xFFFFu);
+                        if (!((waiting >> i) & 1) && key[i] >= fill) {
+                            s_oidx[p * g + s_used[p] + pos[i]] = (int16_t)((key[i] >> 16) & 0xFFFFu);
+                            atomicAdd(&s_new[p], 1);
+                        } else if (p == filled) {
                             const int w = atomicAdd(s_nwork, 1);
                             s_work[w] = (uint16_t)((key[i] >> 16) & 0xFFFFu);
                             s_gk[w] = 0;
@@ -1029,27 +1018,25 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
                             s_fk[atomicAdd(&s_cnt[q ^ 1], 1)] = key[i];
                         }
                     }
+                for (int p = tt; p < c; p += NT) s_dem[p] = 0;
                 tile_sync<NT>();
             }
-            // 8. new heads, one thread per (column, pattern): these columns are few and a loop
+            // 6. new heads, one thread per (column, pattern): these columns are few and a loop
             //    over the patterns is a chain of LDS round trips; the best key of a column is
-            //    gathered with an LDS maximum (the grouped list, free between two rounds, holds it)
+            //    gathered with an LDS maximum (the grouped list, free between two rounds, holds
+            //    it, and the next round reads it from there)
             const int nwork = *s_nwork;
             if (nwork > 0) {
                 const int cl = Q.cpad_log2;
                 for (int e = tt; e < (nwork << cl); e += NT) {
                     const int w = e >> cl, p = e & ((1 << cl) - 1);
-                    if (p < c && s_used[p] < g) {
+                    if (p < c && s_used[p] + s_new[p] < g) {
                         float a[8];
                         load_col(s_work[w], a);
                         const uint32_t sb = score_bits(score(a, s_mask[p])) + 1;
                         atomicMax((unsigned long long *)&s_gk[w], ((unsigned long long)sb << 32) | (unsigned)p);
                     }
                 }
-                tile_sync<NT>();
-                for (int w = tt; w < nwork; w += NT)
-                    s_fk[atomicAdd(&s_cnt[q ^ 1], 1)] = s_gk[w] | ((uint64_t)s_work[w] << 16);
-                if (tt == 0) *s_nwork = 0;
                 tile_sync<NT>();
             }
         }
