@@ -119,6 +119,8 @@ def main():
     ap.add_argument("--kernel", default="auto")
     ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--eager", action="store_true", help="launch every step from Python, decode shapes too")
+    ap.add_argument("--graph", action="store_true", help="replay the timed steps from a HIP graph, large shapes too")
     ap.add_argument("--calibrate-copy", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -188,22 +190,42 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+
+    # Decode shapes: the K timed steps are recorded once into a HIP graph and replayed, as a
+    # serving loop would launch them -- a step lasts 6-13 us on the device, less than one launch
+    # through Python and ctypes costs on the host (about 15 us).  The large shapes keep the host
+    # busy for less than a step and are launched eagerly (--graph replays them too).
+    graph = None
+    if (kind in ("decode", "w4") and not args.eager) or (args.graph and kind not in ("step", "sparsify")):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(args.steps):
+                step()
+        graph.replay()
+        torch.cuda.synchronize()
+
+    def run_steps():
+        if graph is not None:
+            graph.replay()
+        else:
+            for _ in range(args.steps):
+                step()
+
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
+    run_steps()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / args.steps
 
-    # average duration of a step on the device: one HIP event pair around K back-to-back steps,
-    # recorded on the stream the kernels are launched on (torch's current stream)
+    # average duration of a step on the device: one HIP event pair around the K back-to-back
+    # steps, recorded on the stream they are launched on (torch's current stream)
     stream = torch.cuda.current_stream()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record(stream)
-    for _ in range(args.steps):
-        step()
+    run_steps()
     e1.record(stream)
     torch.cuda.synchronize()
     kern_ms = e0.elapsed_time(e1) / args.steps
+    launch = "hip graph of the timed steps, replayed" if graph is not None else "eager"
 
     out = {
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -218,7 +240,7 @@ def main():
         out.update({
             "metric": "nmg sparse x dense GEMM TFLOP/s (dense-equiv)",
             "value": dense_flops / wall / 1e12, "unit": "TFLOP/s",
-            "config": {"workload": desc, "kernel": args.kernel, "variant": args.variant,
+            "config": {"workload": desc, "kernel": args.kernel, "variant": args.variant, "launch": launch,
                        "effective_tflops": eff_flops / wall / 1e12, "kernel_ms": kern_ms},
             "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP16_TFLOPS,
                          "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS,
@@ -230,7 +252,7 @@ def main():
         out.update({
             "metric": "nmg sparsifier GB/s" if kind == "sparsify" else "nmg sparse x dense decode GB/s",
             "value": algo_bytes / wall / 1e9, "unit": "GB/s",
-            "config": {"workload": desc, "kernel": args.kernel, "kernel_ms": kern_ms,
+            "config": {"workload": desc, "kernel": args.kernel, "launch": launch, "kernel_ms": kern_ms,
                        "algorithmic_bytes": algo_bytes},
             "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": achieved / PEAK_HBM_GBS, "traffic": committed_traffic(args.workload)},

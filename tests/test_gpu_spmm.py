@@ -442,3 +442,29 @@ def test_decode_kernels_all_token_counts(T, dtype, M, K, n, m, g):
     ref = to_np(x).astype(np.float64) @ Wd.T + to_np(b).astype(np.float64)
     y = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)
     assert rel_l2(to_np(y), ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("M,K,T", [
+    (1024, 1024, 4),       # decode kernel
+    (1024, 1024, 512),     # sparse matrix cores, direct kernel
+])
+def test_hip_graph_replays_match_eager(M, K, T):
+    # A serving loop records the product once and replays it.  Every replay is checked against
+    # an eager call on the same input, with eager work and synchronisations between the replays.
+    print(f"case graph replay M={M} K={K} T={T}", flush=True)
+    w = make(seeded((M, K), torch.float16, seed=31, std=0.05), 2, 4, 16, 1)
+    x = seeded((T, K), torch.float16, seed=32).to(DEV)
+    b = seeded((M,), torch.float16, seed=33).to(DEV)
+    sten.spmm(w, x, b, reduce_dim=1)           # first call: tables and operand caches are set up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = sten.spmm(w, x, b, reduce_dim=1)
+    for seed in (40, 41, 42):
+        x.copy_(seeded((T, K), torch.float16, seed=seed).to(DEV))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = y.clone()
+        want = sten.spmm(w, x, b, reduce_dim=1)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay with input seed {seed} differs from the eager call"

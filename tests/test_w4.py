@@ -96,3 +96,24 @@ def test_registered_linear_like_the_reference_test():
     assert rel_l2(to_np(y), to_np(ref)) <= 2e-3
     with pytest.raises(sten.NmgError):
         sten.SparseMarlinTensor.from_dense(torch.zeros(8, 100, dtype=torch.float16, device="cuda:0"))
+
+
+@pytest.mark.gpu
+def test_hip_graph_replays_match_eager():
+    import sten_amd as sten
+    dev = "cuda:0"
+    q4 = sten.SparseMarlinTensor.from_dense(seeded((512, 1024), torch.float16, seed=3, std=0.02).to(dev))
+    x = seeded((4, 1024), torch.float16, seed=4).to(dev)
+    q4.linear(x)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = q4.linear(x)
+    for seed in (50, 51, 52):
+        x.copy_(seeded((4, 1024), torch.float16, seed=seed).to(dev))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = y.clone()
+        want = q4.linear(x)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay with input seed {seed} differs from the eager call"
