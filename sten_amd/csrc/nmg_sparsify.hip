@@ -744,9 +744,14 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
     }
 
     // ---- cooperative load of the workgroup's tiles (zero beyond G / S) ----
-    // Last tiles first: the tiles of the last chunk of the group dim are padded with zero
-    // columns, whose equal keys make them the most expensive ones; they should not be the tail.
-    const int64_t tile0 = ((int64_t)gridDim.x - 1 - blockIdx.x) * tiles;
+    // Workgroups go to the 8 XCDs in turn, each with an L2 of its own, and up to 8 workgroups on
+    // consecutive tiles (adjacent along the sparse dim) read from the same 128-byte lines: among
+    // every 64 workgroups, XCD x gets the tile groups 8x .. 8x+7, so a line is fetched from HBM
+    // once, not once per XCD.  Last tiles first: the tiles of the last chunk of the group dim
+    // are padded with zero columns and should not be the tail.
+    int64_t grp = blockIdx.x;
+    if (grp < (int64_t)(gridDim.x & ~63u)) grp = (grp & ~63LL) | ((grp & 7) << 3) | ((grp >> 3) & 7);
+    const int64_t tile0 = ((int64_t)gridDim.x - 1 - grp) * tiles;
     const T *dense = (const T *)P.dense;
     const int64_t tiles_per_b = P.view.num_chunks * P.view.num_blocks;
     if (P.view.stride_g == 1) {
