@@ -57,6 +57,15 @@ WORKLOADS = {
 }
 
 
+# committed rocprofv3 --pmc summaries (FETCH_SIZE / WRITE_SIZE) of the workloads that have one
+PMC_SUMMARIES = {
+    "c2": "spmm_c2_pmc.txt",
+    "decode_1": "spmm_decode_1_pmc.txt",
+    "c4_b1": "w4_linear_c4_b1_pmc.txt",
+    "sparsify_c2": "sparsify_rounds_sparsify_c2_pmc.txt",
+}
+
+
 def cpu_baseline(M, K, N, n, m, g, seconds=15.0):
     import numpy as np
     from oracle import nmg_oracle as O
@@ -88,15 +97,15 @@ def cpu_baseline(M, K, N, n, m, g, seconds=15.0):
 
 def committed_traffic(workload):
     """HBM bytes per launch from profiles/ (FETCH_SIZE + WRITE_SIZE, calibrated), or None."""
-    for name in (f"spmm_{workload}_pmc.txt", f"{workload}_pmc.txt"):
-        try:
-            text = open(os.path.join(ROOT, "profiles", name)).read()
-        except OSError:
-            continue
-        mt = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", text, re.M)
-        if mt:
-            return float(mt.group(1))
-    return None
+    name = PMC_SUMMARIES.get(workload)
+    if name is None:
+        return None
+    try:
+        text = open(os.path.join(ROOT, "profiles", name)).read()
+    except OSError:
+        return None
+    mt = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", text, re.M)
+    return float(mt.group(1)) if mt else None
 
 
 def calibrate_copy():
@@ -211,19 +220,17 @@ def main():
             for _ in range(args.steps):
                 step()
 
-    t0 = time.perf_counter()
-    run_steps()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / args.steps
-
-    # average duration of a step on the device: one HIP event pair around the K back-to-back
-    # steps, recorded on the stream they are launched on (torch's current stream)
+    # The timed region: K back-to-back steps between two synchronisations.  The average duration
+    # of a step on the device comes from one HIP event pair around the same K steps, recorded on
+    # the stream they are launched on (torch's current stream).
     stream = torch.cuda.current_stream()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
     e0.record(stream)
     run_steps()
     e1.record(stream)
     torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / args.steps
     kern_ms = e0.elapsed_time(e1) / args.steps
     launch = "hip graph of the timed steps, replayed" if graph is not None else "eager"
 
