@@ -675,6 +675,7 @@ struct RoundParams {
     int r_gk, r_fk, r_oidx, r_work, r_int;     // offsets inside a tile region
     int tiles;                                 // tiles per workgroup
     int cpad_log2;                             // log2 of the power of two >= c
+    uint32_t masks[32];                        // position mask of every pattern, four per word
     uint64_t magic_cols, magic_g;
 };
 
@@ -717,10 +718,9 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
     const int tile = tid / NT, tt = tid % NT;
     const int tiles = Q.tiles;
 
-    // LDS: [order table][pattern masks][tile regions]
-    int8_t *s_order = (int8_t *)smem;
-    uint8_t *s_mask = (uint8_t *)(smem + ((c * n + 15) & ~15));
-    const int order_bytes = ((c * n + 15) & ~15) + ((c + 15) & ~15);
+    // LDS: [pattern masks][tile regions]
+    uint8_t *s_mask = (uint8_t *)smem;
+    const int order_bytes = (c + 15) & ~15;
     unsigned char *region = smem + order_bytes + (size_t)tile * Q.region_bytes;
     T *s_d = (T *)region;
     uint64_t *s_gk = (uint64_t *)(region + Q.r_gk);     // proposals grouped by pattern: key >> 16
@@ -736,11 +736,13 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
     int *s_props = s_nwork + 1;                         // proposals of this round
     uint64_t *s_fill = (uint64_t *)(s_dem + 4 * c + 4);   // largest fill key of the round
 
-    for (int i = tid; i < c * n; i += nthr) s_order[i] = P.order[i];
-    for (int p = tid; p < c; p += nthr) {
-        int mk = 0;
-        for (int j = 0; j < n; j++) mk |= 1 << P.order[p * n + j];
-        s_mask[p] = (uint8_t)mk;
+    // The position masks of the patterns (bit r = position r is kept; a pattern's positions in
+    // ascending order are its entry of the order table) come with the kernel arguments and go
+    // to LDS through the scalar unit: a workgroup lives for some ten microseconds and would
+    // spend one or two of them waiting for a table in global memory.
+    for (int w = 0; w < (c + 3) / 4; w++) {
+        const uint32_t four = Q.masks[w];
+        if (tid == 0) ((uint32_t *)s_mask)[w] = four;
     }
 
     // ---- cooperative load of the workgroup's tiles (zero beyond G / S) ----
@@ -1061,7 +1063,11 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
         const T *col = (const T *)reg + o * m;
         const int64_t at = t * (int64_t)cols + slot;
         P.idx[at] = (int16_t)o;
-        for (int j = 0; j < n; j++) val[at * n + j] = col[s_order[p * n + j]];
+        int mk = s_mask[p];
+        for (int j = 0; j < n; j++) {
+            val[at * n + j] = col[__ffs(mk) - 1];   // the j-th kept position
+            mk &= mk - 1;
+        }
     }
 }
 
@@ -1089,11 +1095,15 @@ static int launch_sparsify_rounds(SparsifyParams &P, hipStream_t stream, bool *d
     off = align_up(off + (4 * c + 6) * 4, 8);
     Q.region_bytes = off;
     const int threads = NT == 64 ? 256 : NT;
-    const size_t order_bytes = (size_t)align_up(c * n, 16) + (size_t)align_up(c, 16);
+    const size_t order_bytes = (size_t)align_up(c, 16);
     const size_t lds = order_bytes + (size_t)Q.tiles * Q.region_bytes;
     if (lds > 160 * 1024) return NMG_OK;   // too large for this kernel: the caller falls back
     Q.cpad_log2 = 0;
     while ((1 << Q.cpad_log2) < c) Q.cpad_log2++;
+    const int8_t *order = host_order(n, m);
+    NMG_REQUIRE(order != nullptr, NMG_ERR_ARG, "invalid n:m = %d:%d", n, m);
+    for (int p = 0; p < c; p++)
+        for (int j = 0; j < n; j++) Q.masks[p / 4] |= 1u << (8 * (p % 4) + order[p * n + j]);
     Q.magic_cols = (((uint64_t)1 << 32) + cols - 1) / cols;
     Q.magic_g = (((uint64_t)1 << 32) + P.g - 1) / P.g;
     auto kern = sparsify_rounds_kernel<T, NT, CPT>;
