@@ -664,8 +664,9 @@ template <typename T, int L> static int launch_sparsify_teams(SparsifyParams &P,
 //   5. the columns whose head pattern is now full compute a new head.
 // Every round fills at least one pattern or ends the tile, so a tile takes at most c rounds.
 //
-// A tile belongs to NT threads: one wavefront (four tiles per workgroup, wavefront-level
-// synchronisation only) or a whole workgroup.  The free columns live in a compact list that
+// A tile belongs to NT threads: 16, 32 or 64 lanes of a wavefront (256 threads per workgroup,
+// wavefront-level synchronisation only; the teams of a wavefront run the same instruction stream
+// on their own tiles and simply diverge where their rounds differ) or a whole workgroup.  The free columns live in a compact list that
 // every round rewrites, so a round costs as many wavefront passes as the columns that are still
 // free need, not as the tile has.  For scores of 32 bits (every type but double) and m <= 8; a
 // key is one 64-bit word: (score bits + 1) << 32 | column << 16 | pattern.
@@ -681,7 +682,7 @@ struct RoundParams {
 
 template <int NT> __device__ __forceinline__ void tile_sync()
 {
-    if (NT == 64) {
+    if (NT <= 64) {
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
     } else {
@@ -689,26 +690,26 @@ template <int NT> __device__ __forceinline__ void tile_sync()
     }
 }
 
-// Inclusive prefix sum over the 64 lanes of a wavefront with DPP moves: shifts by 1, 2, 4, 8
+// Inclusive prefix sum over the 64 lanes of a wavefront (or over each half of it) with DPP moves: shifts by 1, 2, 4, 8
 // inside the rows of 16 lanes, then lane 15 of rows 0 and 2 is added to rows 1 and 3, then lane
 // 31 to rows 2 and 3.
 template <int CTRL, int ROWS> __device__ __forceinline__ int dpp_move0(int v)
 {
     return __builtin_amdgcn_update_dpp(0, v, CTRL, ROWS, 0xF, CTRL < 0x140);
 }
-__device__ __forceinline__ int wave_prefix_sum(int v)
+template <int LANES> __device__ __forceinline__ int wave_prefix_sum(int v)
 {
     v += dpp_move0<0x111, 0xF>(v);   // row_shr:1
     v += dpp_move0<0x112, 0xF>(v);   // row_shr:2
     v += dpp_move0<0x114, 0xF>(v);   // row_shr:4
     v += dpp_move0<0x118, 0xF>(v);   // row_shr:8
-    v += dpp_move0<0x142, 0xA>(v);   // row_bcast:15 into rows 1 and 3
-    v += dpp_move0<0x143, 0xC>(v);   // row_bcast:31 into rows 2 and 3
-    return v;
+    if (LANES >= 32) v += dpp_move0<0x142, 0xA>(v);   // row_bcast:15 into rows 1 and 3
+    if (LANES == 64) v += dpp_move0<0x143, 0xC>(v);   // row_bcast:31 into rows 2 and 3
+    return v;   // LANES == 32, 16: one sum per half, per row of the wavefront
 }
 
 template <typename T, int NT, int CPT>
-__global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(RoundParams Q)
+__global__ __launch_bounds__(NT <= 64 ? 256 : NT) void sparsify_rounds_kernel(RoundParams Q)
 {
     const SparsifyParams &P = Q.sp;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -913,7 +914,7 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
             if (tt < 64) {
                 const int p0 = 2 * tt, p1 = 2 * tt + 1;
                 const int d0 = p0 < c ? s_dem[p0] : 0, d1 = p1 < c ? s_dem[p1] : 0;
-                const int excl = wave_prefix_sum(d0 + d1) - (d0 + d1);
+                const int excl = wave_prefix_sum<(NT < 64 ? NT : 64)>(d0 + d1) - (d0 + d1);
                 if (p0 < c) {
                     s_start[p0] = excl;
                     s_used[p0] += s_new[p0];
@@ -929,7 +930,7 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
                     *s_nwork = 0;
                     *s_fill = 0;
                 }
-                if (tt == 63) *s_props = excl + d0 + d1;   // proposals of this round
+                if (tt == (NT < 64 ? NT : 64) - 1) *s_props = excl + d0 + d1;   // proposals of this round
             }
             tile_sync<NT>();
             if (hold && *s_props == 0) {
@@ -940,7 +941,7 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
                 if (tt < 64) {
                     const int p0 = c - 1 - 2 * tt, p1 = c - 2 - 2 * tt;
                     const int r0 = p0 >= 0 ? g - s_used[p0] : 0, r1 = p1 >= 0 ? g - s_used[p1] : 0;
-                    const int excl = wave_prefix_sum(r0 + r1) - (r0 + r1);
+                    const int excl = wave_prefix_sum<(NT < 64 ? NT : 64)>(r0 + r1) - (r0 + r1);
                     if (p0 >= 0) s_start[p0] = excl;
                     if (p1 >= 0) s_start[p1] = excl + r0;
                 }
@@ -1080,7 +1081,8 @@ static int launch_sparsify_rounds(SparsifyParams &P, hipStream_t stream, bool *d
     Q.sp = P;
     const int cols = P.cols, m = P.m, c = P.c, n = P.n;
     if (m > 8 || c > 128 || n < 1 || cols > NT * CPT) return NMG_OK;
-    Q.tiles = NT == 64 ? 4 : 1;
+    Q.tiles = NT <= 64 ? 256 / NT : 1;
+    if (NT < 64 && c > 2 * NT) return NMG_OK;   // the prefix sums take two patterns per lane
     if ((int64_t)Q.tiles * cols >= 65536) return NMG_OK;   // the magic divisions hold below 2^16
     int off = align_up(cols * m * (int)sizeof(T), 8);
     Q.r_gk = off;
@@ -1094,7 +1096,7 @@ static int launch_sparsify_rounds(SparsifyParams &P, hipStream_t stream, bool *d
     Q.r_int = off;
     off = align_up(off + (4 * c + 6) * 4, 8);
     Q.region_bytes = off;
-    const int threads = NT == 64 ? 256 : NT;
+    const int threads = NT <= 64 ? 256 : NT;
     const size_t order_bytes = (size_t)align_up(c, 16);
     const size_t lds = order_bytes + (size_t)Q.tiles * Q.region_bytes;
     if (lds > 160 * 1024) return NMG_OK;   // too large for this kernel: the caller falls back
@@ -1120,22 +1122,27 @@ static int launch_sparsify_rounds(SparsifyParams &P, hipStream_t stream, bool *d
 
 template <typename T> static int dispatch_sparsify(SparsifyParams &P, hipStream_t stream)
 {
-    // Tiles of more than 32 columns: batched rounds, with as many threads per tile as its first
-    // round keeps busy (measured on 4096 x 4096 fp16, 2:4 with g = 8 / 16 / 32 / 64: 305 / 208 /
-    // 155 / 200 us against 407 / 402 / 742 / 1204 us for the lane teams below; 8192 x 8192,
-    // 2:8:32 and 4:8:32: 1.06 and 3.2 ms against 10.9 and 56 ms for the step-by-step kernel).
-    // Smaller tiles would leave most of a wavefront idle: they stay with the lane teams.
-    if (P.cols > 32 && P.n > 0) {
+    // Tiles of at least 16 columns: batched rounds, with as many lanes per tile as its later
+    // rounds keep busy -- a quarter, a half or a whole wavefront (several tiles share the
+    // wavefront's instruction stream), else a workgroup.  Measured on 4096 x 4096 fp16, 2:4 with
+    // g = 4 / 8 / 16 / 32 / 64: 208 / 147 / 142 / 147 / 161 us against 320 / 407 / 402 / 742 / 1204 us
+    // for the lane teams below; 8192 x 8192, 1:8:32 / 2:8:32 / 4:8:32: 0.40 / 1.06 / 3.4 ms against
+    // 2.6 / 10.9 / 56 ms for the step-by-step kernels.  Half a wavefront loses to a whole one from
+    // about 20 patterns on (2:8:4, 112 columns: 430 against 367 us); tiles of fewer than 16 columns
+    // stay with the lane teams (2:4:2: 200 against 315 us).
+    if (P.cols >= 16 && P.n > 0) {
         bool done = false;
         int rc;
-        if (P.cols <= 128) rc = launch_sparsify_rounds<T, 64, 2>(P, stream, &done);
+        if (P.cols <= 64 && P.c <= 32) rc = launch_sparsify_rounds<T, 16, 4>(P, stream, &done);
+        else if (P.cols <= 128 && P.c <= 20) rc = launch_sparsify_rounds<T, 32, 4>(P, stream, &done);
+        else if (P.cols <= 128) rc = launch_sparsify_rounds<T, 64, 2>(P, stream, &done);
         else if (P.cols <= 256) rc = launch_sparsify_rounds<T, 64, 4>(P, stream, &done);
         else if (P.cols <= 512) rc = launch_sparsify_rounds<T, 128, 4>(P, stream, &done);
         else if (P.cols <= 1024) rc = launch_sparsify_rounds<T, 256, 4>(P, stream, &done);
         else rc = launch_sparsify_rounds<T, 1024, 4>(P, stream, &done);
         if (rc != NMG_OK || done) return rc;
     }
-    // What the rounds do not take (tiles of at most 32 columns, double, m > 8, more than 128
+    // What the rounds do not take (tiles of fewer than 16 columns, double, m > 8, more than 128
     // patterns) goes step by step: lane teams for tiles of up to 512 columns, else one
     // wavefront per tile (four tiles per workgroup) or four wavefronts per tile -- more of them
     // lose to the two workgroup barriers of every step (measured on 896-column tiles: 1 / 2 / 4 /

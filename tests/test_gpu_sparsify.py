@@ -74,11 +74,15 @@ def test_ties_and_zeros():
 
 
 @pytest.mark.parametrize("n,m,g,rows", [
-    (2, 4, 16, 96 * 2 + 40),     # one wavefront per tile; 56 padded columns in the last chunk
+    (2, 4, 16, 96 * 2 + 40),     # half a wavefront per tile; 56 padded columns in the last chunk
     (2, 4, 64, 384 + 7),         # 384 columns: two wavefronts per tile, 377 padded columns
+    (2, 8, 4, 112 + 30),         # one wavefront per tile (28 patterns)
+    (2, 4, 32, 192 + 9),         # one wavefront per tile, four entries per lane
     (2, 8, 32, 896 + 130),       # four wavefronts per tile, 766 padded columns
     (4, 8, 32, 2240 + 33),       # sixteen wavefronts per tile
-    (1, 8, 8, 64 * 3 + 1),       # a single real column beside 63 padded ones
+    (1, 8, 8, 64 * 3 + 1),       # quarter wavefronts; a single real column beside 63 padded ones
+    (2, 4, 8, 48 * 2 + 5),       # quarter wavefronts, 43 padded columns
+    (3, 6, 4, 80 + 13),          # half wavefronts, 20 patterns
 ])
 def test_zero_columns_beside_zero_padding(n, m, g, rows):
     # Zero padding is placed in closed form after the keys with a positive score; real columns
