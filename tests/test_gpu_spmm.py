@@ -468,3 +468,24 @@ def test_hip_graph_replays_match_eager(M, K, T):
         want = sten.spmm(w, x, b, reduce_dim=1)
         torch.cuda.synchronize()
         assert torch.equal(got, want), f"replay with input seed {seed} differs from the eager call"
+
+
+def test_tile_boundary_sweep_default_route():
+    # The reference sweeps every size across each tile boundary +-1 (matmul_generator.py:1482-1521).
+    # Here the boundaries are those of the default kernels: 32 / 64 / 256 lines, 16 / 128 / 256
+    # tokens, 64 / 128 reduction positions; whatever kernel the sizes select must agree with the
+    # dense product of the oracle's weight.
+    n, m, g = 2, 4, 16
+    for M in (255, 256, 257, 96 * 3 + 1):
+        for K in (64, 120, 128, 136, 192, 200):
+            W = seeded((M, K), torch.float16, seed=M * 7 + K, std=0.5)
+            Wd, _ = dense_ref(W, n, m, g, 1)
+            w = make(W, n, m, g, 1)
+            for T in (1, 15, 16, 17, 127, 128, 129, 255, 256, 257):
+                print(f"case sweep M={M} K={K} T={T}", flush=True)
+                x = seeded((T, K), torch.float16, seed=T)
+                y = sten.spmm(w, x.to(DEV), reduce_dim=1)
+                assert rel_l2(to_np(y), to_np(x).astype(np.float64) @ Wd.T) <= TOL[torch.float16], (M, K, T)
+                gy = seeded((T, M), torch.float16, seed=T + 1)
+                gx = sten.spmm(w, gy.to(DEV), reduce_dim=0)
+                assert rel_l2(to_np(gx), to_np(gy).astype(np.float64) @ Wd) <= TOL[torch.float16], (M, K, T)
