@@ -853,7 +853,6 @@ __global__ __launch_bounds__(NT <= 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
                 bp[i] = 0;
                 if (i < ns0) load_col(tt + NT * i < real_cols ? tt + NT * i : 0, a[i]);
             }
-#pragma unroll 2
             for (int p = 0; p < c; p++) {
                 const int mk = __builtin_amdgcn_readfirstlane((int)s_mask[p]);
 #pragma unroll

@@ -61,6 +61,7 @@ SIGNATURES = {
     "nmg_fragpack_supported": (_I, [_I, _I]),
     "nmg_fragpack_sizes": (_I, [_I64, _I64, ctypes.POINTER(_I64), ctypes.POINTER(_I64)]),
     "nmg_fragpack": (_I, [_P, _P, _I64, _I64, _P, _P, _I, _I, _I, _P]),
+    "nmg_pack_operands": (_I, [_P, _P, _I64, _I64, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "nmg_spmm_smfmac": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _P]),
     "nmg_gemm_nt": (_I, [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I, _P]),
 }

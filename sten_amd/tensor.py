@@ -175,27 +175,41 @@ class GroupedNMTensor:
         return self
 
     # ---- matmul operand ---------------------------------------------------------------------------
-    def rowpack(self):
-        """(pk_val [G, nb, n], pk_pat [G, nb]) -- per line of the group dim and block of the
-        sparse dim, the kept values and the pattern number; cached until ``val`` changes."""
+    def _pack(self):
+        """Derive the matmul operands from val/idx in one pass: the rowpack operand always, the
+        operand of the sparse matrix cores when the type and the pattern have one."""
         lay = self.layout
         if len(lay.dense_shape) != 2:
             raise native.NmgError("matmul needs a 2-D grouped n:m tensor")
         key = (self.val.data_ptr(), self.val._version, self.idx.data_ptr())
-        if self._rowpack is None or self._rowpack[0] != key:
-            native.require_gpu(self.val)
-            lib = native.load()
-            pat_bytes = lib.nmg_rowpack_pat_bytes(lay.n, lay.m)
-            pk_val = torch.empty((lay.G, lay.num_blocks, lay.n), dtype=self.val.dtype, device=self.val.device)
-            pk_pat = torch.empty((lay.G, lay.num_blocks),
-                                 dtype=torch.uint8 if pat_bytes == 1 else torch.int16,
-                                 device=self.val.device)
-            with torch.cuda.device(self.val.device):
-                native.check(lib.nmg_rowpack(
-                    native.ptr(self.val), native.ptr(self.idx), lay.G, lay.S, native.ptr(pk_val),
-                    native.ptr(pk_pat), lay.n, lay.m, lay.group_size,
-                    native.dtype_code(self.val.dtype), native.stream_ptr(self.val.device)))
-            self._rowpack = (key, pk_val, pk_pat)
+        if self._rowpack is not None and self._rowpack[0] == key:
+            return
+        native.require_gpu(self.val)
+        lib = native.load()
+        dev, dt = self.val.device, self.val.dtype
+        pat_bytes = lib.nmg_rowpack_pat_bytes(lay.n, lay.m)
+        pk_val = torch.empty((lay.G, lay.num_blocks, lay.n), dtype=dt, device=dev)
+        pk_pat = torch.empty((lay.G, lay.num_blocks), dtype=torch.uint8 if pat_bytes == 1 else torch.int16,
+                             device=dev)
+        fp_val = fp_idx = None
+        if dt in (torch.float16, torch.bfloat16) and lib.nmg_fragpack_supported(lay.n, lay.m):
+            ve, iw = ctypes.c_int64(), ctypes.c_int64()
+            native.check(lib.nmg_fragpack_sizes(lay.G, lay.S, ctypes.byref(ve), ctypes.byref(iw)))
+            fp_val = torch.empty(ve.value, dtype=dt, device=dev)
+            fp_idx = torch.empty(iw.value, dtype=torch.int32, device=dev)
+        with torch.cuda.device(dev):
+            native.check(lib.nmg_pack_operands(
+                native.ptr(self.val), native.ptr(self.idx), lay.G, lay.S, native.ptr(pk_val),
+                native.ptr(pk_pat), native.ptr(fp_val) if fp_val is not None else None,
+                native.ptr(fp_idx) if fp_idx is not None else None, lay.n, lay.m, lay.group_size,
+                native.dtype_code(dt), native.stream_ptr(dev)))
+        self._rowpack = (key, pk_val, pk_pat)
+        self._fragpack = (key, fp_val, fp_idx) if fp_val is not None else None
+
+    def rowpack(self):
+        """(pk_val [G, nb, n], pk_pat [G, nb]) -- per line of the group dim and block of the
+        sparse dim, the kept values and the pattern number; cached until ``val`` changes."""
+        self._pack()
         return self._rowpack[1], self._rowpack[2]
 
     def densefrag(self, reduce_dim):
@@ -241,27 +255,9 @@ class GroupedNMTensor:
         """Operand of the sparse-matrix-core kernel (values + 2-bit positions in instruction
         register order); ``None`` when the n:m pattern does not fit 2-of-4 groups or the dtype is
         not 16-bit.  Cached until ``val`` changes."""
-        lay = self.layout
-        lib = native.load()
-        if self.val.dtype not in (torch.float16, torch.bfloat16):
-            return None
-        if not lib.nmg_fragpack_supported(lay.n, lay.m):
-            return None
-        pk_val, pk_pat = self.rowpack()
-        key = self._rowpack[0]
+        self._pack()
         cached = getattr(self, "_fragpack", None)
-        if cached is None or cached[0] != key:
-            ve, iw = ctypes.c_int64(), ctypes.c_int64()
-            native.check(lib.nmg_fragpack_sizes(lay.G, lay.S, ctypes.byref(ve), ctypes.byref(iw)))
-            fp_val = torch.empty(ve.value, dtype=self.val.dtype, device=self.val.device)
-            fp_idx = torch.empty(iw.value, dtype=torch.int32, device=self.val.device)
-            with torch.cuda.device(self.val.device):
-                native.check(lib.nmg_fragpack(
-                    native.ptr(pk_val), native.ptr(pk_pat), lay.G, lay.S, native.ptr(fp_val),
-                    native.ptr(fp_idx), lay.n, lay.m, native.dtype_code(self.val.dtype),
-                    native.stream_ptr(self.val.device)))
-            self._fragpack = (key, fp_val, fp_idx)
-        return self._fragpack[1], self._fragpack[2]
+        return None if cached is None else (cached[1], cached[2])
 
     def __repr__(self):
         lay = self.layout
