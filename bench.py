@@ -44,6 +44,7 @@ WORKLOADS = {
     "c5_fwd": ("fwd", 16384, 4096, 4096, 2, 4, 16, "configs[4]: W 16384x4096 fp16 2:4:16 x 4096 tokens, forward"),
     "c5_grad_x": ("grad_x", 16384, 4096, 4096, 2, 4, 16, "configs[4]: dY 4096x16384 x W 16384x4096 fp16 2:4:16, grad_input"),
     "c5_step": ("step", 16384, 4096, 4096, 2, 4, 16, "configs[4]: training step of a sparse linear 4096 -> 16384, 4096 tokens: forward, grad_input, masked grad_weight in val layout"),
+    "c5_train": ("train", 16384, 4096, 4096, 2, 4, 16, "configs[4] + optimizer: the training step of c5_step followed by an SGD update of the compressed weight (pattern kept) and the re-derivation of the matmul operands"),
     "c2_grad_x": ("grad_x", 4096, 4096, 2048, 2, 4, 16, "configs[1] shape: dY 2048x4096 x W 4096x4096 fp16 2:4:16, grad_input"),
     "decode_1": ("decode", 4096, 11008, 1, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 1 token"),
     "decode_4": ("decode", 4096, 11008, 4, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 4 tokens"),
@@ -147,7 +148,7 @@ def main():
     torch.manual_seed(0)
     W = (torch.randn(M, K) * 0.02).half().to(dev)
 
-    if kind == "step":
+    if kind in ("step", "train"):
         # the registered F.linear through the dispatch layer, compressed weight gradient
         lin = torch.nn.Linear(K, M, bias=False).half().to(dev)
         with torch.no_grad():
@@ -161,10 +162,19 @@ def main():
         X = torch.randn(N, K, dtype=torch.float16, device=dev, requires_grad=True)
         dY = torch.randn(N, M, dtype=torch.float16, device=dev)
 
-        def step():
-            slin.weight.grad = None
-            X.grad = None
-            slin(X).backward(dY)
+        if kind == "train":
+            opt = torch.optim.SGD(slin.parameters(), lr=1e-3)
+
+            def step():
+                opt.zero_grad(set_to_none=True)
+                X.grad = None
+                slin(X).backward(dY)
+                opt.step()
+        else:
+            def step():
+                slin.weight.grad = None
+                X.grad = None
+                slin(X).backward(dY)
         algo_bytes = 0
     elif kind == "w4":
         w = sten.SparseMarlinTensor.from_dense(W)
@@ -205,7 +215,7 @@ def main():
     # through Python and ctypes costs on the host (about 15 us).  The large shapes keep the host
     # busy for less than a step and are launched eagerly (--graph replays them too).
     graph = None
-    if (kind in ("decode", "w4") and not args.eager) or (args.graph and kind not in ("step", "sparsify")):
+    if (kind in ("decode", "w4") and not args.eager) or (args.graph and kind not in ("step", "train", "sparsify")):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             for _ in range(args.steps):
@@ -240,8 +250,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
     }
-    if kind in ("fwd", "grad_x", "step"):
-        dense_flops = 2.0 * M * K * N * (3 if kind == "step" else 1)
+    if kind in ("fwd", "grad_x", "step", "train"):
+        dense_flops = 2.0 * M * K * N * (3 if kind in ("step", "train") else 1)
         eff_flops = dense_flops * n / m
         achieved = eff_flops / (kern_ms * 1e-3) / 1e12
         out.update({
