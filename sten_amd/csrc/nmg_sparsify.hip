@@ -1408,22 +1408,31 @@ template <typename T>
 static int launch_scatter_tiled(bool gather, ScatterParams &P, hipStream_t s, bool *done)
 {
     *done = false;
-    if (P.view.stride_s != 1 || P.view.num_blocks < 8) return NMG_OK;
-    // as many tiles per workgroup as 64 KiB of LDS hold, at most 64, at least 8
+    if (P.view.stride_s != 1 || P.view.num_blocks < 4) return NMG_OK;
+    // Tiles per workgroup: about 8 KiB of LDS (many small workgroups overlap each other's
+    // latencies: a 16384 x 4096 2:4:16 gather takes 81 us with 10 tiles, 112 us with 64), but at
+    // least 8 tiles so that a row of the region is a decent run of bytes, or 4 where 8 do not fit
+    // (2:8:32 with 8 tiles of 896 lines: 139 us against 760 us for the slot-per-thread kernel).
+    const int V = 16 / (int)sizeof(T);
     const int64_t per_tile = (int64_t)P.cols * P.m * (int64_t)sizeof(T);
-    int nt = (int)std::min<int64_t>(64, (60 * 1024) / per_tile);
-    if (nt < 8) return NMG_OK;
+    int nt = (int)std::min<int64_t>(64, (8 * 1024) / per_tile);
+    if (nt < 8) nt = 8;
     nt = (int)std::min<int64_t>(nt, P.view.num_blocks);
+    auto pitch_of = [&](int tiles, bool pad) { return ((tiles * P.m + V - 1) / V) * V + (pad ? V : 0); };
+    bool pad = true;
+    auto lds_of = [&](int tiles, bool pd) { return (size_t)P.cols * pitch_of(tiles, pd) * sizeof(T); };
+    if (lds_of(nt, pad) > 150 * 1024) nt = (int)std::min<int64_t>(4, P.view.num_blocks);
+    if (lds_of(nt, pad) > 150 * 1024) pad = false;    // rows without the vector of padding
+    if (lds_of(nt, pad) > 150 * 1024 || nt < 4) return NMG_OK;
     TiledParams Q{};
     Q.sp = P;
     Q.nt = nt;
-    const int V = 16 / (int)sizeof(T);
-    Q.pitch = ((nt * P.m + V - 1) / V) * V + V;         // 16-byte rows, one vector of padding
+    Q.pitch = pitch_of(nt, pad);
     Q.groups_per_chunk = (int)((P.view.num_blocks + nt - 1) / nt);
     Q.magic_cols = (((uint64_t)1 << 32) + P.cols - 1) / P.cols;
     Q.magic_g = (((uint64_t)1 << 32) + P.g - 1) / P.g;
-    const size_t lds = (size_t)P.cols * Q.pitch * sizeof(T);
-    if (lds > 160 * 1024 || (int64_t)nt * P.cols >= 65536) return NMG_OK;
+    const size_t lds = lds_of(nt, pad);
+    if ((int64_t)nt * P.cols >= 65536) return NMG_OK;
     const int64_t chunks = P.outer / P.view.num_blocks;   // batches x group-dim chunks
     const int64_t grid = chunks * Q.groups_per_chunk;
     if (grid > 0x7fffffffLL) return NMG_OK;
