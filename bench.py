@@ -13,8 +13,9 @@ For the bandwidth-bound workloads (decode shapes, sparsifier) value = GB/s of al
 (weight values + int16 indices + activations + output; dense input + val + idx for the
 sparsifier) and the roofline is HBM.  roofline.traffic is read from the committed rocprofv3 --pmc
 summary of the same command, when there is one.
-cpu_baseline (default workload only) = the CPU restatement of the reference's AVX/OpenMP kernel
-(oracle/nmg_cpu_simd.cpp) on the host cores, same shape, fp32.
+cpu_baseline (default workload) = the CPU restatement of the reference's AVX/OpenMP kernel
+(oracle/nmg_cpu_simd.cpp) on the host cores, same shape, fp32; for the sparsifier workloads the
+restatement of the reference's single-threaded sort-and-scan on a slab of the weight.
 
 Other modes: --workload picks another BASELINE shape; --calibrate-copy runs a plain device copy
 of known size (the counter calibration for FETCH_SIZE / WRITE_SIZE).
@@ -93,6 +94,33 @@ def cpu_baseline(M, K, N, n, m, g, seconds=15.0):
         "cores": info["threads"],
         "kind": "port",
         "sample": f"{M_s}x{K} fp32 slab of the weight x {N} tokens, {it} passes, kernel {info['kernel']}",
+    }
+
+
+def cpu_baseline_sparsify(M, K, n, m, g, seconds=10.0):
+    """The CPU restatement of the reference's sort-and-scan sparsifier (oracle/nmg_oracle.c), single
+    thread as the reference's (no OpenMP there), on a slab of whole chunks of the same weight."""
+    import math
+    import numpy as np
+    from oracle import nmg_oracle as O
+    cols = math.comb(m, n) * g
+    rows = min(M, max(cols, (256 // cols) * cols))
+    rng = np.random.default_rng(0)
+    W = (rng.standard_normal((rows, K)) * 0.02).astype(np.float16)
+    t0 = time.perf_counter()
+    it = 0
+    while True:
+        val, idx, _ = O.sparsify(W, n, m, 1, g, 0)
+        it += 1
+        if time.perf_counter() - t0 > seconds or it >= 20:
+            break
+    dt = (time.perf_counter() - t0) / it
+    return {
+        "value": (W.nbytes + val.nbytes + idx.nbytes) / dt / 1e9,
+        "unit": "GB/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": f"{rows}x{K} fp16 slab of the weight ({rows // cols} chunks of {cols} lines), {it} passes",
     }
 
 
@@ -276,6 +304,8 @@ def main():
         })
     if not args.no_cpu and args.workload == "c2":
         out["cpu_baseline"] = cpu_baseline(M, K, N, n, m, g)
+    if not args.no_cpu and kind == "sparsify":
+        out["cpu_baseline"] = cpu_baseline_sparsify(M, K, n, m, g)
     print(json.dumps(out))
 
 
