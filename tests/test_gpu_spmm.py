@@ -489,3 +489,33 @@ def test_tile_boundary_sweep_default_route():
                 gy = seeded((T, M), torch.float16, seed=T + 1)
                 gx = sten.spmm(w, gy.to(DEV), reduce_dim=0)
                 assert rel_l2(to_np(gx), to_np(gy).astype(np.float64) @ Wd) <= TOL[torch.float16], (M, K, T)
+
+
+def test_weight_of_more_than_2_31_elements():
+    # 40000 x 54016 fp16: element, slot and byte offsets beyond 32 bits in every kernel of the
+    # path.  Tiles are independent, so the oracle checks whole chunks cut out of the weight; the
+    # products are checked against the dense product of the library's own to_dense.
+    M, K = 40000, 54016
+    torch.manual_seed(0)
+    W = torch.empty(M, K, dtype=torch.float16, device=DEV).normal_(0, 0.02)
+    w = sten.GroupedNMTensor.from_dense(W, 2, 4, sparse_dim=1, group_size=16, group_dim=0)
+    lay = w.layout
+    cols, nb = lay.cols, lay.num_blocks
+    assert M * K > 2 ** 31 and w.val.numel() * 2 > 2 ** 31       # elements, bytes of val
+    for kc in (0, M // cols - 1, M // cols):          # first, last whole and the ragged last chunk
+        print(f"case big chunk {kc}", flush=True)
+        r0, r1 = kc * cols, min(M, (kc + 1) * cols)
+        val, idx, _ = oracle_sparsify(W[r0:r1].cpu(), 2, 4, 1, 16, 0)
+        assert np.array_equal(to_np(w.idx[kc * nb:(kc + 1) * nb]), idx)
+        assert np.array_equal(to_np(w.val[kc * nb:(kc + 1) * nb]).view(np.uint16), val.view(np.uint16))
+    D = w.to_dense()
+    assert bool(((D == W) | (D == 0)).all())
+    del W
+    for T in (5, 200):
+        print(f"case big T={T}", flush=True)
+        x = torch.randn(T, K, dtype=torch.float16, device=DEV)
+        ref = (x @ D.t()).float()
+        assert float((sten.spmm(w, x, reduce_dim=1).float() - ref).norm() / ref.norm()) <= 2e-3
+        gy = torch.randn(T, M, dtype=torch.float16, device=DEV)
+        ref = (gy @ D).float()
+        assert float((sten.spmm(w, gy, reduce_dim=0).float() - ref).norm() / ref.norm()) <= 2e-3
