@@ -992,11 +992,22 @@ __global__ __launch_bounds__(NT <= 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
                         // Eight entries are in flight at a time (the loop is bound by the LDS round
                         // trip).  A proposal that has seen `room` larger keys cannot be accepted in
                         // this round -- its pattern fills above it -- and stops counting.
-                        int r = 0;
-                        for (int j0 = 0; j0 < d && r < room; j0 += 8) {
+                        // Whole batches are counted unmasked; the last, partial one reads past
+                        // the group (into the next group or the array behind the list, both inside
+                        // the tile's LDS) and masks what it read there.
+                        const uint64_t *grp = s_gk + seg;
+                        int r = 0, j0 = 0;
+                        for (; j0 + 8 <= d && r < room; j0 += 8) {
                             uint64_t e[8];
 #pragma unroll
-                            for (int u = 0; u < 8; u++) e[u] = s_gk[seg + (j0 + u < d ? j0 + u : d - 1)];
+                            for (int u = 0; u < 8; u++) e[u] = grp[j0 + u];
+#pragma unroll
+                            for (int u = 0; u < 8; u++) r += e[u] > mine ? 1 : 0;
+                        }
+                        if (j0 < d && r < room) {
+                            uint64_t e[8];
+#pragma unroll
+                            for (int u = 0; u < 8; u++) e[u] = grp[j0 + u];
 #pragma unroll
                             for (int u = 0; u < 8; u++) r += (j0 + u < d && e[u] > mine) ? 1 : 0;
                         }
