@@ -510,6 +510,11 @@ template <typename T> static int launch_smfmac_pipe(SmfParams &P, hipStream_t s)
 // wavefront issues XL DMA loads and 3*FB register loads for step kp+DR_D, so "step kp+1 has
 // landed" is vmcnt <= OPS*(DR_D-1); the barrier that follows publishes the activation rows of
 // all four wavefronts.  Tile order, swizzle and preconditions as in the kernel above.
+//
+// A K step is cut into 2 * NH phases (k-step of 32 x a part of the wavefront's token blocks): the
+// MFMAs of a phase run while the activation fragments of the next one are read from LDS into a
+// second register set.  Short phases pay: with four MFMAs per phase the 256 x 128 tile is 3-12 %
+// faster than with eight (fewer fragments wait in registers, the LDS reads are spread thinner).
 constexpr int DR_D = 3;                 // K steps in flight
 constexpr int DR_NS = 4;                // activation stages in LDS (>= DR_D + 1)
 
@@ -717,16 +722,15 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
                 // unissued: 5 % on the 256 x 128 tile); in the last phase they come before the
                 // counted wait, which assumes them.
                 constexpr int L0 = PH * OPS / NP, L1 = (PH + 1) * OPS / NP;
-                static_assert(L1 - L0 <= NM - 2, "more loads than MFMAs to put them between");
                 if (PH != NP - 1) {
 #pragma unroll
                     for (int i = L0; i < L1; i++) {
                         __builtin_amdgcn_sched_barrier(0);
                         issue_one(kp + DR_D, ws[(u + DR_D) % (DR_D + 1)], i);
                         __builtin_amdgcn_sched_barrier(0);
-                        mma(ws[u], fr[PH % 2], ph_tag, 2 + i - L0, 3 + i - L0);
+                        if (2 + i - L0 < NM) mma(ws[u], fr[PH % 2], ph_tag, 2 + i - L0, 3 + i - L0);
                     }
-                    mma(ws[u], fr[PH % 2], ph_tag, 2 + L1 - L0, NM);
+                    if (2 + L1 - L0 < NM) mma(ws[u], fr[PH % 2], ph_tag, 2 + L1 - L0, NM);
                 } else {
                     mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
 #pragma unroll
@@ -739,11 +743,17 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
             };
             phase(std::integral_constant<int, 0>{});
             phase(std::integral_constant<int, 1>{});
-            if constexpr (NP == 4) {
+            if constexpr (NP >= 4) {
                 phase(std::integral_constant<int, 2>{});
                 phase(std::integral_constant<int, 3>{});
             }
-            static_assert(NP == 2 || NP == 4, "one or two token parts");
+            if constexpr (NP == 8) {
+                phase(std::integral_constant<int, 4>{});
+                phase(std::integral_constant<int, 5>{});
+                phase(std::integral_constant<int, 6>{});
+                phase(std::integral_constant<int, 7>{});
+            }
+            static_assert(NP == 2 || NP == 4 || NP == 8, "one, two or four token parts");
         }
     }
     pin_acc();
@@ -1225,12 +1235,10 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
 {
     if (variant < 0) {
         // Large-batch default.  The 256 x 256 tile moves a quarter fewer bytes per flop through
-        // the vector caches and runs a tile pair in ~0.8 of the time of two 256 x 128 tiles, but
-        // there are half as many tiles to spread over the 256 CUs: compare rounds of tiles.
-        const int64_t tm = (P.M + 255) / 256;
-        const int64_t n128 = tm * ((P.T + 127) / 128), n256 = tm * ((P.T + 255) / 256);
-        const double cost128 = (double)((n128 + 255) / 256), cost256 = 1.6 * (double)((n256 + 255) / 256);
-        variant = cost256 < cost128 ? 8 : 6;
+        // the vector caches, but with its K step split in four phases (LDS reads of one phase
+        // behind the MFMAs of the other) the 256 x 128 tile runs as fast per flop on shapes with
+        // many tiles (8192^2 x 4096: 267 us both) and fills the CUs better on shapes with few.
+        variant = 6;
     }
     switch (variant) {
     case 0: return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);  // 256 lines x 128 tokens, 1 wave/SIMD
@@ -1256,8 +1264,8 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
     case 8:                                                     // 256 x 256
         if (P.K % 64 != 0 || P.T * P.ldx * 2 >= (int64_t)1 << 31)
             return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
-        if (variant == 8) return launch_smfmac_direct<T, 2, 8, 4, 1, 2>(P, s);
-        return launch_smfmac_direct<T, 2, 4, 4, 1, 1>(P, s);
+        if (variant == 8) return launch_smfmac_direct<T, 2, 8, 4, 1, 4>(P, s);
+        return launch_smfmac_direct<T, 2, 4, 4, 1, 2>(P, s);
     }
     return NMG_ERR_ARG;
 }
