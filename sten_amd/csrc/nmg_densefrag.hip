@@ -120,7 +120,9 @@ constexpr int DD_NS = 4;   // activation stages in LDS (>= DD_D + 1)
 // FB x TB accumulator blocks (32 outputs x 32 tokens) per wavefront, WM x WN wavefronts, NH token
 // parts per k-step.  A K step (64) is 4 k-steps of 16; a phase is one (k-step, token part) pair:
 // its MFMAs run while the activation fragments of the next phase are read from LDS, and the
-// loads of K step kp+DD_D are issued in the first two phases.
+// loads of K step kp+DD_D are dealt out over the phases.  Short phases pay on the 256 x 256 tile
+// (sixteen phases of four MFMAs: 2-3 % over eight of eight); on the 256 x 128 tile they gain 12 %
+// on large shapes and lose as much on one-round shapes, where that tile is the one in use.
 template <typename T, int FB, int TB, int WM, int WN, int NH>
 __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
 {
@@ -313,8 +315,8 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
                 __builtin_amdgcn_sched_barrier(0);
                 if (PH == NP - 1) {
 #pragma unroll
-                    for (int i = 0; i < OPS / NP; i++)
-                        issue_one(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)], PH * (OPS / NP) + i);
+                    for (int i = PH * OPS / NP; i < OPS; i++)
+                        issue_one(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)], i);
                     __builtin_amdgcn_sched_barrier(0);
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // fragments of step kp are in registers
                     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DD_D - 1) * OPS) : "memory");  // my share of kp+1 landed
@@ -328,17 +330,16 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
                 // MFMAs: a burst would find the CU's vector memory path busy (16 clocks per 1 KiB
                 // instruction, shared by the four wavefronts) and stall with its MFMAs unissued.
                 // (In the last phase the loads come before the counted wait, which assumes them.)
-                constexpr int LPP = OPS / NP;               // loads per phase
-                static_assert(OPS % NP == 0 && LPP <= NM - 2, "loads spread evenly over the phases");
+                constexpr int L0 = PH * OPS / NP, L1 = (PH + 1) * OPS / NP;   // this phase's loads
                 if (PH != NP - 1) {
 #pragma unroll
-                    for (int i = 0; i < LPP; i++) {
+                    for (int i = L0; i < L1; i++) {
                         __builtin_amdgcn_sched_barrier(0);
-                        issue_one(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)], PH * LPP + i);
+                        issue_one(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)], i);
                         __builtin_amdgcn_sched_barrier(0);
-                        mma(ws[u], fr[PH % 2], ph_tag, 2 + i, 3 + i);
+                        if (2 + i - L0 < NM) mma(ws[u], fr[PH % 2], ph_tag, 2 + i - L0, 3 + i - L0);
                     }
-                    mma(ws[u], fr[PH % 2], ph_tag, 2 + LPP, NM);
+                    if (2 + L1 - L0 < NM) mma(ws[u], fr[PH % 2], ph_tag, 2 + L1 - L0, NM);
                 } else {
                     mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
                 }
@@ -348,13 +349,23 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
             phase(std::integral_constant<int, 1>{});
             phase(std::integral_constant<int, 2>{});
             phase(std::integral_constant<int, 3>{});
-            if constexpr (NP == 8) {
+            if constexpr (NP >= 8) {
                 phase(std::integral_constant<int, 4>{});
                 phase(std::integral_constant<int, 5>{});
                 phase(std::integral_constant<int, 6>{});
                 phase(std::integral_constant<int, 7>{});
             }
-            static_assert(NP == 4 || NP == 8, "one or two token parts");
+            if constexpr (NP == 16) {
+                phase(std::integral_constant<int, 8>{});
+                phase(std::integral_constant<int, 9>{});
+                phase(std::integral_constant<int, 10>{});
+                phase(std::integral_constant<int, 11>{});
+                phase(std::integral_constant<int, 12>{});
+                phase(std::integral_constant<int, 13>{});
+                phase(std::integral_constant<int, 14>{});
+                phase(std::integral_constant<int, 15>{});
+            }
+            static_assert(NP == 4 || NP == 8 || NP == 16, "one, two or four token parts");
         }
     }
     pin_acc();
@@ -392,7 +403,7 @@ template <typename T> static int launch_dense(DfParams &P, int variant, hipStrea
         const double cost128 = (double)((n128 + 255) / 256), cost256 = 1.7 * (double)((n256 + 255) / 256);
         variant = cost256 < cost128 ? 1 : 0;
     }
-    if (variant == 1) return launch_dense_direct<T, 2, 8, 4, 1, 2>(P, s);
+    if (variant == 1) return launch_dense_direct<T, 2, 8, 4, 1, 4>(P, s);
     return launch_dense_direct<T, 2, 4, 4, 1, 1>(P, s);
 }
 
