@@ -120,9 +120,7 @@ constexpr int DD_NS = 4;   // activation stages in LDS (>= DD_D + 1)
 // FB x TB accumulator blocks (32 outputs x 32 tokens) per wavefront, WM x WN wavefronts, NH token
 // parts per k-step.  A K step (64) is 4 k-steps of 16; a phase is one (k-step, token part) pair:
 // its MFMAs run while the activation fragments of the next phase are read from LDS, and the
-// loads of K step kp+DD_D are dealt out over the phases.  Short phases pay on the 256 x 256 tile
-// (sixteen phases of four MFMAs: 2-3 % over eight of eight); on the 256 x 128 tile they gain 12 %
-// on large shapes and lose as much on one-round shapes, where that tile is the one in use.
+// loads of K step kp+DD_D are dealt out over the phases.
 template <typename T, int FB, int TB, int WM, int WN, int NH>
 __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
 {
@@ -403,7 +401,7 @@ template <typename T> static int launch_dense(DfParams &P, int variant, hipStrea
         const double cost128 = (double)((n128 + 255) / 256), cost256 = 1.7 * (double)((n256 + 255) / 256);
         variant = cost256 < cost128 ? 1 : 0;
     }
-    if (variant == 1) return launch_dense_direct<T, 2, 8, 4, 1, 4>(P, s);
+    if (variant == 1) return launch_dense_direct<T, 2, 8, 4, 1, 2>(P, s);
     return launch_dense_direct<T, 2, 4, 4, 1, 1>(P, s);
 }
 

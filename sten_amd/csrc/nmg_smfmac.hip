@@ -1264,7 +1264,7 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
     case 8:                                                     // 256 x 256
         if (P.K % 64 != 0 || P.T * P.ldx * 2 >= (int64_t)1 << 31)
             return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
-        if (variant == 8) return launch_smfmac_direct<T, 2, 8, 4, 1, 4>(P, s);
+        if (variant == 8) return launch_smfmac_direct<T, 2, 8, 4, 1, 2>(P, s);
         return launch_smfmac_direct<T, 2, 4, 4, 1, 2>(P, s);
     }
     return NMG_ERR_ARG;

@@ -519,3 +519,26 @@ def test_weight_of_more_than_2_31_elements():
         gy = torch.randn(T, M, dtype=torch.float16, device=DEV)
         ref = (gy @ D).float()
         assert float((sten.spmm(w, gy, reduce_dim=0).float() - ref).norm() / ref.norm()) <= 2e-3
+
+
+def test_direct_kernels_on_a_full_chip_with_a_long_reduction():
+    # One tile per CU (or two) and 256 K steps: the shape on which a mistimed wait in the
+    # hand-scheduled kernels shows.  The pipelined variants must reproduce the plain kernel
+    # (variant 0) bit for bit on every run, and the dense route the dense product.
+    M, K, T = 4096, 16384, 4096
+    print(f"case full chip M={M} K={K} T={T}", flush=True)
+    w = make(seeded((M, K), torch.float16, seed=77, std=0.02), 2, 4, 16, 1)
+    x = seeded((T, K), torch.float16, seed=78).to(DEV)
+    w.spmm_opt["variant"] = 0
+    ref = sten.spmm(w, x, reduce_dim=1, kernel="smfmac").clone()
+    for variant in (6, 8):
+        w.spmm_opt["variant"] = variant
+        for _ in range(4):
+            assert torch.equal(sten.spmm(w, x, reduce_dim=1, kernel="smfmac"), ref), f"variant {variant}"
+    g = seeded((T, M), torch.float16, seed=79).to(DEV)
+    want = (g @ w.to_dense()).float()
+    for dense_variant in (0, 1):
+        w.spmm_opt["dense_variant"] = dense_variant
+        for _ in range(4):
+            got = sten.spmm(w, g, reduce_dim=0, kernel="densefrag").float()
+            assert float((got - want).norm() / want.norm()) <= 1e-4, f"dense variant {dense_variant}"
