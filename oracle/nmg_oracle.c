@@ -17,12 +17,15 @@
  *                        :724-805 (loop nest), :599-613 (tile constants)
  *
  * Parity status of each function (what pins it besides its own text):
- *   nmg_ref_order      -- pinned for (n,m) in {2:4, 1:8, 1:4, 1:m closed form} by
- *                         hand-traced tables, and for every (n,m) by the validity
+ *   nmg_ref_order      -- pinned by tables traced by hand through the recursion
+ *                         (tests/golden/hand_traced.json: 1:2, 1:3, 2:3, 1:4, 2:4,
+ *                         3:4, 2:5, 3:5, 2:6, 3:6, 1:8, 2:8, 3:8, 4:8, 7:8), by the
+ *                         1:m closed form, and for every (n,m) by the validity
  *                         invariants (increasing tuples, neighbours differ in one
- *                         slot, count C(m,n)).  The exact order for c>8 is fixed
- *                         only by the recursion itself: "parity unpinned" beyond
- *                         the invariants for those.
+ *                         slot, count C(m,n)).  For the other (n,m) with more than
+ *                         8 patterns (5:8, 6:8, m > 8) the exact order is fixed only
+ *                         by the recursion itself: "parity unpinned" beyond the
+ *                         invariants for those.
  *   nmg_ref_sparsify_* -- pinned by hand-worked tiles, the n==m closed form, the
  *                         all-zero closed form and a brute-force matcher on tiny
  *                         tiles (tests/test_oracle.py).
