@@ -673,9 +673,11 @@ template <typename T, int L> static int launch_sparsify_teams(SparsifyParams &P,
 struct RoundParams {
     SparsifyParams sp;
     int region_bytes;                          // LDS bytes of one tile
-    int r_gk, r_fk, r_oidx, r_work, r_int;     // offsets inside a tile region
+    int r_gk, r_fk, r_oidx, r_int;             // offsets inside a tile region
     int tiles;                                 // tiles per workgroup
     int cpad_log2;                             // log2 of the power of two >= c
+    int vec_bytes;                             // m values of a column are one aligned load of 4, 8 or 16 bytes (else 0)
+    int val_pairs;                             // val is aligned to 4 bytes
     uint32_t masks[32];                        // position mask of every pattern, four per word
     uint64_t magic_cols, magic_g;
 };
@@ -724,10 +726,11 @@ __global__ __launch_bounds__(NT <= 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
     const int order_bytes = (c + 15) & ~15;
     unsigned char *region = smem + order_bytes + (size_t)tile * Q.region_bytes;
     T *s_d = (T *)region;
-    uint64_t *s_gk = (uint64_t *)(region + Q.r_gk);     // proposals grouped by pattern: key >> 16
+    // proposals grouped by pattern: key >> 16; between two rounds its first entries are the
+    // columns waiting for a new head: best (score bits + 1) << 32 | column << 16 | pattern
+    uint64_t *s_gk = (uint64_t *)(region + Q.r_gk);
     uint64_t *s_fk = (uint64_t *)(region + Q.r_fk);     // free columns: key of the head
     int16_t *s_oidx = (int16_t *)(region + Q.r_oidx);
-    uint16_t *s_work = (uint16_t *)(region + Q.r_work); // columns waiting for a new head
     int *s_dem = (int *)(region + Q.r_int);             // proposals per pattern in this round
     int *s_start = s_dem + c;                           // first entry of the pattern's group
     int *s_used = s_start + c;                          // slots taken
@@ -757,7 +760,42 @@ __global__ __launch_bounds__(NT <= 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
     const int64_t tile0 = ((int64_t)gridDim.x - 1 - grp) * tiles;
     const T *dense = (const T *)P.dense;
     const int64_t tiles_per_b = P.view.num_chunks * P.view.num_blocks;
-    if (P.view.stride_g == 1) {
+    if (Q.vec_bytes != 0) {
+        // the m values of a column are contiguous and aligned: one load and one LDS write each.
+        // Consecutive threads take the same column of consecutive tiles (adjacent along the
+        // sparse dim, so adjacent in memory), then the next columns.
+        const int walkers = nthr / tiles;
+        if (tid < walkers * tiles) {
+            const int o0 = tid / tiles, tm = tid - o0 * tiles;
+            const int64_t t = tile0 + tm;
+            unsigned char *dst = smem + order_bytes + (size_t)tm * Q.region_bytes;
+            const T *src = nullptr;
+            int valid_cols = 0;
+            if (t < P.outer) {
+                const int64_t b = t / tiles_per_b;
+                const int64_t rem = t - b * tiles_per_b;
+                const int64_t kc = rem / P.view.num_blocks;
+                const int64_t mb = rem - kc * P.view.num_blocks;
+                src = dense + b * P.view.stride_b + kc * cols * P.view.stride_g + mb * m;
+                const int64_t left = P.view.G - kc * cols;
+                valid_cols = left < cols ? (int)left : cols;
+            }
+            const int64_t sg = P.view.stride_g;
+            if (Q.vec_bytes == 16) {
+#pragma unroll 4
+                for (int o = o0; o < cols; o += walkers)
+                    ((uint4 *)dst)[o] = o < valid_cols ? *(const uint4 *)(src + o * sg) : make_uint4(0, 0, 0, 0);
+            } else if (Q.vec_bytes == 8) {
+#pragma unroll 4
+                for (int o = o0; o < cols; o += walkers)
+                    ((uint2 *)dst)[o] = o < valid_cols ? *(const uint2 *)(src + o * sg) : make_uint2(0, 0);
+            } else {
+#pragma unroll 4
+                for (int o = o0; o < cols; o += walkers)
+                    ((uint32_t *)dst)[o] = o < valid_cols ? *(const uint32_t *)(src + o * sg) : 0u;
+            }
+        }
+    } else if (P.view.stride_g == 1) {
         // the columns are contiguous: consecutive threads walk them
         for (int line = 0; line < tiles * m; line++) {
             const int tm = line / m, r = line - tm * m;
@@ -825,8 +863,23 @@ __global__ __launch_bounds__(NT <= 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
     // positions in ascending order, in single precision, as the reference's.
     auto load_col = [&](int o, float (&a)[8]) {
         const T *col = s_d + o * m;
+        if (sizeof(T) == 2 && m == 8) {
+            // the tile starts on a 16-byte boundary of LDS: one read for the column
+            const uint4 raw = *(const uint4 *)col;
+            T v[8];
+            __builtin_memcpy(v, &raw, 16);
 #pragma unroll
-        for (int r = 0; r < 8; r++) a[r] = score_of(col[r < m ? r : 0]);
+            for (int r = 0; r < 8; r++) a[r] = score_of(v[r]);
+        } else if (sizeof(T) == 2 && m == 4) {
+            const uint2 raw = *(const uint2 *)col;
+            T v[4];
+            __builtin_memcpy(v, &raw, 8);
+#pragma unroll
+            for (int r = 0; r < 8; r++) a[r] = score_of(v[r & 3]);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 8; r++) a[r] = score_of(col[r < m ? r : 0]);
+        }
     };
     auto score = [&](const float (&a)[8], int mk) {
         float acc = 0;
@@ -902,7 +955,7 @@ __global__ __launch_bounds__(NT <= 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
                 pos[i] = 0;
                 const int e = tt + NT * i;
                 if (i < ns && e < nfree) {
-                    key[i] = e < nlist ? s_fk[e] : (s_gk[e - nlist] | ((uint64_t)s_work[e - nlist] << 16));
+                    key[i] = e < nlist ? s_fk[e] : s_gk[e - nlist];
                     if (hold && (key[i] >> 32) == 1) waiting |= 1u << i;
                     else pos[i] = atomicAdd(&s_dem[(int)(key[i] & 0xFFFFu)], 1);
                 }
@@ -968,8 +1021,7 @@ __global__ __launch_bounds__(NT <= 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
                 for (int i = 0; i < CPT; i++)
                     if ((waiting >> i) & 1) {
                         const int w = atomicAdd(s_nwork, 1);
-                        s_work[w] = (uint16_t)((key[i] >> 16) & 0xFFFFu);
-                        s_gk[w] = 0;
+                        s_gk[w] = key[i] & 0xFFFF0000ull;
                     }
                 hold = false;
                 tile_sync<NT>();
@@ -1030,8 +1082,7 @@ __global__ __launch_bounds__(NT <= 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
                             atomicAdd(&s_new[p], 1);
                         } else if (p == filled) {
                             const int w = atomicAdd(s_nwork, 1);
-                            s_work[w] = (uint16_t)((key[i] >> 16) & 0xFFFFu);
-                            s_gk[w] = 0;
+                            s_gk[w] = key[i] & 0xFFFF0000ull;
                         } else {
                             s_fk[atomicAdd(&s_cnt[q ^ 1], 1)] = key[i];
                         }
@@ -1050,9 +1101,11 @@ __global__ __launch_bounds__(NT <= 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
                     const int w = e >> cl, p = e & ((1 << cl) - 1);
                     if (p < c && s_used[p] + s_new[p] < g) {
                         float a[8];
-                        load_col(s_work[w], a);
+                        // the column sits in bits 16..31 of the entry, which the maxima leave alone
+                        const uint32_t o = ((const uint16_t *)&s_gk[w])[1];
+                        load_col((int)o, a);
                         const uint32_t sb = score_bits(score(a, s_mask[p])) + 1;
-                        atomicMax((unsigned long long *)&s_gk[w], ((unsigned long long)sb << 32) | (unsigned)p);
+                        atomicMax((unsigned long long *)&s_gk[w], ((unsigned long long)sb << 32) | (o << 16) | (unsigned)p);
                     }
                 }
                 tile_sync<NT>();
@@ -1075,9 +1128,20 @@ __global__ __launch_bounds__(NT <= 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
         const int64_t at = t * (int64_t)cols + slot;
         P.idx[at] = (int16_t)o;
         int mk = s_mask[p];
-        for (int j = 0; j < n; j++) {
-            val[at * n + j] = col[__ffs(mk) - 1];   // the j-th kept position
+        if (sizeof(T) == 2 && n == 2 && Q.val_pairs) {
+            // both values in one store
+            T v[2];
+            v[0] = col[__ffs(mk) - 1];
             mk &= mk - 1;
+            v[1] = col[__ffs(mk) - 1];
+            uint32_t raw;
+            __builtin_memcpy(&raw, v, 4);
+            ((uint32_t *)val)[at] = raw;
+        } else {
+            for (int j = 0; j < n; j++) {
+                val[at * n + j] = col[__ffs(mk) - 1];   // the j-th kept position
+                mk &= mk - 1;
+            }
         }
     }
 }
@@ -1100,13 +1164,18 @@ static int launch_sparsify_rounds(SparsifyParams &P, hipStream_t stream, bool *d
     Q.r_fk = off;
     off += cols * 8;
     Q.r_oidx = off;
-    off = align_up(off + cols * 2, 4);
-    Q.r_work = off;
     off = align_up(off + cols * 2, 8);
     Q.r_int = off;
     off = align_up(off + (4 * c + 6) * 4, 8);
-    Q.region_bytes = off;
+    Q.region_bytes = align_up(off, 16);
     const int threads = NT <= 64 ? 256 : NT;
+    // one aligned load per column where its m values are contiguous: sparse dim with stride 1
+    // and no partial last block, every column start a multiple of the vector size
+    const int vb = m * (int)sizeof(T);
+    if ((vb == 4 || vb == 8 || vb == 16) && P.view.stride_s == 1 && P.view.S % m == 0 &&
+        (uintptr_t)P.dense % vb == 0 && P.view.stride_g % m == 0 && P.view.stride_b % m == 0)
+        Q.vec_bytes = vb;
+    Q.val_pairs = (uintptr_t)P.val % 4 == 0;
     const size_t order_bytes = (size_t)align_up(c, 16);
     const size_t lds = order_bytes + (size_t)Q.tiles * Q.region_bytes;
     if (lds > 160 * 1024) return NMG_OK;   // too large for this kernel: the caller falls back
@@ -1136,10 +1205,13 @@ template <typename T> static int dispatch_sparsify(SparsifyParams &P, hipStream_
     // rounds keep busy -- a quarter, a half or a whole wavefront (several tiles share the
     // wavefront's instruction stream), else a workgroup.  Measured on 4096 x 4096 fp16, 2:4 with
     // g = 4 / 8 / 16 / 32 / 64: 208 / 147 / 142 / 147 / 161 us against 320 / 407 / 402 / 742 / 1204 us
-    // for the lane teams below; 8192 x 8192, 1:8:32 / 2:8:32 / 4:8:32: 0.40 / 1.06 / 3.4 ms against
+    // for the lane teams below; 8192 x 8192, 1:8:32 / 2:8:32 / 4:8:32: 0.39 / 0.92 / 2.1 ms against
     // 2.6 / 10.9 / 56 ms for the step-by-step kernels.  Half a wavefront loses to a whole one from
     // about 20 patterns on (2:8:4, 112 columns: 430 against 367 us); tiles of fewer than 16 columns
-    // stay with the lane teams (2:4:2: 200 against 315 us).
+    // stay with the lane teams (2:4:2: 200 against 315 us).  A tile's rounds are a chain of
+    // barriers and LDS round trips, so what counts is how many tiles a CU holds at once (34 bytes
+    // of LDS per column): 2240-column tiles (4:8:32) take 2.1 ms with 512 threads, two tiles per
+    // CU, against 3.4 ms with 1024 threads, whose registers allow one.
     if (P.cols >= 16 && P.n > 0) {
         bool done = false;
         int rc;
@@ -1149,6 +1221,7 @@ template <typename T> static int dispatch_sparsify(SparsifyParams &P, hipStream_
         else if (P.cols <= 256) rc = launch_sparsify_rounds<T, 64, 4>(P, stream, &done);
         else if (P.cols <= 512) rc = launch_sparsify_rounds<T, 128, 4>(P, stream, &done);
         else if (P.cols <= 1024) rc = launch_sparsify_rounds<T, 256, 4>(P, stream, &done);
+        else if (P.cols <= 2560) rc = launch_sparsify_rounds<T, 512, 5>(P, stream, &done);
         else rc = launch_sparsify_rounds<T, 1024, 4>(P, stream, &done);
         if (rc != NMG_OK || done) return rc;
     }

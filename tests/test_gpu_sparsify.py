@@ -130,6 +130,22 @@ def test_non_contiguous_input_and_empty():
     assert t.val.numel() == 0 and tuple(t.to_dense().shape) == (0, 8)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("n,m,g", [(2, 4, 16), (1, 8, 8), (2, 8, 4), (1, 2, 16)])
+def test_device_views_with_offsets_and_row_strides(dtype, n, m, g):
+    # the compressor reads a column's m values with one aligned load where it can; views whose
+    # base or row stride break the alignment, or whose rows are longer than the view, must give
+    # the same bits as a contiguous copy
+    for width, lo, hi in [(208, 8, 200), (208, 0, 192), (203, 3, 195), (203, 4, 196), (208, 1, 193)]:
+        big = seeded((130, width), dtype, seed=width + lo).to(DEV)
+        view = big[:, lo:hi]
+        print(f"case view of ({130},{width})[:, {lo}:{hi}] dtype={dtype} n:m:g={n}:{m}:{g}", flush=True)
+        val, idx, lay = oracle_sparsify(view.cpu().contiguous(), n, m, 1, g, 0)
+        t = sten.GroupedNMTensor.from_dense(view, n, m, sparse_dim=1, group_size=g, group_dim=0)
+        assert np.array_equal(to_np(t.idx), idx)
+        assert same_bits(t.val, val)
+
+
 def test_clone_layout_matches_oracle_gather():
     w = seeded((100, 72), torch.float32, seed=11)
     t, val, idx, lay = check_parity(w, 2, 4, 1, 4, 0)
