@@ -904,19 +904,36 @@ __global__ __launch_bounds__(NT <= 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
             for (int i = 0; i < CPT; i++) {
                 bs[i] = 0;
                 bp[i] = 0;
-                if (i < ns0) load_col(tt + NT * i < real_cols ? tt + NT * i : 0, a[i]);
+                load_col(i < ns0 && tt + NT * i < real_cols ? tt + NT * i : 0, a[i]);
             }
-            for (int p = 0; p < c; p++) {
-                const int mk = __builtin_amdgcn_readfirstlane((int)s_mask[p]);
+            // Four masks per LDS word; a position of the pattern is a branch of the whole
+            // wavefront around one addition per column (0 + x is x: the first one is exact too).
+            for (int w = 0; w < (c + 3) / 4; w++) {
+                const uint32_t four = __builtin_amdgcn_readfirstlane(((const uint32_t *)s_mask)[w]);
 #pragma unroll
-                for (int i = 0; i < CPT; i++)
-                    if (i < ns0) {
-                        const uint32_t sb = score_bits(score(a[i], mk)) + 1;
+                for (int j = 0; j < 4; j++) {
+                    const int p = 4 * w + j;
+                    if (p >= c) break;
+                    const uint32_t mk = (four >> (8 * j)) & 0xFFu;
+                    float acc[CPT];
+#pragma unroll
+                    for (int i = 0; i < CPT; i++) acc[i] = 0;
+#pragma unroll
+                    for (int r = 0; r < 8; r++)
+                        if ((mk >> r) & 1) {
+                            asm volatile("");   // keeps the branch: a select per column costs more
+#pragma unroll
+                            for (int i = 0; i < CPT; i++) acc[i] += a[i][r];
+                        }
+#pragma unroll
+                    for (int i = 0; i < CPT; i++) {
+                        const uint32_t sb = score_bits(acc[i]) + 1;
                         if (sb >= bs[i]) {
                             bs[i] = sb;
                             bp[i] = p;
                         }
                     }
+                }
             }
 #pragma unroll
             for (int i = 0; i < CPT; i++) {
