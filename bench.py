@@ -32,6 +32,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
+ROTATE_BYTES = 512 * 1024 * 1024
 PEAK_HBM_GBS = 8000.0
 
 WORKLOADS = {
@@ -51,6 +52,8 @@ WORKLOADS = {
     "decode_4": ("decode", 4096, 11008, 4, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 4 tokens"),
     "decode_8": ("decode", 4096, 11008, 8, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 8 tokens"),
     "decode_16": ("decode", 4096, 11008, 16, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 16 tokens"),
+    "decode_up_1": ("decode", 11008, 4096, 1, 2, 4, 16, "W 11008x4096 fp16 2:4:16 x 1 token (the up-projection beside the north_star shape)"),
+    "decode_up_16": ("decode", 11008, 4096, 16, 2, 4, 16, "W 11008x4096 fp16 2:4:16 x 16 tokens"),
     "c4_b1": ("w4", 11008, 4096, 1, 2, 4, 1, "configs[3]: W 11008x4096 2:4 + int4 (scale per 128) x 1 token"),
     "c4_b4": ("w4", 11008, 4096, 4, 2, 4, 1, "configs[3]: W 11008x4096 2:4 + int4 (scale per 128) x 4 tokens"),
     "c4_b16": ("w4", 11008, 4096, 16, 2, 4, 1, "configs[3]: W 11008x4096 2:4 + int4 (scale per 128) x 16 tokens"),
@@ -160,6 +163,9 @@ def main():
     ap.add_argument("--eager", action="store_true", help="launch every step from Python, decode shapes too")
     ap.add_argument("--graph", action="store_true", help="replay the timed steps from a HIP graph, large shapes too")
     ap.add_argument("--calibrate-copy", action="store_true")
+    ap.add_argument("--copies", type=int, default=0,
+                    help="decode shapes: separate copies of the weight that the steps take in turn "
+                         "(0: as many as exceed 512 MiB, so that no step finds its weight in a cache)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU; multi-GPU runs are not part of this build", file=sys.stderr)
@@ -173,6 +179,10 @@ def main():
 
     dev = "cuda:0"
     kind, M, K, N, n, m, g, desc = WORKLOADS[args.workload]
+    # Decode shapes are bound by the stream of the weight from HBM, and a weight of 18-54 MB
+    # would stay in the 256 MB memory-side cache between two steps: the steps take separate
+    # copies of it in turn, more than 512 MiB in all.
+    copies, turn = 1, [0]
     torch.manual_seed(0)
     W = (torch.randn(M, K) * 0.02).half().to(dev)
 
@@ -205,22 +215,30 @@ def main():
                 slin(X).backward(dY)
         algo_bytes = 0
     elif kind == "w4":
-        w = sten.SparseMarlinTensor.from_dense(W)
+        # int4 kept values + 2-bit positions + fp16 scales + activations + output
+        algo_bytes = M * K // 4 + M * K // 8 + (K // 128) * M * 2 + N * K * 2 + N * M * 2
+        copies = args.copies or -(-ROTATE_BYTES // algo_bytes)
+        ws = [sten.SparseMarlinTensor.from_dense(W) for _ in range(copies)]
         del W
         X = torch.randn(N, K).half().to(dev)
 
         def step():
-            return w.linear(X)
-        # int4 kept values + 2-bit positions + fp16 scales + activations + output
-        algo_bytes = M * K // 4 + M * K // 8 + (K // 128) * M * 2 + N * K * 2 + N * M * 2
+            turn[0] += 1
+            return ws[turn[0] % copies].linear(X)
     elif kind == "sparsify":
         def step():
             return sten.GroupedNMTensor.from_dense(W, n, m, sparse_dim=1, group_size=g, group_dim=0)
         w = step()
         algo_bytes = M * K * 2 + w.val.numel() * 2 + w.idx.numel() * 2
     else:
-        w = sten.GroupedNMTensor.from_dense(W, n, m, sparse_dim=1, group_size=g, group_dim=0)
-        w.spmm_opt["variant"] = args.variant
+        # weight values + one int16 index per (line, block) + activations + output
+        algo_bytes = M * K * n // m * 2 + M * K // m * 2 + N * K * 2 + N * M * 2
+        if kind == "decode":
+            copies = args.copies or -(-ROTATE_BYTES // algo_bytes)
+        ws = [sten.GroupedNMTensor.from_dense(W, n, m, sparse_dim=1, group_size=g, group_dim=0)
+              for _ in range(copies)]
+        for w in ws:
+            w.spmm_opt["variant"] = args.variant
         del W
         if kind == "grad_x":
             X = torch.randn(N, M).half().to(dev)      # upstream gradient dY [tokens, out features]
@@ -230,11 +248,11 @@ def main():
             rd = 1
 
         def step():
-            return sten.spmm(w, X, reduce_dim=rd, kernel=args.kernel)
-        # weight values + one int16 index per (line, block) + activations + output
-        algo_bytes = M * K * n // m * 2 + M * K // m * 2 + N * K * 2 + N * M * 2
+            turn[0] += 1
+            return sten.spmm(ws[turn[0] % copies], X, reduce_dim=rd, kernel=args.kernel)
 
-    for _ in range(args.warmup):
+    # every copy of the weight derives its kernel operands before anything is timed or captured
+    for _ in range(max(args.warmup, copies)):
         step()
     torch.cuda.synchronize()
 
@@ -298,7 +316,7 @@ def main():
             "metric": "nmg sparsifier GB/s" if kind == "sparsify" else "nmg sparse x dense decode GB/s",
             "value": algo_bytes / wall / 1e9, "unit": "GB/s",
             "config": {"workload": desc, "kernel": args.kernel, "launch": launch, "kernel_ms": kern_ms,
-                       "algorithmic_bytes": algo_bytes},
+                       "algorithmic_bytes": algo_bytes, "weight_copies": copies},
             "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": achieved / PEAK_HBM_GBS, "traffic": committed_traffic(args.workload)},
         })

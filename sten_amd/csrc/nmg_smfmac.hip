@@ -908,19 +908,27 @@ template <typename T, int NW, int UN> static int launch_smfmac_skinny(SmfParams 
 // Chunk = 2 k pairs (128 dense positions): ND DMA loads (4 token rows each) + 6 weight loads.
 // One chunk is in flight while the previous one is multiplied.  16-byte pieces of a row are
 // XOR-swizzled with the row number so that the 16 rows of a fragment read hit distinct banks.
-template <typename T, int SK_NW, int ND>
+// A weight of few blocks (4096 lines: 128) would leave half of the CUs without a workgroup:
+// SPLIT workgroups share a block, each fetches the runs of its 32 / SPLIT lines of every
+// fragment and multiplies zeros in the other lanes -- no sum across workgroups is needed.
+template <typename T, int SK_NW, int ND, int SPLIT>
 __global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_decode_staged_kernel(SmfParams P)
 {
     using S = Smf<T>;
     constexpr int OPS = ND + 6;
+    constexpr int LPB = 32 / SPLIT;                     // lines of the block that this workgroup owns
     constexpr int BUF = 16 * 256;                       // one chunk: 16 token rows x 256 bytes
     extern __shared__ __align__(16) unsigned char smem[];
     static_assert(SK_NW * 2 * BUF >= SK_NW * 32 * 17 * 4, "the reduction buffer reuses the staging area");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int mb = blockIdx.x;
+    const int mb = blockIdx.x / SPLIT, part = blockIdx.x % SPLIT;
     const int KP = P.KP;
     const int j = lane & 31, h = lane >> 5;
+    // The lanes of this workgroup's lines fetch their share of a fragment (a run of 16 * LPB
+    // bytes in each half of it); the other lanes repeat those addresses and multiply zeros.
+    const bool mine = (j / LPB) == part;
+    const int src_lane = (lane & 32) | (part * LPB + (j & (LPB - 1)));
     // an even number of k pairs per wavefront: chunks never straddle two ranges (KP is even)
     const int per = (((KP + SK_NW - 1) / SK_NW) + 1) & ~1;
     const int kp_lo = wave * per, kp_hi = min(KP, kp_lo + per);
@@ -932,7 +940,7 @@ __global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_decode_staged_kernel(S
 
     const unsigned char *aval = (const unsigned char *)P.fp_val + ((int64_t)mb * KP * 2) * 1024;
     const unsigned char *aidx = (const unsigned char *)P.fp_idx + ((int64_t)mb * KP) * 256;
-    const uint32_t lane16 = lane * 16, lane4 = lane * 4;
+    const uint32_t lane16 = src_lane * 16, lane4 = src_lane * 4;
     // DMA source of lane l in load i: token row 4i + l/16 (clamped: surplus rows repeat the last
     // token and are never stored), logical 16-byte piece (l%16) ^ row
     uint32_t x_off[ND];
@@ -958,17 +966,20 @@ __global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_decode_staged_kernel(S
         uint32_t ix[2];
     };
     ASet as[2];
-    // Loads of the chunk that starts at k pair kp0 (clamped into the operand when it lies beyond
-    // the wavefront's range: the count of operations stays uniform, the data is zeroed later).
-    auto issue = [&](int kp0, unsigned char *buf, ASet &A) {
-        const int kpc = min(kp0, KP - 2 >= 0 ? KP - 2 : 0);
-        const unsigned char *xb = (const unsigned char *)P.x + (int64_t)kpc * 128;
+    // Loads of the chunk that starts at k pair kp0.  Beyond the wavefront's range they repeat its
+    // last chunk (just fetched: no traffic to HBM), so the count of operations stays uniform;
+    // the data is zeroed later.
+    const int kp_last = max(kp_hi - 2, 0);
+    auto issue_x = [&](int kp0, unsigned char *buf) {
+        const unsigned char *xb = (const unsigned char *)P.x + (int64_t)min(kp0, kp_last) * 128;
 #pragma unroll
         for (int i = 0; i < ND; i++)
             __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[i]), (lds_ptr_t)(buf + i * 1024), 16, 0, 0);
+    };
+    auto issue_w = [&](int kp0, ASet &A) {
 #pragma unroll
         for (int kl = 0; kl < 2; kl++) {
-            const int kp = min(kp0 + kl, KP - 1);
+            const int kp = min(kp0, kp_last) + kl;
             const unsigned char *av = aval + (int64_t)kp * 2048;
             const unsigned char *ai = aidx + (int64_t)kp * 256;
             asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(A.a[kl][0]) : "v"(lane16), "s"(av) : "memory");
@@ -988,7 +999,7 @@ __global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_decode_staged_kernel(S
         for (int kl = 0; kl < 2; kl++) {
             // k pairs beyond the wavefront's range (or, when K is not a multiple of 128, beyond the
             // chunk's real extent) contribute nothing: their weights are replaced by zeros
-            const bool live = kp0 + kl < kp_hi;
+            const bool live = kp0 + kl < kp_hi && (SPLIT == 1 || mine);
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
                 union {
@@ -1011,16 +1022,19 @@ __global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_decode_staged_kernel(S
         }
     };
 
-    issue(kp_lo, stage, as[0]);
+    issue_x(kp_lo, stage);
+    issue_w(kp_lo, as[0]);
     for (int kp0 = kp_lo; kp0 < kp_hi; kp0 += 4) {
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             const int kc = kp0 + 2 * u;
+            if (kc >= kp_hi) break;
             // (the other buffer was read out before the MFMAs of the previous chunk)
-            issue(kc + 2, stage + ((u + 1) & 1) * BUF, as[(u + 1) & 1]);
+            issue_x(kc + 2, stage + ((u + 1) & 1) * BUF);
+            issue_w(kc + 2, as[(u + 1) & 1]);
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(OPS) : "memory");   // chunk kc has landed
             __builtin_amdgcn_sched_barrier(0);
-            consume(kc, stage + u * BUF, as[u]);
+            consume(kc, stage + (u & 1) * BUF, as[u]);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -1033,8 +1047,8 @@ __global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_decode_staged_kernel(S
         for (int r = 0; r < 16; r++) red[wave][(r >> 2) * 8 + h * 4 + (r & 3)][j] = acc[r];
     }
     __syncthreads();
-    for (int e = tid; e < 32 * 16; e += 64 * SK_NW) {
-        const int line = e & 31, tok = e >> 5;
+    for (int e = tid; e < LPB * 16; e += 64 * SK_NW) {
+        const int line = part * LPB + (e & (LPB - 1)), tok = e / LPB;
         const int64_t f = (int64_t)mb * 32 + line;
         if (tok >= P.T || f >= P.M) continue;
         float s = 0.f;
@@ -1045,11 +1059,12 @@ __global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_decode_staged_kernel(S
     }
 }
 
-template <typename T, int NW, int ND> static int launch_smfmac_decode_staged(SmfParams &P, hipStream_t s)
+template <typename T, int NW, int ND, int SPLIT>
+static int launch_smfmac_decode_staged(SmfParams &P, hipStream_t s)
 {
-    dim3 grid((unsigned)((P.M + 31) / 32));
+    dim3 grid((unsigned)((P.M + 31) / 32 * SPLIT));
     const size_t lds = (size_t)NW * 2 * 16 * 256;
-    auto k = spmm_smfmac_decode_staged_kernel<T, NW, ND>;
+    auto k = spmm_smfmac_decode_staged_kernel<T, NW, ND, SPLIT>;
     if (lds > 64 * 1024)
         NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(k, grid, dim3(64 * NW), lds, s, P);
@@ -1057,13 +1072,14 @@ template <typename T, int NW, int ND> static int launch_smfmac_decode_staged(Smf
     return NMG_OK;
 }
 
-template <typename T, int NW> static int launch_smfmac_decode_staged_nd(SmfParams &P, hipStream_t s)
+template <typename T, int NW, int SPLIT = 1>
+static int launch_smfmac_decode_staged_nd(SmfParams &P, hipStream_t s)
 {
     switch ((int)(P.T + 3) / 4) {
-    case 1: return launch_smfmac_decode_staged<T, NW, 1>(P, s);
-    case 2: return launch_smfmac_decode_staged<T, NW, 2>(P, s);
-    case 3: return launch_smfmac_decode_staged<T, NW, 3>(P, s);
-    default: return launch_smfmac_decode_staged<T, NW, 4>(P, s);
+    case 1: return launch_smfmac_decode_staged<T, NW, 1, SPLIT>(P, s);
+    case 2: return launch_smfmac_decode_staged<T, NW, 2, SPLIT>(P, s);
+    case 3: return launch_smfmac_decode_staged<T, NW, 3, SPLIT>(P, s);
+    default: return launch_smfmac_decode_staged<T, NW, 4, SPLIT>(P, s);
     }
 }
 
@@ -1251,8 +1267,14 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
         // many line blocks: small workgroups pack several per CU and balance better
         // reduction extents that are a multiple of 128: activations staged through LDS
         if (P.K % 128 == 0 && P.T * P.ldx * 2 < ((int64_t)1 << 31)) {
-            if ((P.M + 31) / 32 >= 256) return launch_smfmac_decode_staged_nd<T, 4>(P, s);
-            return launch_smfmac_decode_staged_nd<T, 16>(P, s);
+            // Weights that are not in a cache, 4096 x 11008 (128 blocks), 1 / 16 tokens: one
+            // workgroup of 16 wavefronts per block 13.2 / 18.4 us, two of 8 wavefronts 12.1 / 15.5,
+            // two of 16 12.2 / 16.7, four of 4 16.2 / 22.9 (runs of 128 bytes).  11008 x 4096
+            // (344 blocks): one of 4 wavefronts 11.6 / 14.0, two of 4 12.1 / 16.2.
+            const int64_t blocks = (P.M + 31) / 32;
+            if (blocks >= 256) return launch_smfmac_decode_staged_nd<T, 4, 1>(P, s);
+            if (blocks >= 64) return launch_smfmac_decode_staged_nd<T, 8, 2>(P, s);
+            return launch_smfmac_decode_staged_nd<T, 16, 2>(P, s);
         }
         if ((P.M + 31) / 32 >= 256) return launch_smfmac_skinny<T, 4, 4>(P, s);
         return launch_smfmac_skinny<T, 16, 1>(P, s);
