@@ -114,11 +114,13 @@ __global__ __launch_bounds__(256) void w4_pack_kernel(W4Params P)
 }
 
 // 8 nibbles of one instruction -> 8 fp16 weights: (1024 + q) - 1032 = q - 8 exactly, then one
-// rounding in the product with the scale.
+// rounding in the product with the scale.  A nibble at bits 4..7 of a half is read in place
+// under the exponent of 64, where the last mantissa place is 1/16: (64 + q) - 72.
 __device__ __forceinline__ u32x4 w4_dequant(uint32_t word, w4_f16x2 s2)
 {
     u32x4 out;
-    const w4_f16x2 off = {(_Float16)1032.0f, (_Float16)1032.0f};
+    const w4_f16x2 off_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
+    const w4_f16x2 off_hi = {(_Float16)72.0f, (_Float16)72.0f};
     uint32_t o[4];
 #pragma unroll
     for (int t = 0; t < 4; t++) {
@@ -126,8 +128,16 @@ __device__ __forceinline__ u32x4 w4_dequant(uint32_t word, w4_f16x2 s2)
             uint32_t u;
             w4_f16x2 h;
         } c;
-        c.u = ((word >> (4 * t)) & 0x000F000Fu) | 0x64006400u;
-        c.h = (c.h - off) * s2;
+        const uint32_t w = t < 2 ? word : word >> 8;
+        // (w & mask) | exponent in one instruction (two literals do not fit one: the mask comes
+        // in a register)
+        if (t & 1) {
+            asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(c.u) : "v"(w), "v"(0x00F000F0u), "s"(0x54005400u));
+            c.h = (c.h - off_hi) * s2;
+        } else {
+            asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(c.u) : "v"(w), "v"(0x000F000Fu), "s"(0x64006400u));
+            c.h = (c.h - off_lo) * s2;
+        }
         o[t] = c.u;
     }
     out.x = o[0];
