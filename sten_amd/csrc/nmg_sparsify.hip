@@ -1221,10 +1221,10 @@ template <typename T> static int dispatch_sparsify(SparsifyParams &P, hipStream_
     // Tiles of at least 16 columns: batched rounds, with as many lanes per tile as its later
     // rounds keep busy -- a quarter, a half or a whole wavefront (several tiles share the
     // wavefront's instruction stream), else a workgroup.  Measured on 4096 x 4096 fp16, 2:4 with
-    // g = 4 / 8 / 16 / 32 / 64: 208 / 147 / 142 / 147 / 161 us against 320 / 407 / 402 / 742 / 1204 us
+    // g = 4 / 8 / 16 / 32 / 64: 182 / 125 / 125 / 130 / 141 us against 320 / 407 / 402 / 742 / 1204 us
     // for the lane teams below; 8192 x 8192, 1:8:32 / 2:8:32 / 4:8:32: 0.39 / 0.92 / 2.1 ms against
     // 2.6 / 10.9 / 56 ms for the step-by-step kernels.  Half a wavefront loses to a whole one from
-    // about 20 patterns on (2:8:4, 112 columns: 430 against 367 us); tiles of fewer than 16 columns
+    // about 20 patterns on (2:8:4, 112 columns: 430 against 324 us); tiles of fewer than 16 columns
     // stay with the lane teams (2:4:2: 200 against 315 us).  A tile's rounds are a chain of
     // barriers and LDS round trips, so what counts is how many tiles a CU holds at once (34 bytes
     // of LDS per column): 2240-column tiles (4:8:32) take 2.1 ms with 512 threads, two tiles per
