@@ -21,6 +21,7 @@
 #include "nmg_common.h"
 #include "nmg_tile.h"
 
+#include <algorithm>
 #include <type_traits>
 
 namespace nmg {
@@ -57,6 +58,11 @@ struct SmfParams {
     int64_t M, K, T, ldx, ldy;
     int MB, KP;          // feature blocks of 32, k pairs of 64
     int tiles_m, tiles_n;
+    // direct kernel with the reduction cut into slices (0 / 1: whole): slice s of a tile writes
+    // its sums in single precision to part[s][token][feature], part_ld features per token
+    int ksplit;
+    float *part;
+    int64_t part_ld;
 };
 
 constexpr int SMF_ROW = 144;  // bytes per token row in LDS: 64 k * 2 B + 16 B pad (conflict-free b128 reads)
@@ -540,6 +546,9 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
 
     int id = blockIdx.x;
     const int ntiles = P.tiles_m * P.tiles_n;
+    // slices of the reduction: the slices of a tile are workgroups ntiles apart
+    const int slice = P.ksplit > 1 ? id / ntiles : 0;
+    id -= slice * ntiles;
     if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
     constexpr int GH = 4;
     const int band = id / (GH * P.tiles_n);
@@ -547,7 +556,11 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
     const int in_band = id - band * GH * P.tiles_n;
     const int tile_m = band * GH + in_band % band_h, tile_n = in_band / band_h;
     const int64_t f0 = (int64_t)tile_m * TF, t0 = (int64_t)tile_n * TT;
-    const int KP = P.KP, KS = KP * 2;
+    // k pairs kp_lo .. kp_lo + KP - 1 of the operand's KPT (the host leaves no slice empty)
+    const int KPT = P.KP;
+    const int kp_per = P.ksplit > 1 ? (KPT + P.ksplit - 1) / P.ksplit : KPT;
+    const int kp_lo = slice * kp_per;
+    const int KP = min(KPT, kp_lo + kp_per) - kp_lo;
     const int wm = wave / WN, wn = wave % WN;
     const int mb0 = (int)(f0 / 32) + wm * FB;
 
@@ -557,11 +570,11 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
     const unsigned char *ai_base[FB];
 #pragma unroll
     for (int fb = 0; fb < FB; fb++) {
-        av_base[fb] = (const unsigned char *)P.fp_val + ((int64_t)(mb0 + fb) * KS) * 1024;
-        ai_base[fb] = (const unsigned char *)P.fp_idx + ((int64_t)(mb0 + fb) * KP) * 256;
+        av_base[fb] = (const unsigned char *)P.fp_val + (((int64_t)(mb0 + fb) * KPT + kp_lo) * 2) * 1024;
+        ai_base[fb] = (const unsigned char *)P.fp_idx + ((int64_t)(mb0 + fb) * KPT + kp_lo) * 256;
     }
     const uint32_t lane16 = lane * 16, lane4 = lane * 4;
-    const unsigned char *x_base = (const unsigned char *)P.x;
+    const unsigned char *x_base = (const unsigned char *)P.x + (int64_t)kp_lo * 128;
     uint32_t x_off[XL];
 #pragma unroll
     for (int i = 0; i < XL; i++) {
@@ -759,9 +772,57 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
     pin_acc();
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     asm volatile("s_barrier" ::: "memory");
+    if (P.ksplit > 1) {
+        // the slice's sums as they are: a lane holds token j and features 8*(r/4) + 4*h + r%4, four
+        // consecutive features are one 16-byte store (part_ld covers the padded features)
+        float *part = P.part + (int64_t)slice * P.T * P.part_ld;
+#pragma unroll
+        for (int tb = 0; tb < TB; tb++) {
+            const int64_t tok = t0 + (wn * TB + tb) * 32 + j;
+            if (tok >= P.T) continue;
+#pragma unroll
+            for (int fb = 0; fb < FB; fb++)
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) {
+                    const int64_t f = f0 + (wm * FB + fb) * 32 + rq * 8 + h * 4;
+                    float4 v;
+                    v.x = acc[fb][tb][rq * 4 + 0];
+                    v.y = acc[fb][tb][rq * 4 + 1];
+                    v.z = acc[fb][tb][rq * 4 + 2];
+                    v.w = acc[fb][tb][rq * 4 + 3];
+                    *(float4 *)(part + tok * P.part_ld + f) = v;
+                }
+        }
+        return;
+    }
     const TileOut out{P.y, P.bias, P.M, P.T, P.ldy};
     smf_store_tile<T, FB, TB>(acc, smem + wave * (TB * 32 * (FB * 64 + 16)), lane, f0 + wm * FB * 32,
                               t0 + wn * TB * 32, out);
+}
+
+// Sum of the slices of a split reduction: y[token][feature] = sum over s of part[s][token][feature]
+// (+ bias), in slice order, rounded once.  One thread per four features.
+template <typename T> __global__ __launch_bounds__(256) void splitk_sum_kernel(SmfParams P)
+{
+    const int64_t quads = (P.M + 3) / 4;
+    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= P.T * quads) return;
+    const int64_t tok = gid / quads, f = (gid - tok * quads) * 4;
+    const float *src = P.part + tok * P.part_ld + f;
+    float4 sum = *(const float4 *)src;
+    for (int sl = 1; sl < P.ksplit; sl++) {
+        const float4 v = *(const float4 *)(src + (int64_t)sl * P.T * P.part_ld);
+        sum.x += v.x;
+        sum.y += v.y;
+        sum.z += v.z;
+        sum.w += v.w;
+    }
+    const float o[4] = {sum.x, sum.y, sum.z, sum.w};
+    uint16_t *dst = (uint16_t *)P.y + tok * P.ldy + f;
+    const T *bias = (const T *)P.bias;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (f + i < P.M) dst[i] = f32_to_bits16(o[i] + (bias ? to_f32(bias[f + i]) : 0.f), (T *)nullptr);
 }
 
 template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_smfmac_direct(SmfParams &P, hipStream_t s)
@@ -770,7 +831,8 @@ template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_
     static_assert(TF == 256, "the operand is padded to 256 lines");
     P.tiles_m = (int)((P.M + TF - 1) / TF);
     P.tiles_n = (int)((P.T + TT - 1) / TT);
-    dim3 grid((unsigned)(P.tiles_m * P.tiles_n));
+    const int slices = P.ksplit > 1 ? P.ksplit : 1;
+    dim3 grid((unsigned)(P.tiles_m * P.tiles_n * slices));
     constexpr size_t ring = (size_t)DR_NS * TT * 128, stg = (size_t)4 * TB * 32 * (FB * 64 + 16);
     constexpr size_t lds = ring > stg ? ring : stg;
     static_assert(lds <= 160 * 1024, "LDS");
@@ -778,6 +840,11 @@ template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_
     NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(k, grid, dim3(256), lds, s, P);
     NMG_HIP_TRY(hipGetLastError());
+    if (slices > 1) {
+        const int64_t threads = P.T * ((P.M + 3) / 4);
+        hipLaunchKernelGGL(splitk_sum_kernel<T>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, P);
+        NMG_HIP_TRY(hipGetLastError());
+    }
     return NMG_OK;
 }
 
@@ -1321,4 +1388,77 @@ extern "C" int nmg_spmm_smfmac(const void *d_fp_val, const void *d_fp_idx, int64
     hipStream_t s = (hipStream_t)stream;
     return dtype == NMG_F16 ? launch_smfmac<__half>(P, variant, s)
                             : launch_smfmac<__hip_bfloat16>(P, variant, s);
+}
+
+// Largest number of reduction slices that leaves none empty: slices of ceil(KP / S) k pairs.
+static int splitk_fit(int64_t KP, int64_t S)
+{
+    while (S > 1 && (S - 1) * ((KP + S - 1) / S) >= KP) S--;
+    return (int)(S < 1 ? 1 : S);
+}
+
+extern "C" int nmg_spmm_smfmac_splitk_plan(int64_t M, int64_t K, int64_t T, int *slices,
+                                           int64_t *workspace_bytes)
+{
+    NMG_REQUIRE(M >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
+    NMG_REQUIRE(slices && workspace_bytes, NMG_ERR_ARG, "null output pointer");
+    const int64_t tiles_m = (M + 255) / 256, tiles = tiles_m * ((T + 127) / 128), KP = (K + 63) / 64;
+    int S = 1;
+    // Between the decode shapes and a batch that fills the chip a product has fewer tiles of
+    // 256 x 128 than the GPU has CUs, and every workgroup walks the whole reduction: the slices
+    // bring the workgroups towards one per CU, at eight K steps or more each and at most eight
+    // slices (sixteen for a handful of tiles): every slice writes and the sum reads a tile in
+    // single precision.  4096 x 11008 2:4 on 17 / 64 / 128 / 256 / 512 / 1024 tokens: 58 / 58 / 64 /
+    // 65 / 72 / 94 us whole, 20 / 20 / 25 / 33 / 42 / 67 us in 8 / 8 / 8 / 8 / 4 / 2 slices (16 slices
+    // at 64 tokens: 22 us).
+    if (T > 16 && K % 64 == 0 && tiles > 0 && tiles <= 128)
+        S = splitk_fit(KP, std::min<int64_t>(std::min<int64_t>(256 / tiles, tiles <= 8 ? 16 : 8), KP / 8));
+    *slices = S;
+    *workspace_bytes = S > 1 ? (int64_t)S * T * tiles_m * 256 * 4 : 0;
+    return NMG_OK;
+}
+
+extern "C" int nmg_spmm_smfmac_splitk(const void *d_fp_val, const void *d_fp_idx, int64_t M, int64_t K,
+                                      const void *d_x, int64_t ldx, void *d_y, int64_t ldy,
+                                      const void *d_bias, int64_t T, int dtype, int slices,
+                                      void *d_workspace, int64_t workspace_bytes, void *stream)
+{
+    if (slices <= 1)
+        return nmg_spmm_smfmac(d_fp_val, d_fp_idx, M, K, d_x, ldx, d_y, ldy, d_bias, T, dtype, -1, stream);
+    NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED,
+                "the sparse matrix cores take f16/bf16 only");
+    NMG_REQUIRE(M >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
+    NMG_REQUIRE(ldx >= K && ldy >= M, NMG_ERR_ARG, "leading dimension smaller than row length");
+    NMG_REQUIRE((K % 64) == 0 && (ldx % 8) == 0 && ((uintptr_t)d_x % 16) == 0, NMG_ERR_UNSUPPORTED,
+                "a split reduction needs K % 64 == 0 and 16-byte aligned activations");
+    NMG_REQUIRE(T > 16 && T * ldx * 2 < ((int64_t)1 << 31), NMG_ERR_UNSUPPORTED,
+                "a split reduction takes more than 16 tokens and activations below 2 GiB");
+    if (M == 0 || K == 0) return NMG_OK;
+    const int64_t KP = K / 64, tiles_m = (M + 255) / 256;
+    NMG_REQUIRE(slices <= 256 && splitk_fit(KP, slices) == slices, NMG_ERR_ARG,
+                "%d slices leave one empty (%lld K steps)", slices, (long long)KP);
+    const int64_t need = (int64_t)slices * T * tiles_m * 256 * 4;
+    NMG_REQUIRE(d_workspace && workspace_bytes >= need && ((uintptr_t)d_workspace % 16) == 0, NMG_ERR_ARG,
+                "workspace of %lld bytes (16-byte aligned) needed, %lld given", (long long)need,
+                (long long)workspace_bytes);
+    NMG_REQUIRE(d_fp_val && d_fp_idx && d_x && d_y, NMG_ERR_ARG, "null device pointer");
+    SmfParams P{};
+    P.fp_val = d_fp_val;
+    P.fp_idx = (const uint32_t *)d_fp_idx;
+    P.x = d_x;
+    P.y = d_y;
+    P.bias = d_bias;
+    P.M = M;
+    P.K = K;
+    P.T = T;
+    P.ldx = ldx;
+    P.ldy = ldy;
+    P.MB = (int)(tiles_m * 8);
+    P.KP = (int)KP;
+    P.ksplit = slices;
+    P.part = (float *)d_workspace;
+    P.part_ld = tiles_m * 256;
+    hipStream_t s = (hipStream_t)stream;
+    return dtype == NMG_F16 ? launch_smfmac_direct<__half, 2, 4, 4, 1, 2>(P, s)
+                            : launch_smfmac_direct<__hip_bfloat16, 2, 4, 4, 1, 2>(P, s);
 }

@@ -303,6 +303,21 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
     if packed is not None:
         if T <= 16 and kname in ("auto", "skinny"):
             variant = 5                 # decode shapes: streaming kernel on the same operand
+        lib = native.load()
+        if T > 16 and variant == -1 and K % 64 == 0 and T * x.stride(0) * 2 < 2 ** 31:
+            # few tiles for the chip: the reduction is cut into slices, summed by a second kernel
+            slices, ws_bytes = ctypes.c_int(1), ctypes.c_int64(0)
+            native.check(lib.nmg_spmm_smfmac_splitk_plan(O, K, T, ctypes.byref(slices), ctypes.byref(ws_bytes)))
+            slices = int(weight.spmm_opt.get("slices", slices.value))
+            if slices > 1:
+                tiles_m = (O + 255) // 256
+                ws = torch.empty((slices * T * tiles_m * 256,), dtype=torch.float32, device=x.device)
+                with torch.cuda.device(x.device):
+                    native.check(lib.nmg_spmm_smfmac_splitk(
+                        native.ptr(packed[0]), native.ptr(packed[1]), O, K, native.ptr(x), x.stride(0),
+                        native.ptr(y), O, native.ptr(bias), T, native.dtype_code(x.dtype), slices,
+                        native.ptr(ws), ws.numel() * 4, native.stream_ptr(x.device)))
+                return y
         with torch.cuda.device(x.device):
             native.check(native.load().nmg_spmm_smfmac(
                 native.ptr(packed[0]), native.ptr(packed[1]), O, K, native.ptr(x),

@@ -53,6 +53,23 @@ def test_argument_errors_need_no_gpu():
     assert lib.nmg_spmm(one, one, 8, 8, one, 4, one, 8, None, 4, 1, 2, 4, native.NMG_F16, 0, None) == 1
 
 
+def test_split_reduction_plan_and_argument_errors():
+    lib = native.load()
+    slices, ws = ctypes.c_int(0), ctypes.c_int64(0)
+    plan = lambda M, K, T: (lib.nmg_spmm_smfmac_splitk_plan(M, K, T, ctypes.byref(slices), ctypes.byref(ws)),
+                            slices.value, ws.value)
+    assert plan(4096, 11008, 64) == (0, 8, 8 * 64 * 4096 * 4)         # 16 tiles -> 8 slices of 22 K steps
+    assert plan(4096, 11008, 512) == (0, 4, 4 * 512 * 4096 * 4)
+    assert plan(4096, 11008, 16) == (0, 1, 0)                         # decode shapes are not split
+    assert plan(4096, 11008, 2048) == (0, 1, 0)                       # enough tiles
+    assert plan(4096, 200, 64) == (0, 1, 0)                           # K % 64 != 0
+    assert plan(1000, 256, 64)[1] == 1                                # four K steps: too short to cut
+    one = ctypes.c_void_p(16)  # never dereferenced: validation fails first
+    args = lambda sl, wsb: (one, one, 512, 1152, one, 1152, one, 512, None, 40, native.NMG_F16, sl, one, wsb, None)
+    assert lib.nmg_spmm_smfmac_splitk(*args(17, 1 << 30)) == 1 and b"empty" in lib.nmg_last_error()
+    assert lib.nmg_spmm_smfmac_splitk(*args(2, 100)) == 1 and b"workspace" in lib.nmg_last_error()
+
+
 def test_cpu_tensors_are_refused_loudly():
     import torch
     import sten_amd as sten

@@ -3,6 +3,7 @@ Oracle: the equation the reference asserts, C == to_dense(A) @ B (dace_gnm_mult.
 evaluated in fp64 from the oracle's own val/idx, plus the CPU restatement of the reference kernel.
 Tolerances: rel-L2 <= 1e-3 for 16-bit inputs with fp32 accumulation, <= 1e-5 for fp32."""
 import copy
+import ctypes
 import warnings
 
 import numpy as np
@@ -10,6 +11,7 @@ import pytest
 import torch
 
 import sten_amd as sten
+from sten_amd import native
 from oracle import nmg_oracle as O
 from helpers import oracle_sparsify, rel_l2, seeded, to_np
 
@@ -216,6 +218,47 @@ def test_spmm_sparse_matrix_cores(variant, dtype, M, K, T, n, m, g):
     assert rel_l2(to_np(y), ref) <= TOL[dtype]
     y2 = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1, kernel="mfma")
     assert rel_l2(to_np(y), to_np(y2)) <= 2 * TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,K,T,n,m,g,slices", [
+    (512, 1152, 40, 2, 4, 16, None),     # planned: 2 tiles, 18 K steps -> 2 slices
+    (512, 1152, 129, 2, 4, 16, 3),       # two token tiles, uneven slices (6 + 6 + 6)
+    (1000, 2048, 200, 2, 4, 8, 7),       # ragged lines and tokens, slices of 5, 5, ..., 2
+    (300, 704, 17, 1, 4, 4, 11),         # one K step per slice
+    (2048, 4096, 64, 2, 8, 32, None),    # 2:8 in 2-of-4 slots, planned
+])
+def test_split_reduction_matches_dense(dtype, M, K, T, n, m, g, slices):
+    print(f"case split-K {dtype} M={M} K={K} T={T} {n}:{m}:{g} slices={slices}", flush=True)
+    W = seeded((M, K), dtype, seed=M + K + T, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, 1)
+    w = make(W, n, m, g, 1)
+    if slices is not None:
+        w.spmm_opt["slices"] = slices
+    else:
+        planned, ws = ctypes.c_int(0), ctypes.c_int64(0)
+        assert native.load().nmg_spmm_smfmac_splitk_plan(M, K, T, ctypes.byref(planned), ctypes.byref(ws)) == 0
+        assert planned.value > 1 and ws.value == planned.value * T * ((M + 255) // 256) * 256 * 4
+    x = seeded((T, K), dtype, seed=1)
+    b = seeded((M,), dtype, seed=2)
+    for bias in (None, b.to(DEV)):
+        y = sten.spmm(w, x.to(DEV), bias, reduce_dim=1)
+        ref = to_np(x).astype(np.float64) @ Wd.T + (0 if bias is None else to_np(b).astype(np.float64))
+        assert rel_l2(to_np(y), ref) <= TOL[dtype]
+    w.spmm_opt["slices"] = 1                      # the same product on whole reductions
+    y1 = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)
+    assert rel_l2(to_np(y), to_np(y1)) <= 2 * TOL[dtype]
+
+
+def test_split_reduction_on_the_target_weight_at_intermediate_batches():
+    torch.manual_seed(0)
+    W = (torch.randn(4096, 11008) * 0.02).half()
+    w = make(W, 2, 4, 16, 1)
+    Wd = w.to_dense().double()
+    for T in (17, 128, 500):
+        x = torch.randn(T, 11008, dtype=torch.float16, device=DEV)
+        y = sten.spmm(w, x, reduce_dim=1)
+        assert rel_l2(to_np(y), to_np(x.double() @ Wd.t())) <= TOL[torch.float16]
 
 
 def test_sparse_matrix_cores_refuse_incompatible_patterns():
