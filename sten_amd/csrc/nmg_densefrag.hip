@@ -112,6 +112,11 @@ struct DfParams {
     int64_t O, K, T, ldx, ldy;
     int KP;              // K steps of 64
     int tiles_m, tiles_n;
+    // reduction cut into slices (0 / 1: whole): slice s of a tile stores its sums in single
+    // precision at part[s][token][output], part_ld outputs per token
+    int ksplit;
+    float *part;
+    int64_t part_ld;
 };
 
 constexpr int DD_D = 2;    // K steps in flight (a dense K step takes twice the MFMA time of a sparse one)
@@ -146,6 +151,9 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
     // a compact block of tiles whose weights and activations stay in that XCD's L2.
     int id = blockIdx.x;
     const int ntiles = P.tiles_m * P.tiles_n;
+    // slices of the reduction: the slices of a tile are workgroups ntiles apart
+    const int slice = P.ksplit > 1 ? id / ntiles : 0;
+    id -= slice * ntiles;
     if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
     constexpr int GH = 4;
     const int band = id / (GH * P.tiles_n);
@@ -153,7 +161,11 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
     const int in_band = id - band * GH * P.tiles_n;
     const int tile_m = band * GH + in_band % band_h, tile_n = in_band / band_h;
     const int64_t f0 = (int64_t)tile_m * TF, t0 = (int64_t)tile_n * TT;
-    const int KP = P.KP;
+    // K steps kp_lo .. kp_lo + KP - 1 of the operand's KPT (the host leaves no slice empty)
+    const int KPT = P.KP;
+    const int kp_per = P.ksplit > 1 ? (KPT + P.ksplit - 1) / P.ksplit : KPT;
+    const int kp_lo = slice * kp_per;
+    const int KP = min(KPT, kp_lo + kp_per) - kp_lo;
     const int wm = wave / WN, wn = wave % WN;
     const int ob0 = (int)(f0 / 32) + wm * FB;
 
@@ -162,9 +174,9 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
     const unsigned char *av_base[FB];
 #pragma unroll
     for (int fb = 0; fb < FB; fb++)
-        av_base[fb] = (const unsigned char *)P.df + ((int64_t)(ob0 + fb) * KP * 4) * 1024;
+        av_base[fb] = (const unsigned char *)P.df + (((int64_t)(ob0 + fb) * KPT + kp_lo) * 4) * 1024;
     const uint32_t lane16 = lane * 16;
-    const unsigned char *x_base = (const unsigned char *)P.x;
+    const unsigned char *x_base = (const unsigned char *)P.x + (int64_t)kp_lo * 128;
     uint32_t x_off[XL];
 #pragma unroll
     for (int i = 0; i < XL; i++) {
@@ -369,6 +381,11 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
     pin_acc();
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     asm volatile("s_barrier" ::: "memory");
+    if (P.ksplit > 1) {
+        store_partial_tile<FB, TB>(acc, P.part + (int64_t)slice * P.T * P.part_ld, P.part_ld, lane,
+                                   f0 + wm * FB * 32, t0 + wn * TB * 32, P.T);
+        return;
+    }
     const TileOut out{P.y, P.bias, P.O, P.T, P.ldy};
     smf_store_tile<T, FB, TB>(acc, smem + wave * (TB * 32 * (FB * 64 + 16)), lane, f0 + wm * FB * 32,
                               t0 + wn * TB * 32, out);
@@ -380,7 +397,8 @@ template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_
     static_assert(TF == 256, "the operand is padded to 256 outputs");
     P.tiles_m = (int)((P.O + TF - 1) / TF);
     P.tiles_n = (int)((P.T + TT - 1) / TT);
-    dim3 grid((unsigned)(P.tiles_m * P.tiles_n));
+    const int slices = P.ksplit > 1 ? P.ksplit : 1;
+    dim3 grid((unsigned)(P.tiles_m * P.tiles_n * slices));
     constexpr size_t ring = (size_t)DD_NS * TT * 128, stg = (size_t)4 * TB * 32 * (FB * 64 + 16);
     constexpr size_t lds = ring > stg ? ring : stg;
     static_assert(lds <= 160 * 1024, "LDS");
@@ -388,6 +406,10 @@ template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_
     NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(k, grid, dim3(256), lds, s, P);
     NMG_HIP_TRY(hipGetLastError());
+    if (slices > 1) {
+        const SplitSum Q{P.part, P.y, P.bias, P.O, P.T, P.ldy, P.part_ld, slices};
+        return launch_splitk_sum<T>(Q, s);
+    }
     return NMG_OK;
 }
 
@@ -489,4 +511,43 @@ extern "C" int nmg_spmm_densefrag(const void *d_df, int64_t O, int64_t K, const 
     P.KP = (int)(K / 64);
     hipStream_t s = (hipStream_t)stream;
     return dtype == NMG_F16 ? launch_dense<__half>(P, variant, s) : launch_dense<__hip_bfloat16>(P, variant, s);
+}
+
+extern "C" int nmg_spmm_densefrag_splitk(const void *d_df, int64_t O, int64_t K, const void *d_x, int64_t ldx,
+                                         void *d_y, int64_t ldy, const void *d_bias, int64_t T, int dtype,
+                                         int slices, void *d_workspace, int64_t workspace_bytes, void *stream)
+{
+    if (slices <= 1) return nmg_spmm_densefrag(d_df, O, K, d_x, ldx, d_y, ldy, d_bias, T, dtype, -1, stream);
+    NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED, "densefrag takes f16/bf16");
+    NMG_REQUIRE(O >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
+    NMG_REQUIRE(ldx >= K && ldy >= O, NMG_ERR_ARG, "leading dimension smaller than row length");
+    NMG_REQUIRE(K % 64 == 0 && K > 0 && ldx % 8 == 0 && ((uintptr_t)d_x % 16) == 0, NMG_ERR_UNSUPPORTED,
+                "needs K %% 64 == 0 and 16-byte aligned activation rows");
+    NMG_REQUIRE(T * ldx * 2 < ((int64_t)1 << 31), NMG_ERR_UNSUPPORTED, "activations must be smaller than 2 GiB");
+    if (O == 0 || T == 0) return NMG_OK;
+    const int64_t KP = K / 64, tiles_m = (O + 255) / 256;
+    NMG_REQUIRE(slices <= 256 && splitk_fit(KP, slices) == slices, NMG_ERR_ARG,
+                "%d slices leave one empty (%lld K steps)", slices, (long long)KP);
+    const int64_t need = (int64_t)slices * T * tiles_m * 256 * 4;
+    NMG_REQUIRE(d_workspace && workspace_bytes >= need && ((uintptr_t)d_workspace % 16) == 0, NMG_ERR_ARG,
+                "workspace of %lld bytes (16-byte aligned) needed, %lld given", (long long)need,
+                (long long)workspace_bytes);
+    NMG_REQUIRE(d_df && d_x && d_y, NMG_ERR_ARG, "null device pointer");
+    DfParams P{};
+    P.df = d_df;
+    P.x = d_x;
+    P.y = d_y;
+    P.bias = d_bias;
+    P.O = O;
+    P.K = K;
+    P.T = T;
+    P.ldx = ldx;
+    P.ldy = ldy;
+    P.KP = (int)KP;
+    P.ksplit = slices;
+    P.part = (float *)d_workspace;
+    P.part_ld = tiles_m * 256;
+    hipStream_t s = (hipStream_t)stream;
+    return dtype == NMG_F16 ? launch_dense_direct<__half, 2, 4, 4, 1, 1>(P, s)
+                            : launch_dense_direct<__hip_bfloat16, 2, 4, 4, 1, 1>(P, s);
 }

@@ -773,56 +773,13 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     asm volatile("s_barrier" ::: "memory");
     if (P.ksplit > 1) {
-        // the slice's sums as they are: a lane holds token j and features 8*(r/4) + 4*h + r%4, four
-        // consecutive features are one 16-byte store (part_ld covers the padded features)
-        float *part = P.part + (int64_t)slice * P.T * P.part_ld;
-#pragma unroll
-        for (int tb = 0; tb < TB; tb++) {
-            const int64_t tok = t0 + (wn * TB + tb) * 32 + j;
-            if (tok >= P.T) continue;
-#pragma unroll
-            for (int fb = 0; fb < FB; fb++)
-#pragma unroll
-                for (int rq = 0; rq < 4; rq++) {
-                    const int64_t f = f0 + (wm * FB + fb) * 32 + rq * 8 + h * 4;
-                    float4 v;
-                    v.x = acc[fb][tb][rq * 4 + 0];
-                    v.y = acc[fb][tb][rq * 4 + 1];
-                    v.z = acc[fb][tb][rq * 4 + 2];
-                    v.w = acc[fb][tb][rq * 4 + 3];
-                    *(float4 *)(part + tok * P.part_ld + f) = v;
-                }
-        }
+        store_partial_tile<FB, TB>(acc, P.part + (int64_t)slice * P.T * P.part_ld, P.part_ld, lane,
+                                   f0 + wm * FB * 32, t0 + wn * TB * 32, P.T);
         return;
     }
     const TileOut out{P.y, P.bias, P.M, P.T, P.ldy};
     smf_store_tile<T, FB, TB>(acc, smem + wave * (TB * 32 * (FB * 64 + 16)), lane, f0 + wm * FB * 32,
                               t0 + wn * TB * 32, out);
-}
-
-// Sum of the slices of a split reduction: y[token][feature] = sum over s of part[s][token][feature]
-// (+ bias), in slice order, rounded once.  One thread per four features.
-template <typename T> __global__ __launch_bounds__(256) void splitk_sum_kernel(SmfParams P)
-{
-    const int64_t quads = (P.M + 3) / 4;
-    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (gid >= P.T * quads) return;
-    const int64_t tok = gid / quads, f = (gid - tok * quads) * 4;
-    const float *src = P.part + tok * P.part_ld + f;
-    float4 sum = *(const float4 *)src;
-    for (int sl = 1; sl < P.ksplit; sl++) {
-        const float4 v = *(const float4 *)(src + (int64_t)sl * P.T * P.part_ld);
-        sum.x += v.x;
-        sum.y += v.y;
-        sum.z += v.z;
-        sum.w += v.w;
-    }
-    const float o[4] = {sum.x, sum.y, sum.z, sum.w};
-    uint16_t *dst = (uint16_t *)P.y + tok * P.ldy + f;
-    const T *bias = (const T *)P.bias;
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-        if (f + i < P.M) dst[i] = f32_to_bits16(o[i] + (bias ? to_f32(bias[f + i]) : 0.f), (T *)nullptr);
 }
 
 template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_smfmac_direct(SmfParams &P, hipStream_t s)
@@ -841,9 +798,8 @@ template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_
     hipLaunchKernelGGL(k, grid, dim3(256), lds, s, P);
     NMG_HIP_TRY(hipGetLastError());
     if (slices > 1) {
-        const int64_t threads = P.T * ((P.M + 3) / 4);
-        hipLaunchKernelGGL(splitk_sum_kernel<T>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, P);
-        NMG_HIP_TRY(hipGetLastError());
+        const SplitSum Q{P.part, P.y, P.bias, P.M, P.T, P.ldy, P.part_ld, slices};
+        return launch_splitk_sum<T>(Q, s);
     }
     return NMG_OK;
 }
@@ -1390,14 +1346,8 @@ extern "C" int nmg_spmm_smfmac(const void *d_fp_val, const void *d_fp_idx, int64
                             : launch_smfmac<__hip_bfloat16>(P, variant, s);
 }
 
-// Largest number of reduction slices that leaves none empty: slices of ceil(KP / S) k pairs.
-static int splitk_fit(int64_t KP, int64_t S)
-{
-    while (S > 1 && (S - 1) * ((KP + S - 1) / S) >= KP) S--;
-    return (int)(S < 1 ? 1 : S);
-}
 
-extern "C" int nmg_spmm_smfmac_splitk_plan(int64_t M, int64_t K, int64_t T, int *slices,
+extern "C" int nmg_splitk_plan(int64_t M, int64_t K, int64_t T, int *slices,
                                            int64_t *workspace_bytes)
 {
     NMG_REQUIRE(M >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");

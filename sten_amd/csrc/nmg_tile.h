@@ -91,4 +91,79 @@ __device__ __forceinline__ void smf_store_tile(const f32x16 (&acc)[FB][TB], unsi
     }
 }
 
+// ---- reductions cut into slices (products with fewer tiles than the GPU has CUs) ----
+// Slice s of a tile stores its sums in single precision at part[s][token][feature] (part_ld
+// features per token, a multiple of 256: the padded features of the last tile are stored too);
+// splitk_sum_kernel adds the slices in order (+ bias) and rounds once.
+struct SplitSum {
+    const float *part;
+    void *y;
+    const void *bias;
+    int64_t M, T, ldy, part_ld;
+    int slices;
+};
+
+// A lane holds token l%32 and features 8*(r/4) + 4*(l/32) + r%4 of every 32 x 32 block: four
+// consecutive features are one 16-byte store.  fw / tw = first feature / token of the wavefront.
+template <int FB, int TB>
+__device__ __forceinline__ void store_partial_tile(const f32x16 (&acc)[FB][TB], float *part, int64_t part_ld,
+                                                   int lane, int64_t fw, int64_t tw, int64_t T)
+{
+    const int j = lane & 31, h = lane >> 5;
+#pragma unroll
+    for (int tb = 0; tb < TB; tb++) {
+        const int64_t tok = tw + tb * 32 + j;
+        if (tok >= T) continue;
+#pragma unroll
+        for (int fb = 0; fb < FB; fb++)
+#pragma unroll
+            for (int rq = 0; rq < 4; rq++) {
+                float4 v;
+                v.x = acc[fb][tb][rq * 4 + 0];
+                v.y = acc[fb][tb][rq * 4 + 1];
+                v.z = acc[fb][tb][rq * 4 + 2];
+                v.w = acc[fb][tb][rq * 4 + 3];
+                *(float4 *)(part + tok * part_ld + fw + fb * 32 + rq * 8 + h * 4) = v;
+            }
+    }
+}
+
+template <typename T> __global__ __launch_bounds__(256) void splitk_sum_kernel(SplitSum P)
+{
+    const int64_t quads = (P.M + 3) / 4;
+    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= P.T * quads) return;
+    const int64_t tok = gid / quads, f = (gid - tok * quads) * 4;
+    const float *src = P.part + tok * P.part_ld + f;
+    float4 sum = *(const float4 *)src;
+    for (int sl = 1; sl < P.slices; sl++) {
+        const float4 v = *(const float4 *)(src + (int64_t)sl * P.T * P.part_ld);
+        sum.x += v.x;
+        sum.y += v.y;
+        sum.z += v.z;
+        sum.w += v.w;
+    }
+    const float o[4] = {sum.x, sum.y, sum.z, sum.w};
+    uint16_t *dst = (uint16_t *)P.y + tok * P.ldy + f;
+    const T *bias = (const T *)P.bias;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (f + i < P.M) dst[i] = f32_to_bits16(o[i] + (bias ? to_f32(bias[f + i]) : 0.f), (T *)nullptr);
+}
+
+template <typename T> static inline int launch_splitk_sum(const SplitSum &P, hipStream_t s)
+{
+    const int64_t threads = P.T * ((P.M + 3) / 4);
+    hipLaunchKernelGGL(splitk_sum_kernel<T>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, P);
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
+// Largest number of slices <= S that leaves none empty: slices of ceil(KP / S) K steps.
+static inline int splitk_fit(int64_t KP, int64_t S)
+{
+    while (S > 1 && (S - 1) * ((KP + S - 1) / S) >= KP) S--;
+    return (int)(S < 1 ? 1 : S);
+}
+
 }  // namespace nmg

@@ -53,6 +53,7 @@ SIGNATURES = {
     "nmg_densefrag_elems": (_I, [_I64, _I64, ctypes.POINTER(ctypes.c_int64)]),
     "nmg_densefrag": (_I, [_P, _P, _I64, _I64, _I, _P, _I, _I, _I, _P]),
     "nmg_spmm_densefrag": (_I, [_P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _P]),
+    "nmg_spmm_densefrag_splitk": (_I, [_P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _P, _I64, _P]),
     "nmg_w4_sizes": (_I, [_I64, _I64] + [ctypes.POINTER(ctypes.c_int64)] * 3),
     "nmg_w4_pack": (_I, [_P, _I64, _I64, _I64, _P, _P, _P, _P]),
     "nmg_w4_to_dense": (_I, [_P, _P, _P, _I64, _I64, _P, _I64, _P]),
@@ -63,7 +64,7 @@ SIGNATURES = {
     "nmg_fragpack": (_I, [_P, _P, _I64, _I64, _P, _P, _I, _I, _I, _P]),
     "nmg_pack_operands": (_I, [_P, _P, _I64, _I64, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "nmg_spmm_smfmac": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _P]),
-    "nmg_spmm_smfmac_splitk_plan": (_I, [_I64, _I64, _I64, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int64)]),
+    "nmg_splitk_plan": (_I, [_I64, _I64, _I64, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int64)]),
     "nmg_spmm_smfmac_splitk": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _P, _I64, _P]),
     "nmg_gemm_nt": (_I, [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I, _P]),
 }

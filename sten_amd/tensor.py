@@ -307,7 +307,7 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
         if T > 16 and variant == -1 and K % 64 == 0 and T * x.stride(0) * 2 < 2 ** 31:
             # few tiles for the chip: the reduction is cut into slices, summed by a second kernel
             slices, ws_bytes = ctypes.c_int(1), ctypes.c_int64(0)
-            native.check(lib.nmg_spmm_smfmac_splitk_plan(O, K, T, ctypes.byref(slices), ctypes.byref(ws_bytes)))
+            native.check(lib.nmg_splitk_plan(O, K, T, ctypes.byref(slices), ctypes.byref(ws_bytes)))
             slices = int(weight.spmm_opt.get("slices", slices.value))
             if slices > 1:
                 tiles_m = (O + 255) // 256
@@ -332,6 +332,20 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
         # "expand, then multiply": one HBM-bound pass writes the weight in the register order of
         # the dense matrix cores into scratch, the pipelined kernel multiplies from there
         df = weight.densefrag(reduce_dim)
+        lib = native.load()
+        slices, ws_bytes = ctypes.c_int(1), ctypes.c_int64(0)
+        if int(weight.spmm_opt.get("dense_variant", -1)) == -1:
+            native.check(lib.nmg_splitk_plan(O, K, T, ctypes.byref(slices), ctypes.byref(ws_bytes)))
+        slices = int(weight.spmm_opt.get("slices", slices.value))
+        if slices > 1:
+            # few tiles for the chip: the reduction is cut into slices, summed by a second kernel
+            ws = torch.empty((slices * T * ((O + 255) // 256) * 256,), dtype=torch.float32, device=x.device)
+            with torch.cuda.device(x.device):
+                native.check(lib.nmg_spmm_densefrag_splitk(
+                    native.ptr(df), O, K, native.ptr(x), x.stride(0), native.ptr(y), O, native.ptr(bias), T,
+                    native.dtype_code(x.dtype), slices, native.ptr(ws), ws.numel() * 4,
+                    native.stream_ptr(x.device)))
+            return y
         with torch.cuda.device(x.device):
             native.check(native.load().nmg_spmm_densefrag(
                 native.ptr(df), O, K, native.ptr(x), x.stride(0), native.ptr(y), O, native.ptr(bias), T,

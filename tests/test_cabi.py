@@ -56,7 +56,7 @@ def test_argument_errors_need_no_gpu():
 def test_split_reduction_plan_and_argument_errors():
     lib = native.load()
     slices, ws = ctypes.c_int(0), ctypes.c_int64(0)
-    plan = lambda M, K, T: (lib.nmg_spmm_smfmac_splitk_plan(M, K, T, ctypes.byref(slices), ctypes.byref(ws)),
+    plan = lambda M, K, T: (lib.nmg_splitk_plan(M, K, T, ctypes.byref(slices), ctypes.byref(ws)),
                             slices.value, ws.value)
     assert plan(4096, 11008, 64) == (0, 8, 8 * 64 * 4096 * 4)         # 16 tiles -> 8 slices of 22 K steps
     assert plan(4096, 11008, 512) == (0, 4, 4 * 512 * 4096 * 4)

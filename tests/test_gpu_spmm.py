@@ -237,7 +237,7 @@ def test_split_reduction_matches_dense(dtype, M, K, T, n, m, g, slices):
         w.spmm_opt["slices"] = slices
     else:
         planned, ws = ctypes.c_int(0), ctypes.c_int64(0)
-        assert native.load().nmg_spmm_smfmac_splitk_plan(M, K, T, ctypes.byref(planned), ctypes.byref(ws)) == 0
+        assert native.load().nmg_splitk_plan(M, K, T, ctypes.byref(planned), ctypes.byref(ws)) == 0
         assert planned.value > 1 and ws.value == planned.value * T * ((M + 255) // 256) * 256 * 4
     x = seeded((T, K), dtype, seed=1)
     b = seeded((M,), dtype, seed=2)
@@ -247,6 +247,34 @@ def test_split_reduction_matches_dense(dtype, M, K, T, n, m, g, slices):
         assert rel_l2(to_np(y), ref) <= TOL[dtype]
     w.spmm_opt["slices"] = 1                      # the same product on whole reductions
     y1 = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)
+    assert rel_l2(to_np(y), to_np(y1)) <= 2 * TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,K,T,n,m,g,rd,slices", [
+    (1024, 2048, 100, 4, 8, 4, 1, None),     # 4:8 forward on the dense matrix cores, planned slices
+    (2048, 1024, 100, 2, 4, 16, 0, None),    # grad_input: reduction along the group dim, planned
+    (2048, 1000, 300, 2, 4, 16, 0, 5),       # ragged outputs, three token tiles, slices of 7, 7, 7, 7, 4
+    (640, 320, 33, 2, 8, 4, 0, 10),          # one K step per slice
+])
+def test_split_reduction_dense_route(dtype, M, K, T, n, m, g, rd, slices):
+    print(f"case split-K dense {dtype} M={M} K={K} T={T} {n}:{m}:{g} reduce_dim={rd} slices={slices}", flush=True)
+    W = seeded((M, K), dtype, seed=M + K + T, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, 1)
+    w = make(W, n, m, g, 1)
+    R, Oo = (K, M) if rd == 1 else (M, K)       # reduction extent, outputs
+    if slices is not None:
+        w.spmm_opt["slices"] = slices
+    else:
+        planned, ws = ctypes.c_int(0), ctypes.c_int64(0)
+        assert native.load().nmg_splitk_plan(Oo, R, T, ctypes.byref(planned), ctypes.byref(ws)) == 0
+        assert planned.value > 1
+    x = seeded((T, R), dtype, seed=1)
+    y = sten.spmm(w, x.to(DEV), reduce_dim=rd, kernel="densefrag")
+    ref = to_np(x).astype(np.float64) @ (Wd.T if rd == 1 else Wd)
+    assert rel_l2(to_np(y), ref) <= TOL[dtype]
+    w.spmm_opt["slices"] = 1
+    y1 = sten.spmm(w, x.to(DEV), reduce_dim=rd, kernel="densefrag")
     assert rel_l2(to_np(y), to_np(y1)) <= 2 * TOL[dtype]
 
 
