@@ -40,6 +40,9 @@ WORKLOADS = {
     "c2": ("fwd", 4096, 4096, 2048, 2, 4, 16, "configs[1]: W 4096x4096 fp16 2:4:16 along K x 2048 tokens, forward"),
     "target_2_4": ("fwd", 4096, 11008, 2048, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 2048 tokens, forward"),
     "target_2_4_4k": ("fwd", 4096, 11008, 4096, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 4096 tokens, forward"),
+    "target_2_4_64": ("fwd", 4096, 11008, 64, 2, 4, 16, "W 4096x11008 fp16 2:4:16 x 64 tokens, forward (split reduction)"),
+    "target_2_4_256": ("fwd", 4096, 11008, 256, 2, 4, 16, "W 4096x11008 fp16 2:4:16 x 256 tokens, forward (split reduction)"),
+    "target_2_4_512": ("fwd", 4096, 11008, 512, 2, 4, 16, "W 4096x11008 fp16 2:4:16 x 512 tokens, forward (split reduction)"),
     "c3_1_8": ("fwd", 8192, 8192, 4096, 1, 8, 32, "configs[2]: W 8192x8192 fp16 1:8:32 x 4096 tokens, forward"),
     "c3_2_8": ("fwd", 8192, 8192, 4096, 2, 8, 32, "configs[2]: W 8192x8192 fp16 2:8:32 x 4096 tokens, forward"),
     "c3_4_8": ("fwd", 8192, 8192, 4096, 4, 8, 32, "configs[2]: W 8192x8192 fp16 4:8:32 x 4096 tokens, forward"),
@@ -258,10 +261,13 @@ def main():
 
     # Decode shapes: the K timed steps are recorded once into a HIP graph and replayed, as a
     # serving loop would launch them -- a step lasts 6-13 us on the device, less than one launch
-    # through Python and ctypes costs on the host (about 15 us).  The large shapes keep the host
-    # busy for less than a step and are launched eagerly (--graph replays them too).
+    # through Python and ctypes costs on the host (about 15 us).  The same holds for products on up
+    # to 1024 tokens (20-70 us on the device, two kernels and two allocations per call).  The large
+    # shapes keep the host busy for less than a step and are launched eagerly (--graph replays
+    # them too).
     graph = None
-    if (kind in ("decode", "w4") and not args.eager) or (args.graph and kind not in ("step", "train", "sparsify")):
+    short = kind in ("decode", "w4") or (kind == "fwd" and N <= 1024)
+    if (short and not args.eager) or (args.graph and kind not in ("step", "train", "sparsify")):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             for _ in range(args.steps):
