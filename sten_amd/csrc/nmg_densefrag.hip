@@ -50,9 +50,14 @@ struct DfExpandParams {
     int64_t G, S, nb;
     int64_t OB, K16;                      // blocks of the operand
     int n, m, pat_bytes, bpt, transpose;  // bpt = blocks of m positions per tile (bpt * m == 128)
+    int order_bytes;                      // size of the order table (specialised kernels: it fits 2 KiB)
 };
 
-template <typename T> __global__ __launch_bounds__(256) void densefrag_kernel(DfExpandParams P)
+// NV = n where the kernel is specialised for it (1, 2, 4: the n values of a block are one load, the
+// order table sits in LDS, and a thread has the loads of four blocks in flight before it scatters
+// the first -- pattern -> order entry -> value is otherwise a chain of round trips per block),
+// 0 = any n.
+template <typename T, int NV> __global__ __launch_bounds__(256) void densefrag_kernel(DfExpandParams P)
 {
     // transpose = 0: tile[line][position], outputs = lines;  transpose = 1: tile[position][line],
     // outputs = positions.  Rows are outputs, columns the reduction; +8 elements of padding keep
@@ -71,21 +76,71 @@ template <typename T> __global__ __launch_bounds__(256) void densefrag_kernel(Df
     }
     __syncthreads();
     const uint16_t *pv = (const uint16_t *)P.pk_val;
-    for (int i = tid; i < DFX_L * P.bpt; i += 256) {
-        const int ql = i / P.bpt, bl = i - ql * P.bpt;
-        const int64_t q = q0 + ql, b = b0 + bl;
-        if (q >= P.G || b >= P.nb) continue;
-        const int64_t blk = q * P.nb + b;
-        const int pat = P.pat_bytes == 1 ? (int)((const uint8_t *)P.pk_pat)[blk]
-                                         : (int)((const uint16_t *)P.pk_pat)[blk];
-        const int8_t *ord = P.order + pat * P.n;
-        for (int j = 0; j < P.n; j++) {
-            const int pos = bl * P.m + ord[j];
-            const uint16_t v = pv[blk * P.n + j];
-            if (P.transpose)
-                tile[pos * pitch + ql] = v;
-            else
-                tile[ql * pitch + pos] = v;
+    if constexpr (NV > 0) {
+        __shared__ int8_t s_ord[2048];
+        for (int i = tid; i < P.order_bytes; i += 256) s_ord[i] = P.order[i];
+        __syncthreads();
+        const int items = DFX_L * P.bpt;
+        for (int base = tid; base < items; base += 4 * 256) {
+            int pat[4];
+            uint16_t v[4][NV];
+            bool live[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int i = base + u * 256;
+                const int ql = i / P.bpt, bl = i - ql * P.bpt;
+                const int64_t q = q0 + ql, b = b0 + bl;
+                live[u] = i < items && q < P.G && b < P.nb;
+                const int64_t blk = live[u] ? q * P.nb + b : 0;
+                pat[u] = P.pat_bytes == 1 ? (int)((const uint8_t *)P.pk_pat)[blk]
+                                          : (int)((const uint16_t *)P.pk_pat)[blk];
+                if constexpr (NV == 1) {
+                    v[u][0] = pv[blk];
+                } else if constexpr (NV == 2) {
+                    const uint32_t w = ((const uint32_t *)pv)[blk];
+                    v[u][0] = (uint16_t)w;
+                    v[u][1] = (uint16_t)(w >> 16);
+                } else {
+                    const uint2 w = ((const uint2 *)pv)[blk];
+                    v[u][0] = (uint16_t)w.x;
+                    v[u][1] = (uint16_t)(w.x >> 16);
+                    v[u][2] = (uint16_t)w.y;
+                    v[u][3] = (uint16_t)(w.y >> 16);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (!live[u]) continue;
+                const int i = base + u * 256;
+                const int ql = i / P.bpt, bl = i - ql * P.bpt;
+                const int8_t *ord = s_ord + pat[u] * NV;
+#pragma unroll
+                for (int j = 0; j < NV; j++) {
+                    const int pos = bl * P.m + ord[j];
+                    if (P.transpose)
+                        tile[pos * pitch + ql] = v[u][j];
+                    else
+                        tile[ql * pitch + pos] = v[u][j];
+                }
+            }
+        }
+    } else {
+        for (int i = tid; i < DFX_L * P.bpt; i += 256) {
+            const int ql = i / P.bpt, bl = i - ql * P.bpt;
+            const int64_t q = q0 + ql, b = b0 + bl;
+            if (q >= P.G || b >= P.nb) continue;
+            const int64_t blk = q * P.nb + b;
+            const int pat = P.pat_bytes == 1 ? (int)((const uint8_t *)P.pk_pat)[blk]
+                                             : (int)((const uint16_t *)P.pk_pat)[blk];
+            const int8_t *ord = P.order + pat * P.n;
+            for (int j = 0; j < P.n; j++) {
+                const int pos = bl * P.m + ord[j];
+                const uint16_t v = pv[blk * P.n + j];
+                if (P.transpose)
+                    tile[pos * pitch + ql] = v;
+                else
+                    tile[ql * pitch + pos] = v;
+            }
         }
     }
     __syncthreads();
@@ -477,10 +532,23 @@ extern "C" int nmg_densefrag(const void *d_pk_val, const void *d_pk_pat, int64_t
     NMG_REQUIRE(gx <= 0x7fffffffLL && gy <= 65535, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
     dim3 grid((unsigned)gx, (unsigned)gy);
     hipStream_t s = (hipStream_t)stream;
+    // the specialised forms load the n values of a block as one word: n * 2 bytes, aligned
+    const int64_t table = binom(m, n) * n;
+    P.order_bytes = (int)(table <= 2048 ? table : 0);
+    const int nv = (n == 1 || n == 2 || n == 4) && table <= 2048 && (uintptr_t)d_pk_val % (2 * n) == 0 ? n : 0;
+    auto launch = [&](auto tag) {
+        using T = decltype(tag);
+        switch (nv) {
+        case 1: hipLaunchKernelGGL((densefrag_kernel<T, 1>), grid, dim3(256), 0, s, P); break;
+        case 2: hipLaunchKernelGGL((densefrag_kernel<T, 2>), grid, dim3(256), 0, s, P); break;
+        case 4: hipLaunchKernelGGL((densefrag_kernel<T, 4>), grid, dim3(256), 0, s, P); break;
+        default: hipLaunchKernelGGL((densefrag_kernel<T, 0>), grid, dim3(256), 0, s, P); break;
+        }
+    };
     if (dtype == NMG_F16)
-        hipLaunchKernelGGL(densefrag_kernel<__half>, grid, dim3(256), 0, s, P);
+        launch(__half{});
     else
-        hipLaunchKernelGGL(densefrag_kernel<__hip_bfloat16>, grid, dim3(256), 0, s, P);
+        launch(__hip_bfloat16{});
     NMG_HIP_TRY(hipGetLastError());
     return NMG_OK;
 }
