@@ -60,14 +60,45 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
         const int64_t kc = r0 / cols + kcl;
         if (kc >= P.num_chunks) break;
         const int64_t slot0 = (kc * P.nb + b0) * cols;   // first slot of the chunk's tiles here
-        for (int e = tid; e < nbw * cols; e += nthr) {
-            const int bl = (int)(((uint64_t)e * P.magic_cols) >> 32), slot = e - bl * cols;
-            const int o = P.idx[slot0 + e];
-            if (o < 0 || kc * cols + o >= P.G) continue;
-            const int at = (kcl * cols + o) * NBW + bl;
-            s_pat[at] = (PT)(((uint64_t)slot * P.magic_g) >> 32);
-            const T *v = val + (slot0 + e) * n;
-            for (int j = 0; j < n; j++) s_val[at * n + j] = v[j];
+        const int cnt = nbw * cols;
+        if (n <= 4) {
+            // four slots per thread are loaded (index and values) before the first is placed:
+            // one round trip to HBM per batch instead of one per slot
+            for (int base = tid; base < cnt; base += 4 * nthr) {
+                int o[4];
+                T vv[4][4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int e = base + u * nthr;
+                    const bool in = e < cnt;
+                    o[u] = in ? (int)P.idx[slot0 + e] : -1;
+                    const T *v = val + (slot0 + (in ? e : 0)) * n;
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        if (j < n) vv[u][j] = v[j];
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int e = base + u * nthr;
+                    if (o[u] < 0 || kc * cols + o[u] >= P.G) continue;
+                    const int bl = (int)(((uint64_t)e * P.magic_cols) >> 32), slot = e - bl * cols;
+                    const int at = (kcl * cols + o[u]) * NBW + bl;
+                    s_pat[at] = (PT)(((uint64_t)slot * P.magic_g) >> 32);
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        if (j < n) s_val[at * n + j] = vv[u][j];
+                }
+            }
+        } else {
+            for (int e = tid; e < cnt; e += nthr) {
+                const int bl = (int)(((uint64_t)e * P.magic_cols) >> 32), slot = e - bl * cols;
+                const int o = P.idx[slot0 + e];
+                if (o < 0 || kc * cols + o >= P.G) continue;
+                const int at = (kcl * cols + o) * NBW + bl;
+                s_pat[at] = (PT)(((uint64_t)slot * P.magic_g) >> 32);
+                const T *v = val + (slot0 + e) * n;
+                for (int j = 0; j < n; j++) s_val[at * n + j] = v[j];
+            }
         }
     }
     __syncthreads();

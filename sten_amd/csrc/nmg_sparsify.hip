@@ -1473,19 +1473,50 @@ __global__ __launch_bounds__(256) void scatter_tiled_kernel(TiledParams Q)
         const uint4 z = {0, 0, 0, 0};
         for (int i = tid; i < cols * pitch * (int)sizeof(T) / 16; i += 256) ((uint4 *)tile)[i] = z;
     }
+    // the order table in LDS where it fits: a slot's positions are then one LDS read away instead
+    // of a round trip to L2 behind the load of its index
+    __shared__ int8_t s_ord[1024];
+    const bool ord_lds = P.c * n <= 1024;
+    if (ord_lds)
+        for (int i = tid; i < P.c * n; i += 256) s_ord[i] = P.order[i];
+    const int8_t *order = ord_lds ? s_ord : P.order;
     __syncthreads();
-    // slots of the NT tiles: contiguous in val / idx
-    for (int e = tid; e < tiles * cols; e += 256) {
-        const int tm = (int)(((uint64_t)e * Q.magic_cols) >> 32), slot = e - tm * cols;
-        const int p = (int)(((uint64_t)slot * Q.magic_g) >> 32);
-        const int64_t at = (t0 + tm) * (int64_t)cols + slot;
-        const int o = P.idx[at];
-        T *v = (T *)P.val + at * n;
-        if (GATHER) {
-            for (int j = 0; j < n; j++)
-                v[j] = (o >= 0 && o < cols) ? tile[o * pitch + tm * m + P.order[p * n + j]] : Zero<T>::v();
-        } else if (o >= 0 && o < cols) {
-            for (int j = 0; j < n; j++) tile[o * pitch + tm * m + P.order[p * n + j]] = v[j];
+    // slots of the NT tiles: contiguous in val / idx (slot e of the workgroup is element
+    // t0 * cols + e).  Four slots per thread are loaded before the first is used: index -> LDS ->
+    // store is otherwise one round trip to HBM per slot and thread.
+    const int total = tiles * cols;
+    const int64_t at0 = t0 * (int64_t)cols;
+    const bool pair = sizeof(T) == 2 && n == 2 && ((uintptr_t)P.val % 4) == 0;
+    for (int base = tid; base < total; base += 4 * 256) {
+        int o[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int e = base + u * 256;
+            o[u] = e < total ? (int)P.idx[at0 + e] : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int e = base + u * 256;
+            if (e >= total) continue;
+            const int tm = (int)(((uint64_t)e * Q.magic_cols) >> 32), slot = e - tm * cols;
+            const int p = (int)(((uint64_t)slot * Q.magic_g) >> 32);
+            const bool ok = o[u] >= 0 && o[u] < cols;
+            T *v = (T *)P.val + (at0 + e) * n;
+            const T *row = tile + (ok ? o[u] : 0) * pitch + tm * m;
+            if (GATHER) {
+                if (pair) {
+                    T w[2];
+                    w[0] = ok ? row[order[p * 2]] : Zero<T>::v();
+                    w[1] = ok ? row[order[p * 2 + 1]] : Zero<T>::v();
+                    uint32_t raw;
+                    __builtin_memcpy(&raw, w, 4);
+                    *(uint32_t *)v = raw;
+                } else {
+                    for (int j = 0; j < n; j++) v[j] = ok ? row[order[p * n + j]] : Zero<T>::v();
+                }
+            } else if (ok) {
+                for (int j = 0; j < n; j++) tile[o[u] * pitch + tm * m + order[p * n + j]] = v[j];
+            }
         }
     }
     if (GATHER) return;
