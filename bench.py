@@ -1,6 +1,6 @@
 """Benchmark of the grouped n:m (nmg) hot path on one MI355X.
 
-Default workload (BASELINE config 2): fp16 weight 4096x4096 ~ N(0, 0.02), grouped 2:4 (group 16)
+Default workload (benchmark config 2): fp16 weight 4096x4096 ~ N(0, 0.02), grouped 2:4 (group 16)
 along the reduction dim; fp16 activations 2048 tokens x 4096 ~ N(0,1); forward only, fp32
 accumulate.  A "step" is one pass of the measured operation over that batch with every operand
 resident in HBM.
@@ -17,7 +17,7 @@ cpu_baseline (default workload) = the CPU restatement of the reference's AVX/Ope
 (oracle/nmg_cpu_simd.cpp) on the host cores, same shape, fp32; for the sparsifier workloads the
 restatement of the reference's single-threaded sort-and-scan on a slab of the weight.
 
-Other modes: --workload picks another BASELINE shape; --calibrate-copy runs a plain device copy
+Other modes: --workload picks another benchmark shape; --calibrate-copy runs a plain device copy
 of known size (the counter calibration for FETCH_SIZE / WRITE_SIZE).
 """
 import argparse

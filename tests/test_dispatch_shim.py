@@ -203,6 +203,6 @@ def test_layout_geometry_matches_oracle_layout():
         assert (a.outer, a.num_chunks, a.num_blocks, a.chunk_size) == (b.outer, b.num_chunks, b.num_blocks, b.c)
         assert a.padded_dense_shape == b.padded_shape
     lay = sten.NMGLayout((4096, 4096), 2, 4, 16, 1, 0)
-    assert lay.outer == 44032 and lay.padded_dense_shape == (4128, 4096)   # BASELINE config 2: 43 chunks of 96 lines x 1024 blocks
+    assert lay.outer == 44032 and lay.padded_dense_shape == (4128, 4096)   # benchmark config 2: 43 chunks of 96 lines x 1024 blocks
     with pytest.raises(ValueError):
         sten.NMGLayout((8, 8), 5, 12, 42, 1, 0)

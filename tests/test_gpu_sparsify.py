@@ -27,7 +27,7 @@ def check_parity(x_cpu, n, m, sd, g, gd):
 
 
 def test_config1_fp32_768_bit_exact():
-    # BASELINE config 1: fp32 768x768 N(0,1) seed 0, 2:4, group 16, n:m along the reduction dim
+    # benchmark config 1: fp32 768x768 N(0,1) seed 0, 2:4, group 16, n:m along the reduction dim
     torch.manual_seed(0)
     w = torch.randn(768, 768)
     check_parity(w, 2, 4, 1, 16, 0)

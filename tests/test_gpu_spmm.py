@@ -53,7 +53,7 @@ def test_spmm_both_directions(kernel, dtype, M, K, T, n, m, g, sd):
 
 
 def test_config1_against_reference_cpu_kernel():
-    # BASELINE config 1 through the reference orientation and the CPU restatement of its kernel
+    # benchmark config 1 through the reference orientation and the CPU restatement of its kernel
     torch.manual_seed(0)
     W = torch.randn(768, 768)
     X = torch.randn(768, 256)          # B [K, N]
@@ -62,7 +62,7 @@ def test_config1_against_reference_cpu_kernel():
     w = make(W, 2, 4, 16, 0)
     C = sten.spmm(w, X.t().contiguous().to(DEV), reduce_dim=1).t()
     assert rel_l2(to_np(C), C_cpu) <= 1e-5
-    w2 = make(W, 2, 4, 16, 1)          # n:m along the reduction dim (BASELINE wording)
+    w2 = make(W, 2, 4, 16, 1)          # n:m along the reduction dim (the benchmark's wording)
     Wd, _ = dense_ref(W, 2, 4, 16, 1)
     C2 = sten.spmm(w2, X.t().contiguous().to(DEV), reduce_dim=1).t()
     assert rel_l2(to_np(C2), Wd @ X.numpy().astype(np.float64)) <= 1e-5
@@ -299,7 +299,7 @@ def test_sparse_matrix_cores_refuse_incompatible_patterns():
 
 
 def test_full_size_config2_smfmac_vs_mfma_and_linearity():
-    # BASELINE config 2 at full size: the two independent kernels agree, and the op is linear in X
+    # benchmark config 2 at full size: the two independent kernels agree, and the op is linear in X
     torch.manual_seed(0)
     W = (torch.randn(4096, 4096) * 0.02).half()
     X = torch.randn(2048, 4096).half().to(DEV)
@@ -441,7 +441,7 @@ def _check_structure(w, n, m):
 
 @pytest.mark.parametrize("n,m", [(2, 8), (4, 8)])
 def test_full_size_config3_forward(n, m):
-    # BASELINE config 3 at full size (8192 x 8192, group 32, 4096 tokens): structure of the
+    # benchmark config 3 at full size (8192 x 8192, group 32, 4096 tokens): structure of the
     # compressed weight, the product against the dense product of its own dense form, linearity
     print(f"case full size config 3 {n}:{m}", flush=True)
     torch.manual_seed(0)
@@ -459,7 +459,7 @@ def test_full_size_config3_forward(n, m):
 
 
 def test_full_size_config5_training_step_pieces():
-    # BASELINE config 5 at full size: forward, grad_input (transposed product) and the masked
+    # benchmark config 5 at full size: forward, grad_input (transposed product) and the masked
     # weight gradient in val layout, each against the dense computation on the dense form
     print("case full size config 5", flush=True)
     torch.manual_seed(0)

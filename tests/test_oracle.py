@@ -253,7 +253,7 @@ def test_gather_inverts_to_dense():
 # ------------------------------------------------------------------------------- spmm
 
 @pytest.mark.parametrize("M,K,N,n,m,g", [
-    (768, 768, 256, 2, 4, 16),   # BASELINE config 1 shape
+    (768, 768, 256, 2, 4, 16),   # benchmark config 1 shape
     (50, 200, 64, 2, 4, 4),      # M and K remainders
     (23, 95, 128, 3, 6, 2),
     (97, 97, 64, 1, 8, 3),       # K one past a tile boundary
