@@ -26,6 +26,7 @@ struct PackParams {
     int R, NBW;          // lines and blocks per workgroup
     int KP, MBtot;       // fragpack extents: pairs of 32 positions, blocks of 32 lines
     int m_log2;
+    int whole_groups;    // m is 4 or 8 and S % 4 == 0: every group of 4 positions lies in one block
     uint64_t magic_cols, magic_g;   // ceil(2^32 / d): x / d == (x * magic) >> 32 for x < 2^16
     uint32_t masks[32];  // position mask of every pattern, four per word (fragpack: m <= 8)
 };
@@ -132,6 +133,73 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
         // then all masks, then all candidate values, so the LDS round trips are three and not one
         // chain per position.
         uint32_t idxword = 0;
+        if (P.whole_groups) {
+            // m = 4 or 8 and no partial group of 4 at the end of the sparse dim: a group of 4
+            // positions lies in one block, so it takes one pattern, one mask and its (at most two)
+            // kept values, which sit side by side in the block's value list
+            for (int ks = 0; ks < 2; ks++) {
+                PT pt[4];
+                int mkb[4], blk[4], base[4];
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int k0 = (kpl * 2 + ks) * 32 + (4 * (q >> 1) + 2 * ga + (q & 1)) * 4;
+                    const bool in = (b0 << P.m_log2) + k0 < P.S;
+                    blk[q] = in ? k0 >> P.m_log2 : 0;
+                    base[q] = k0 & (m - 1);
+                    pt[q] = in ? s_pat[r * NBW + blk[q]] : ABSENT;
+                }
+#pragma unroll
+                for (int q = 0; q < 4; q++) mkb[q] = pt[q] == ABSENT ? 0 : (int)mask[pt[q]];
+                uint16_t c0[4], c1[4];
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int j0 = __popc(mkb[q] & ((1 << base[q]) - 1));
+                    const T *bv = s_val + ((size_t)r * NBW + blk[q]) * n;
+                    const T x0 = bv[j0 < n ? j0 : 0], x1 = bv[j0 + 1 < n ? j0 + 1 : 0];
+                    c0[q] = *reinterpret_cast<const uint16_t *>(&x0);
+                    c1[q] = *reinterpret_cast<const uint16_t *>(&x1);
+                }
+                uint16_t vals[8];
+                uint32_t half = 0;
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int gm = (mkb[q] >> base[q]) & 0xF;
+                    const int cnt = __popc(gm);
+                    int p0 = 0, p1 = 1;
+                    uint16_t v0 = 0, v1 = 0;
+                    if (cnt >= 2) {
+                        p0 = __ffs(gm) - 1;
+                        p1 = __ffs(gm & (gm - 1)) - 1;
+                        v0 = c0[q];
+                        v1 = c1[q];
+                    } else if (cnt == 1) {
+                        // add a zero at an unused position, keeping positions increasing
+                        const int pp = __ffs(gm) - 1;
+                        if (pp == 3) {
+                            p0 = 0;
+                            p1 = 3;
+                            v1 = c0[q];
+                        } else {
+                            p0 = pp;
+                            p1 = 3;
+                            v0 = c0[q];
+                        }
+                    }
+                    vals[2 * q] = v0;
+                    vals[2 * q + 1] = v1;
+                    half |= (uint32_t)(p0 | (p1 << 2)) << (4 * q);
+                }
+                idxword |= half << (16 * ks);
+                uint4 out;
+                out.x = vals[0] | ((uint32_t)vals[1] << 16);
+                out.y = vals[2] | ((uint32_t)vals[3] << 16);
+                out.z = vals[4] | ((uint32_t)vals[5] << 16);
+                out.w = vals[6] | ((uint32_t)vals[7] << 16);
+                *(uint4 *)((uint16_t *)P.fp_val + ((mbg * (P.KP * 2) + kpg * 2 + ks) * 64 + lane) * 8) = out;
+            }
+            P.fp_idx[(mbg * P.KP + kpg) * 64 + lane] = idxword;
+            continue;
+        }
         for (int ks = 0; ks < 2; ks++) {
             PT pat[16];
             int mk[16];
@@ -284,6 +352,7 @@ extern "C" int nmg_pack_operands(const void *d_val, const int16_t *d_idx, int64_
     P.MBtot = (int)((G + 255) / 256 * 8);
     P.m_log2 = 0;
     while ((1 << P.m_log2) < m) P.m_log2++;
+    P.whole_groups = (m == 4 || m == 8) && S % 4 == 0 ? 1 : 0;
     P.magic_cols = (((uint64_t)1 << 32) + tg.cols - 1) / tg.cols;
     P.magic_g = (((uint64_t)1 << 32) + g - 1) / g;
     if (frag) {
