@@ -796,26 +796,56 @@ __global__ __launch_bounds__(NT <= 64 ? 256 : NT) void sparsify_rounds_kernel(Ro
             }
         }
     } else if (P.view.stride_g == 1) {
-        // the columns are contiguous: consecutive threads walk them
-        for (int line = 0; line < tiles * m; line++) {
-            const int tm = line / m, r = line - tm * m;
-            const int64_t t = tile0 + tm;
-            T *dst = (T *)(smem + order_bytes + (size_t)tm * Q.region_bytes) + r;
-            const T *src = nullptr;
-            int valid_cols = 0;
+        // The columns are contiguous: a wavefront takes 64 consecutive columns of one line of
+        // the region (tile, position), four such runs in flight before the first is stored.
+        // The tiles' base offsets come from a small table, computed once.
+        __shared__ int64_t s_tbase[16];
+        __shared__ int s_tcols[16], s_trows[16];
+        if (tid < tiles) {
+            const int64_t t = tile0 + tid;
+            int64_t base = 0;
+            int vc = 0, vr = 0;
             if (t < P.outer) {
                 const int64_t b = t / tiles_per_b;
                 const int64_t rem = t - b * tiles_per_b;
                 const int64_t kc = rem / P.view.num_blocks;
                 const int64_t mb = rem - kc * P.view.num_blocks;
-                const int64_t si = mb * m + r;
-                if (si < P.view.S) {
-                    src = dense + b * P.view.stride_b + kc * cols + si * P.view.stride_s;
-                    const int64_t left = P.view.G - kc * cols;
-                    valid_cols = left < cols ? (int)left : cols;
+                base = b * P.view.stride_b + kc * cols + mb * m * P.view.stride_s;
+                const int64_t left = P.view.G - kc * cols, below = P.view.S - mb * m;
+                vc = left < cols ? (int)left : cols;
+                vr = below < m ? (int)below : m;
+            }
+            s_tbase[tid] = base;
+            s_tcols[tid] = vc;
+            s_trows[tid] = vr;
+        }
+        __syncthreads();
+        const int cpl = (cols + 63) >> 6;                 // runs of 64 columns per line
+        const int nruns = tiles * m * cpl;
+        const int wv = __builtin_amdgcn_readfirstlane(tid >> 6), ln = tid & 63, nw = nthr >> 6;
+        for (int c0 = wv; c0 < nruns; c0 += 4 * nw) {
+            T v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int ce = c0 + u * nw;
+                v[u] = Zero<T>::v();
+                if (ce < nruns) {
+                    const int line = ce / cpl, oc = ce - line * cpl;
+                    const int tm = line / m, r = line - tm * m;
+                    const int o = oc * 64 + ln;
+                    if (o < s_tcols[tm] && r < s_trows[tm])
+                        v[u] = dense[s_tbase[tm] + (int64_t)r * P.view.stride_s + o];
                 }
             }
-            for (int o = tid; o < cols; o += nthr) dst[o * m] = o < valid_cols ? src[o] : Zero<T>::v();
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int ce = c0 + u * nw;
+                if (ce >= nruns) continue;
+                const int line = ce / cpl, oc = ce - line * cpl;
+                const int tm = line / m, r = line - tm * m;
+                const int o = oc * 64 + ln;
+                if (o < cols) ((T *)(smem + order_bytes + (size_t)tm * Q.region_bytes))[o * m + r] = v[u];
+            }
         }
     } else {
         // consecutive threads take the m values of a column, then the same column of the next
