@@ -1225,7 +1225,7 @@ static int launch_sparsify_rounds(SparsifyParams &P, hipStream_t stream, bool *d
     Q.val_pairs = (uintptr_t)P.val % 4 == 0;
     const size_t order_bytes = (size_t)align_up(c, 16);
     const size_t lds = order_bytes + (size_t)Q.tiles * Q.region_bytes;
-    if (lds > 160 * 1024) return NMG_OK;   // too large for this kernel: the caller falls back
+    if (lds > 159 * 1024) return NMG_OK;   // too large for this kernel (which has a small static table too): the caller falls back
     Q.cpad_log2 = 0;
     while ((1 << Q.cpad_log2) < c) Q.cpad_log2++;
     const int8_t *order = host_order(n, m);
