@@ -37,6 +37,8 @@ const int8_t *host_order(int n, int m);
 // Device copy living in this library's file-scope table on the current device; copied there
 // with a blocking hipMemcpy the first time an (n, m) pair is used on that device.
 int device_order(int n, int m, const int8_t **d_order);
+// 256 bytes of zeros on the current device (file-scope array, never written).
+int device_zero_page(const void **d_zero);
 
 inline size_t dtype_size(int dtype)
 {

@@ -122,6 +122,26 @@ int device_order(int n, int m, const int8_t **d_order)
     return NMG_OK;
 }
 
+// 256 zero bytes per GPU: the source of DMA loads that must deliver zeros (reduction positions
+// beyond the end of an operand).  File-scope device arrays start out zero and nothing writes it.
+static __device__ __align__(256) unsigned char g_zero_page[256];
+static std::map<int, const void *> g_zero_pages;
+
+int device_zero_page(const void **d_zero)
+{
+    int dev = 0;
+    NMG_HIP_TRY(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_zero_pages.find(dev);
+    if (it == g_zero_pages.end()) {
+        void *p = nullptr;
+        NMG_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(g_zero_page)));
+        it = g_zero_pages.emplace(dev, p).first;
+    }
+    *d_zero = it->second;
+    return NMG_OK;
+}
+
 }  // namespace nmg
 
 extern "C" {

@@ -1,0 +1,453 @@
+// Masked weight gradient of a grouped n:m weight, written straight into the `val` layout:
+//
+//   val[t, s, j] = sum_tok L[tok, line(t, s)] * P[tok, pos(t, s, j)]
+//
+// L [T, G] holds, per token, the operand that runs along the group dim of the weight (its
+// "lines"), P [T, S] the operand along the sparse dim ("positions"); for a weight W [out, in]
+// that is n:m along `in`, L is the upstream gradient dY [T, out] and P the activations X [T, in].
+// Only the kept positions are stored; no dense [G, S] product is ever written.
+//
+// Both operands have the reduction (tokens) as their slow dim, the opposite of what the matrix
+// cores want (a lane holds 8 consecutive reduction positions of one row).  The transposition is
+// done by the LDS transpose read of gfx950, DS_READ_B64_TR_B16: token-major tiles go global ->
+// LDS by DMA (global_load_lds, 16 bytes per lane), and a fragment of V_MFMA_F32_32X32X16 is two
+// such reads.  Measured lane layout of the instruction: in every group of 16 lanes, lane i
+// receives as element j the 16-bit element (i % 4) of the 8 bytes addressed by lane 4j + i/4.
+//
+// Workgroup: 4 wavefronts, tile 256 positions x 256 lines, each wavefront 128 x 128 (4 x 4
+// accumulator blocks of 32 x 32, 256 accumulator registers).  A K step is 32 tokens; its two
+// operand tiles (2 x 16 KiB) are one stage of a 4-stage LDS ring filled 3 steps ahead.
+//
+// Epilogue: the tile is staged in LDS as [line][position] in the output type; thread = line walks
+// the blocks of m positions, looks up the slot of (line, block) in the slot map (the inverse of
+// `idx`, built once per pattern by nmg_slotmap), derives the pattern from the slot and writes the
+// n kept values of the block to their place in `val`.
+#include "nmg_common.h"
+#include "nmg_tile.h"
+
+#include <type_traits>
+
+namespace nmg {
+
+typedef _Float16 sd_f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 sd_bf16x8 __attribute__((ext_vector_type(8)));
+typedef short sd_i16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) sd_i16x4 *sd_lds_i16x4;
+
+template <typename T> struct SdMma;
+template <> struct SdMma<__half> {
+    using F = sd_f16x8;
+    __device__ static f32x16 run(F a, F b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
+template <> struct SdMma<__hip_bfloat16> {
+    using F = sd_bf16x8;
+    __device__ static f32x16 run(F a, F b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+
+// ------------------------------------------------------------------------------- slot map
+// slot[b][q] (b = block of the sparse dim, q = line of the padded group dim, Gpad = chunks * c*g):
+// the slot s with idx[(q / cg) * nb + b][s] == q % cg.  Every line has exactly one slot per block
+// (idx of a tile is a permutation of 0 .. cg-1).
+struct SlotParams {
+    const int16_t *idx;
+    int16_t *slot;
+    int64_t entries;   // chunks * nb * cg
+    int64_t nb, Gpad;
+    int cg;
+};
+
+__global__ __launch_bounds__(256) void slotmap_kernel(SlotParams P)
+{
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= P.entries) return;
+    const int64_t t = e / P.cg;
+    const int s = (int)(e - t * P.cg);
+    const int64_t kc = t / P.nb, b = t - kc * P.nb;
+    const int col = P.idx[e];
+    if (col < 0 || col >= P.cg) return;   // not a column of the tile (the product kernel clamps what it reads here)
+    P.slot[b * P.Gpad + kc * P.cg + col] = (int16_t)s;
+}
+
+// ------------------------------------------------------------------------------ the product
+struct SddmmParams {
+    const void *lop;   // L [T, G]
+    const void *pop;   // P [T, S]
+    void *val;
+    const int16_t *slot;
+    const int8_t *order;
+    const void *zero;  // 16 zero bytes: source of the tokens beyond T
+    int64_t ldl, ldp, G, S, T, Gpad, nb;
+    int n, m, g, cg;
+    uint32_t inv_g;    // ceil(2^32 / g) for g > 1
+    int order_bytes;
+    int KP;            // K steps of 32 tokens
+    int tiles_p, tiles_l;
+};
+
+constexpr int SD_KS = 32;            // tokens per K step
+constexpr int SD_NS = 4;             // stages of the ring
+constexpr int SD_D = 3;              // K steps in flight
+constexpr int SD_OP = SD_KS * 512;   // bytes of one operand tile: 32 tokens x 256 features
+constexpr int SD_STAGE = 2 * SD_OP;
+constexpr int SD_LPW = 8;            // DMA loads per wavefront per K step (32 KiB / 4 / 1 KiB)
+constexpr int SD_PITCH = 520;        // staged output row: 256 positions x 2 bytes + 8
+constexpr int SD_LDS = 256 * SD_PITCH + kOrderSlotBytes;
+static_assert(SD_NS * SD_STAGE <= 256 * SD_PITCH, "the ring lies inside the staging area");
+static_assert(SD_LDS <= 160 * 1024, "LDS of a CU");
+static_assert(SD_D < SD_NS, "a stage is refilled only after the barrier that ends its last read");
+static_assert(SD_D * SD_LPW < 64, "vmcnt is a 6-bit counter");
+
+template <typename T> __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
+{
+    using Mm = SdMma<T>;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    // Workgroup -> tile.  Consecutive ids are dealt round-robin to the 8 XCDs: give each XCD a
+    // contiguous run of ids, and walk the grid in bands of 4 position tiles, so that a run covers
+    // a compact block of tiles whose operands stay in that XCD's L2.
+    int id = blockIdx.x;
+    const int ntiles = P.tiles_p * P.tiles_l;
+    if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
+    constexpr int GH = 4;
+    const int band = id / (GH * P.tiles_l);
+    const int band_h = min(P.tiles_p - band * GH, GH);
+    const int in_band = id - band * GH * P.tiles_l;
+    const int tile_p = band * GH + in_band % band_h, tile_l = in_band / band_h;
+    const int64_t p0 = (int64_t)tile_p * 256, l0 = (int64_t)tile_l * 256;
+    const int wm = wave >> 1, wn = wave & 1;   // position half / line half of the wavefront
+    const int KP = P.KP;
+
+    // ---- DMA sources.  Wavefronts 0, 1 fetch the position tile, 2, 3 the line tile; load i of a
+    // wavefront fills token rows 2r, 2r+1 (r = (wave & 1) * 8 + i) of its operand tile: 1 KiB of
+    // LDS, lane l -> row 2r + l/32, 16-byte piece l%32.  Piece x of token row t holds the logical
+    // chunk x ^ 4*(t%4) (8 features): the transposing reads below then hit every bank once.
+    const bool is_l = wave >= 2;
+    const unsigned char *gsrc = (const unsigned char *)(is_l ? P.lop : P.pop);
+    const int64_t ld = is_l ? P.ldl : P.ldp, ext = is_l ? P.G : P.S, f0 = is_l ? l0 : p0;
+    uint32_t g_off[SD_LPW];
+#pragma unroll
+    for (int i = 0; i < SD_LPW; i++) {
+        const int tok = (((wave & 1) * 8 + i) << 1) + (lane >> 5);
+        const int chunk = (lane & 31) ^ ((tok & 3) << 2);
+        int64_t feat = f0 + chunk * 8;
+        if (feat > ext - 8) feat = ext - 8;   // columns beyond the extent feed outputs that are never stored
+        g_off[i] = (uint32_t)((tok * ld + feat) * 2);
+    }
+    const int tok_hi = lane >> 5;
+    const unsigned char *zero = (const unsigned char *)P.zero;
+    // The DMA loads are written as instructions: they have no destination registers, so nothing
+    // the compiler does with registers can race with them, and the compiler -- which would make
+    // every LDS read wait for all DMA loads in flight -- does not see them.  Their completion is
+    // tracked by the counted waits below.  (Every load that writes registers is the compiler's.)
+    // K step kp goes to stage kp % SD_NS.  Steps beyond the last are fetched like the last one
+    // (the count of outstanding operations stays uniform; the data is never used).
+    struct Step {
+        const unsigned char *b;   // first token row of the step in the wavefront's operand
+        uint32_t dst;             // LDS address of the wavefront's first load
+        int rem;                  // valid token rows of the step (>= SD_KS except at the end)
+    };
+    auto step_of = [&](int kp) {
+        const int kq = kp < KP ? kp : KP - 1;
+        Step st;
+        st.b = gsrc + (int64_t)kq * SD_KS * ld * 2;
+        st.dst = (uint32_t)(uintptr_t)(lds_ptr_t)(smem + (kp & (SD_NS - 1)) * SD_STAGE + (is_l ? SD_OP : 0) +
+                                                  (wave & 1) * 8 * 1024);
+        st.rem = (int)min((int64_t)SD_KS, P.T - (int64_t)kq * SD_KS);
+        return st;
+    };
+    // tail_tag: the step may hold the end of the operands -- token rows beyond it come from a page
+    // of zeros, at the price of a 64-bit address per lane; the steps before the last take the
+    // scalar base + 32-bit lane offset form.
+    auto issue_one = [&](const Step &st, int i, auto tail_tag) {
+        if constexpr (decltype(tail_tag)::value) {
+            const int tok = (((wave & 1) * 8 + i) << 1) + tok_hi;
+            const unsigned char *src = tok < st.rem ? st.b + g_off[i] : zero;
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                         :: "v"(src), "s"(st.dst + i * 1024) : "memory");
+        } else {
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :: "v"(g_off[i]), "s"(st.b), "s"(st.dst + i * 1024) : "memory");
+        }
+    };
+
+    // ---- fragment addresses.  Lane (q = l/16, i = l%16) of a transposing read supplies the 8
+    // bytes at token 8*(q/2) + i/4 (+ 16*kk + 4*r), features 16*(q%2) + 4*(i%4) .. +3 of the
+    // 32-feature block, and receives feature 16*(q%2) + i = l%32 at tokens 8*(l/32) + 4r + 0..3:
+    // reads r = 0, 1 give the lane its 8 reduction positions of k-step kk, the operand order of
+    // the instruction with reduction slot 8h + 4r + j <-> token 16kk + 8h + 4r + j on both sides.
+    const int q = lane >> 4, i16 = lane & 15, a = i16 >> 2;
+    const int lane_base = (8 * (q >> 1) + a) * 512 + (2 * (q & 1) + ((i16 & 3) >> 1)) * 16 + (i16 & 1) * 8;
+    int fa_off[4], fb_off[4];   // per 32-feature block of the wavefront: position side, line side
+#pragma unroll
+    for (int f = 0; f < 4; f++) {
+        fa_off[f] = lane_base + ((wm * 4 + (f ^ a)) << 6);
+        fb_off[f] = lane_base + ((wn * 4 + (f ^ a)) << 6) + SD_OP;
+    }
+
+    struct Frags {
+        sd_i16x4 a[4][2], b[4][2];
+    };
+    Frags fr[2];
+    // fragment number w in the order the MFMAs first need them: a0, b0, b1, b2, b3, a1, a2, a3
+    auto read_one = [&](Frags &f, const unsigned char *stage, int kk, int w) {
+        const bool is_a = w == 0 || w >= 5;
+        const int x = w == 0 ? 0 : (w >= 5 ? w - 4 : w - 1);
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            if (is_a)
+                f.a[x][r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (sd_lds_i16x4)(stage + fa_off[x] + (16 * kk + 4 * r) * 512));
+            else
+                f.b[x][r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (sd_lds_i16x4)(stage + fb_off[x] + (16 * kk + 4 * r) * 512));
+        }
+    };
+    auto read_frags = [&](Frags &f, const unsigned char *stage, int kk) {
+#pragma unroll
+        for (int w = 0; w < 8; w++) read_one(f, stage, kk, w);
+    };
+
+    f32x16 acc[4][4];   // [position block][line block]
+#pragma unroll
+    for (int x = 0; x < 4; x++)
+#pragma unroll
+        for (int y = 0; y < 4; y++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[x][y][r] = 0.f;
+
+    auto mma = [&](const Frags &f, int lo, int hi) {
+#pragma unroll
+        for (int x = 0; x < 4; x++) {
+            union {
+                sd_i16x4 h[2];
+                typename Mm::F v;
+            } ca;
+            ca.h[0] = f.a[x][0];
+            ca.h[1] = f.a[x][1];
+#pragma unroll
+            for (int y = 0; y < 4; y++) {
+                if (x * 4 + y < lo || x * 4 + y >= hi) continue;
+                union {
+                    sd_i16x4 h[2];
+                    typename Mm::F v;
+                } cb;
+                cb.h[0] = f.b[y][0];
+                cb.h[1] = f.b[y][1];
+                acc[x][y] = Mm::run(ca.v, cb.v, acc[x][y]);
+            }
+        }
+    };
+
+    // Invariants of the ring.  (1) Outstanding memory operations of a wavefront complete in issue
+    // order, SD_LPW per K step; at the counted wait of step kp the steps kp+1 .. kp+SD_D are
+    // outstanding, so vmcnt((SD_D-1) * SD_LPW) means "my share of step kp+1 has landed", and the
+    // barrier after it "everybody's".  (2) Stage (kp+SD_D) % SD_NS is refilled during step kp; its
+    // last readers were the fragment reads of step kp+SD_D-SD_NS <= kp-1, all of which completed
+    // (lgkmcnt(0)) before the barrier that ended that step.
+#pragma unroll
+    for (int s0 = 0; s0 < SD_D; s0++) {
+        const Step st = step_of(s0);
+#pragma unroll
+        for (int i = 0; i < SD_LPW; i++) issue_one(st, i, std::true_type{});
+    }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SD_D - 1) * SD_LPW) : "memory");
+    asm volatile("s_barrier" ::: "memory");
+    read_frags(fr[0], smem, 0);
+
+    // The statements between scheduling fences are issued in this order: one MFMA (32 clocks of
+    // the matrix pipe), then the LDS reads or the DMA load that run in its shadow.
+    auto k_step = [&](int kp, auto tail_tag) {
+        const unsigned char *cur = smem + (kp & (SD_NS - 1)) * SD_STAGE;
+        const unsigned char *nxt = smem + ((kp + 1) & (SD_NS - 1)) * SD_STAGE;
+        const Step st = step_of(kp + SD_D);
+        // k-step 0: under its MFMAs, the fragments of k-step 1, then the loads of step kp+SD_D
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            mma(fr[0], w, w + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            read_one(fr[1], cur, 1, w);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            mma(fr[0], 8 + w, 9 + w);
+            __builtin_amdgcn_sched_barrier(0);
+            issue_one(st, w, tail_tag);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // k-step 1: after its first MFMAs, wait for step kp+1 and meet the other wavefronts (the
+        // LDS reads of step kp are complete); then the first fragments of step kp+1
+        mma(fr[1], 0, 4);
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SD_D - 1) * SD_LPW) : "memory");
+        asm volatile("s_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            mma(fr[1], 4 + w, 5 + w);
+            __builtin_amdgcn_sched_barrier(0);
+            read_one(fr[0], nxt, 0, w);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        mma(fr[1], 12, 16);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // steps whose prefetch (step kp + SD_D) lies before the last step take the short address form
+    const int kp_tail = max(0, KP - 1 - SD_D);
+    for (int kp = 0; kp < kp_tail; kp++) k_step(kp, std::false_type{});
+    for (int kp = kp_tail; kp < KP; kp++) k_step(kp, std::true_type{});
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    asm volatile("s_barrier" ::: "memory");
+
+    // ---- epilogue: stage [line][position] in the output type (D rows = positions 8*(r/4) + 4*(l/32)
+    // + r%4 of the block, column = line l%32: a lane stores 4 consecutive positions of its line)
+    int8_t *s_ord = (int8_t *)(smem + 256 * SD_PITCH);
+    for (int i = tid; i < P.order_bytes; i += 256) s_ord[i] = P.order[i];
+    {
+        const int j = lane & 31, h = lane >> 5;
+#pragma unroll
+        for (int y = 0; y < 4; y++)
+#pragma unroll
+            for (int x = 0; x < 4; x++)
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) {
+                    uint16_t hh[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) hh[e] = f32_to_bits16(acc[x][y][rq * 4 + e], (T *)nullptr);
+                    uint2 pk;
+                    pk.x = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
+                    pk.y = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
+                    const int line = wn * 128 + y * 32 + j, pos = wm * 128 + x * 32 + rq * 8 + h * 4;
+                    *(uint2 *)(smem + line * SD_PITCH + pos * 2) = pk;
+                }
+    }
+    __syncthreads();
+
+    // ---- thread = line: walk the blocks of m positions that meet the tile
+    const int64_t line = l0 + tid;
+    if (line >= P.Gpad) return;
+    const bool line_ok = line < P.G;
+    const int64_t chunk = line / P.cg;
+    const unsigned char *row = smem + tid * SD_PITCH;
+    uint16_t *val = (uint16_t *)P.val;
+    const int n = P.n, m = P.m;
+    const int64_t b_lo = p0 / m, b_hi = min(P.nb, (p0 + 256 + m - 1) / m);
+    const int64_t pend = min(p0 + 256, P.S);
+    const bool whole = (256 % m) == 0;   // blocks do not straddle tiles
+    constexpr int UB = 8;                // blocks in flight: their slots are loaded together
+    for (int64_t bb = b_lo; bb < b_hi; bb += UB) {
+        int slot[UB];
+#pragma unroll
+        for (int u = 0; u < UB; u++) slot[u] = bb + u < b_hi ? (int)P.slot[(bb + u) * P.Gpad + line] : 0;
+#pragma unroll
+        for (int u = 0; u < UB; u++) {
+            const int64_t b = bb + u;
+            if (b >= b_hi) break;
+            const int s = min(max(slot[u], 0), P.cg - 1);
+            const int p = P.g > 1 ? (int)__umulhi((uint32_t)s, P.inv_g) : s;
+            const int8_t *ord = s_ord + p * n;
+            uint16_t *dst = val + (((chunk * P.nb + b) * P.cg + s) * (int64_t)n);
+            const int64_t pb = b * m;
+            if (whole && n == 2) {
+                const int64_t q0 = pb + ord[0], q1 = pb + ord[1];
+                const uint16_t v0 = (line_ok && q0 < pend) ? *(const uint16_t *)(row + (q0 - p0) * 2) : 0;
+                const uint16_t v1 = (line_ok && q1 < pend) ? *(const uint16_t *)(row + (q1 - p0) * 2) : 0;
+                *(uint32_t *)dst = (uint32_t)v0 | ((uint32_t)v1 << 16);
+            } else {
+                for (int j = 0; j < n; j++) {
+                    const int64_t qq = pb + ord[j];
+                    if (qq < p0 || qq >= p0 + 256) continue;   // that position belongs to a neighbouring tile
+                    dst[j] = (line_ok && qq < pend) ? *(const uint16_t *)(row + (qq - p0) * 2) : (uint16_t)0;
+                }
+            }
+        }
+    }
+}
+
+}  // namespace nmg
+
+using namespace nmg;
+
+extern "C" int nmg_slotmap(const int16_t *d_idx, int64_t G, int64_t S, int16_t *d_slot, int n, int m, int g,
+                           void *stream)
+{
+    NMG_REQUIRE(host_order(n, m) != nullptr && g >= 1, NMG_ERR_ARG, "invalid n:m:g = %d:%d:%d", n, m, g);
+    NMG_REQUIRE(G >= 0 && S >= 0, NMG_ERR_ARG, "negative extent");
+    const int64_t cg = binom(m, n) * g;
+    NMG_REQUIRE(cg < 32768, NMG_ERR_ARG, "c*g must be below 2^15");
+    if (G == 0 || S == 0) return NMG_OK;
+    NMG_REQUIRE(d_idx && d_slot, NMG_ERR_ARG, "null device pointer");
+    SlotParams P{};
+    P.idx = d_idx;
+    P.slot = d_slot;
+    P.nb = (S + m - 1) / m;
+    const int64_t chunks = (G + cg - 1) / cg;
+    P.Gpad = chunks * cg;
+    P.cg = (int)cg;
+    P.entries = chunks * P.nb * cg;
+    const int64_t blocks = (P.entries + 255) / 256;
+    NMG_REQUIRE(blocks <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
+    hipLaunchKernelGGL(slotmap_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, P);
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
+extern "C" int nmg_sddmm(const void *d_lines, int64_t ld_lines, const void *d_pos, int64_t ld_pos, int64_t T,
+                         const int16_t *d_slot, int64_t G, int64_t S, void *d_val, int n, int m, int g,
+                         int dtype, void *stream)
+{
+    NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED, "the masked product takes f16/bf16");
+    NMG_REQUIRE(host_order(n, m) != nullptr && g >= 1, NMG_ERR_ARG, "invalid n:m:g = %d:%d:%d", n, m, g);
+    NMG_REQUIRE(G >= 0 && S >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
+    const int64_t cg = binom(m, n) * g;
+    NMG_REQUIRE(cg < 32768, NMG_ERR_ARG, "c*g must be below 2^15");
+    NMG_REQUIRE(ld_lines >= G && ld_pos >= S, NMG_ERR_ARG, "leading dimension smaller than row length");
+    if (G == 0 || S == 0 || n == 0) return NMG_OK;
+    NMG_REQUIRE(T > 0, NMG_ERR_UNSUPPORTED, "no tokens: clear val instead");
+    NMG_REQUIRE(G % 8 == 0 && S % 8 == 0 && ld_lines % 8 == 0 && ld_pos % 8 == 0 &&
+                    ((uintptr_t)d_lines % 16) == 0 && ((uintptr_t)d_pos % 16) == 0,
+                NMG_ERR_UNSUPPORTED, "needs extents and leading dimensions that are multiples of 8 and 16-byte aligned operands");
+    NMG_REQUIRE(ld_lines < ((int64_t)1 << 25) && ld_pos < ((int64_t)1 << 25), NMG_ERR_UNSUPPORTED,
+                "leading dimension too large");
+    NMG_REQUIRE(d_lines && d_pos && d_slot && d_val, NMG_ERR_ARG, "null device pointer");
+    SddmmParams P{};
+    if (int rc = device_order(n, m, &P.order)) return rc;
+    if (int rc = device_zero_page(&P.zero)) return rc;
+    P.lop = d_lines;
+    P.pop = d_pos;
+    P.val = d_val;
+    P.slot = d_slot;
+    P.ldl = ld_lines;
+    P.ldp = ld_pos;
+    P.G = G;
+    P.S = S;
+    P.T = T;
+    P.nb = (S + m - 1) / m;
+    P.Gpad = (G + cg - 1) / cg * cg;
+    P.n = n;
+    P.m = m;
+    P.g = g;
+    P.cg = (int)cg;
+    P.inv_g = g > 1 ? (uint32_t)((((uint64_t)1 << 32) + g - 1) / (uint64_t)g) : 0u;
+    P.order_bytes = (int)(binom(m, n) * n);
+    P.KP = (int)((T + SD_KS - 1) / SD_KS);
+    P.tiles_p = (int)((P.nb * m + 255) / 256);
+    P.tiles_l = (int)((P.Gpad + 255) / 256);
+    NMG_REQUIRE((int64_t)P.tiles_p * P.tiles_l <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid((unsigned)(P.tiles_p * P.tiles_l));
+    if (dtype == NMG_F16) {
+        auto k = sddmm_kernel<__half>;
+        NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, SD_LDS));
+        hipLaunchKernelGGL(k, grid, dim3(256), SD_LDS, s, P);
+    } else {
+        auto k = sddmm_kernel<__hip_bfloat16>;
+        NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, SD_LDS));
+        hipLaunchKernelGGL(k, grid, dim3(256), SD_LDS, s, P);
+    }
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}

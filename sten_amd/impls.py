@@ -23,7 +23,14 @@ class GroupedNMSparsifier:
 
 
 def _masked_weight_grad(weight, lhs_t, rhs):
-    """val-layout gradient: (lhs_t^T @ rhs) gathered at the kept positions of ``weight``."""
+    """val-layout gradient: the kept positions of ``lhs_t^T @ rhs`` (``lhs_t`` [T, rows of W],
+    ``rhs`` [T, columns of W]).  16-bit weights take the fused kernel, which never stores the dense
+    product; fp32 and extents that are not multiples of 8 go through the dense product and the
+    same-pattern gather."""
+    if rhs.dtype != weight.dtype:
+        rhs = rhs.to(weight.dtype)
+    if weight.masked_product_supported(lhs_t, rhs):
+        return weight.masked_product(lhs_t, rhs)
     return weight.clone_layout(torch.mm(lhs_t.t(), rhs))
 
 

@@ -66,6 +66,8 @@ SIGNATURES = {
     "nmg_spmm_smfmac": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _P]),
     "nmg_splitk_plan": (_I, [_I64, _I64, _I64, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int64)]),
     "nmg_spmm_smfmac_splitk": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _P, _I64, _P]),
+    "nmg_slotmap": (_I, [_P, _I64, _I64, _P, _I, _I, _I, _P]),
+    "nmg_sddmm": (_I, [_P, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _I, _I, _I, _I, _P]),
     "nmg_gemm_nt": (_I, [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I, _P]),
 }
 

@@ -141,11 +141,30 @@ class GroupedNMTensor:
         self.spmm_opt = state.get("spmm_opt", {"kernel": "auto"})
 
     # ---- in-place updates that keep the pattern (used by optimizers) ------------------------
+    def _same_pattern(self, other):
+        """True when ``other`` keeps the same positions in the same slots: it shares this
+        tensor's ``idx`` (every ``clone_layout`` result does) or holds an equal copy.  The
+        comparison of two distinct ``idx`` tensors is made once per pair and remembered."""
+        if other.idx is self.idx or (other.idx.data_ptr() == self.idx.data_ptr()
+                                     and other.idx.shape == self.idx.shape):
+            return True
+        key = (other.idx.data_ptr(), other.idx._version, self.idx._version)
+        cached = getattr(self, "_pattern_eq", None)
+        if cached is None or cached[0] != key:
+            same = other.idx.device == self.idx.device and bool(torch.equal(other.idx, self.idx))
+            self._pattern_eq = cached = (key, same)
+        return cached[1]
+
     def _other_val(self, other):
         if isinstance(other, GroupedNMTensor):
             if other.layout != self.layout:
                 raise ValueError("layout mismatch")
-            return other.val
+            if self._same_pattern(other):
+                return other.val
+            # same layout, another choice of columns: slot s of the two tensors names different
+            # positions, so the values go through the dense view and are gathered at this
+            # tensor's kept positions
+            return self.clone_layout(other.to_dense()).val
         if hasattr(other, "wrapped_tensor"):
             return self._other_val(other.wrapped_tensor)
         if hasattr(other, "to_dense") and not isinstance(other, torch.Tensor):
@@ -250,6 +269,69 @@ class GroupedNMTensor:
                 native.ptr(pk_val), native.ptr(pk_pat), lay.G, lay.S, native.ptr(out), K, transpose,
                 lay.n, lay.m, native.dtype_code(out.dtype), native.stream_ptr(out.device)))
         return out
+
+    def slotmap(self):
+        """int16 [num_blocks, Gpad]: for every line of the (padded) group dim and block of the
+        sparse dim, the slot that holds it -- the inverse of ``idx``.  Operand of the masked
+        weight-gradient kernel; depends on the pattern only, cached until ``idx`` changes."""
+        lay = self.layout
+        if len(lay.dense_shape) != 2:
+            raise native.NmgError("the slot map needs a 2-D grouped n:m tensor")
+        key = (self.idx.data_ptr(), self.idx._version)
+        cached = getattr(self, "_slotmap", None)
+        if cached is not None and cached[0] == key:
+            return cached[1]
+        native.require_gpu(self.idx)
+        slot = torch.empty((lay.num_blocks, lay.num_chunks * lay.cols), dtype=torch.int16, device=self.idx.device)
+        with torch.cuda.device(slot.device):
+            native.check(native.load().nmg_slotmap(
+                native.ptr(self.idx), lay.G, lay.S, native.ptr(slot), lay.n, lay.m, lay.group_size,
+                native.stream_ptr(slot.device)))
+        self._slotmap = (key, slot)
+        return slot
+
+    def masked_product(self, rows_op, cols_op):
+        """New tensor with this tensor's pattern whose kept entries are those of
+        ``rows_op^T @ cols_op`` (``rows_op`` [T, R], ``cols_op`` [T, C] for a weight [R, C]): the
+        weight gradient of a linear layer, accumulated in fp32 and written straight into the
+        ``val`` layout.  16-bit types; extents that are multiples of 8."""
+        lay = self.layout
+        R, C = lay.dense_shape
+        native.require_gpu(rows_op, cols_op, self.val)
+        if rows_op.dim() != 2 or cols_op.dim() != 2 or rows_op.shape[0] != cols_op.shape[0] \
+                or rows_op.shape[1] != R or cols_op.shape[1] != C:
+            raise native.NmgError(
+                f"operands must be [T, {R}] and [T, {C}], got {tuple(rows_op.shape)} and {tuple(cols_op.shape)}")
+        dt = self.val.dtype
+        if rows_op.dtype != dt or cols_op.dtype != dt:
+            raise native.NmgError(f"dtype mismatch: operands {rows_op.dtype} / {cols_op.dtype}, weight {dt}")
+        if rows_op.stride(1) != 1:
+            rows_op = rows_op.contiguous()
+        if cols_op.stride(1) != 1:
+            cols_op = cols_op.contiguous()
+        lines, pos = (rows_op, cols_op) if lay.group_dim == 0 else (cols_op, rows_op)
+        val = torch.empty_like(self.val)
+        T = rows_op.shape[0]
+        if T == 0:
+            val.zero_()
+        else:
+            slot = self.slotmap()
+            with torch.cuda.device(val.device):
+                native.check(native.load().nmg_sddmm(
+                    native.ptr(lines), lines.stride(0), native.ptr(pos), pos.stride(0), T, native.ptr(slot),
+                    lay.G, lay.S, native.ptr(val), lay.n, lay.m, lay.group_size, native.dtype_code(dt),
+                    native.stream_ptr(val.device)))
+        out = GroupedNMTensor(val, self.idx, lay)
+        out.spmm_opt = dict(self.spmm_opt)
+        return out
+
+    def masked_product_supported(self, rows_op, cols_op):
+        lay = self.layout
+        return (len(lay.dense_shape) == 2 and self.val.dtype in (torch.float16, torch.bfloat16)
+                and rows_op.dtype == self.val.dtype and cols_op.dtype == self.val.dtype
+                and lay.dense_shape[0] % 8 == 0 and lay.dense_shape[1] % 8 == 0
+                and all(t.stride(1) != 1 or (t.stride(0) % 8 == 0 and t.data_ptr() % 16 == 0)
+                        for t in (rows_op, cols_op)))
 
     def fragpack(self):
         """Operand of the sparse-matrix-core kernel (values + 2-bit positions in instruction
