@@ -44,6 +44,24 @@ template <> struct SdMma<__hip_bfloat16> {
     __device__ static f32x16 run(F a, F b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
 };
 
+// fp32 -> stored 16 bits, round to nearest even (bf16 by the conversion instruction of gfx950)
+template <typename T> __device__ __forceinline__ uint16_t sd_bits16(float x);
+template <> __device__ __forceinline__ uint16_t sd_bits16<__half>(float x) { return __half_as_ushort(__float2half(x)); }
+template <> __device__ __forceinline__ uint16_t sd_bits16<__hip_bfloat16>(float x)
+{
+    const __bf16 b = (__bf16)x;
+    return __builtin_bit_cast(uint16_t, b);
+}
+
+// An accumulator, read where it is used: without this the compiler copies all 256 accumulation
+// registers to architectural ones at the end of the product loop, and spills to make room.
+__device__ __forceinline__ float sd_from_acc(float a)
+{
+    float v;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+    return v;
+}
+
 // ------------------------------------------------------------------------------- slot map
 // slot[b][q] (b = block of the sparse dim, q = line of the padded group dim, Gpad = chunks * c*g):
 // the slot s with idx[(q / cg) * nb + b][s] == q % cg.  Every line has exactly one slot per block
@@ -79,6 +97,7 @@ struct SddmmParams {
     int64_t ldl, ldp, G, S, T, Gpad, nb;
     int n, m, g, cg;
     uint32_t inv_g;    // ceil(2^32 / g) for g > 1
+    uint64_t ord4;     // m == 4: byte p = the kept positions of pattern p, 2 bits each
     int order_bytes;
     int KP;            // K steps of 32 tokens
     int tiles_p, tiles_l;
@@ -97,7 +116,11 @@ static_assert(SD_LDS <= 160 * 1024, "LDS of a CU");
 static_assert(SD_D < SD_NS, "a stage is refilled only after the barrier that ends its last read");
 static_assert(SD_D * SD_LPW < 64, "vmcnt is a 6-bit counter");
 
-template <typename T> __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
+// MODE 1 .. 4: m == 4 and n == MODE.  The 4 consecutive positions a lane holds of its line are one
+// block, so the kept values are picked in registers (one byte permute with a per-pattern selector)
+// and stored by the lane itself; the slots of the lane's 64 (line, block) pairs are fetched when the
+// kernel starts and wait in registers through the product.  MODE 0: any n:m, through the staged tile.
+template <typename T, int MODE> __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
 {
     using Mm = SdMma<T>;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -118,6 +141,35 @@ template <typename T> __global__ __launch_bounds__(256, 1) void sddmm_kernel(Sdd
     const int64_t p0 = (int64_t)tile_p * 256, l0 = (int64_t)tile_l * 256;
     const int wm = wave >> 1, wn = wave & 1;   // position half / line half of the wavefront
     const int KP = P.KP;
+
+    // ---- MODE 1: the lane's slots.  Accumulator block (x, y), register quad rq: line
+    // l0 + wn*128 + y*32 + l%32, block (p0 + wm*128 + x*32 + rq*8 + (l/32)*4) / 4.
+    uint32_t my_slot[MODE >= 1 ? 32 : 1];   // two slots per register: rq even | rq odd << 16
+    if constexpr (MODE >= 1) {
+        // byte selectors of V_PERM_B32 per pattern: kept halves 0, 1 (and 2, 3) out of the 8 bytes
+        // {positions 0, 1 | positions 2, 3} of a block, from the packed order table
+        uint32_t *s_sel = (uint32_t *)(smem + 256 * SD_PITCH);
+        if (tid < 16) {
+            const uint32_t o = (uint32_t)(P.ord4 >> (8 * (tid & 7)));
+            const int jj = (tid >> 3) * 2;
+            const uint32_t a = (o >> (2 * jj)) & 3, b = (o >> (2 * jj + 2)) & 3;
+            s_sel[tid] = (2 * a) | ((2 * a + 1) << 8) | ((2 * b) << 16) | ((2 * b + 1) << 24);
+        }
+        const int j = lane & 31, h = lane >> 5;
+#pragma unroll
+        for (int y = 0; y < 4; y++) {
+            const int64_t line = min(l0 + wn * 128 + y * 32 + j, P.Gpad - 1);
+#pragma unroll
+            for (int x = 0; x < 4; x++)
+#pragma unroll
+                for (int rp = 0; rp < 2; rp++) {
+                    const int blk0 = min((int)(p0 / 4) + wm * 32 + x * 8 + rp * 4 + h, (int)P.nb - 1);
+                    const int blk1 = min((int)(p0 / 4) + wm * 32 + x * 8 + rp * 4 + 2 + h, (int)P.nb - 1);
+                    my_slot[(y * 4 + x) * 2 + rp] = (uint32_t)(uint16_t)P.slot[blk0 * P.Gpad + line] |
+                                                    ((uint32_t)(uint16_t)P.slot[blk1 * P.Gpad + line] << 16);
+                }
+        }
+    }
 
     // ---- DMA sources.  Wavefronts 0, 1 fetch the position tile, 2, 3 the line tile; load i of a
     // wavefront fills token rows 2r, 2r+1 (r = (wave & 1) * 8 + i) of its operand tile: 1 KiB of
@@ -300,10 +352,82 @@ template <typename T> __global__ __launch_bounds__(256, 1) void sddmm_kernel(Sdd
     for (int kp = 0; kp < kp_tail; kp++) k_step(kp, std::false_type{});
     for (int kp = kp_tail; kp < KP; kp++) k_step(kp, std::true_type{});
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    uint16_t *val = (uint16_t *)P.val;
+    const int n = P.n, m = P.m;
+
+    if constexpr (MODE >= 1) {
+        // ---- epilogue in registers (D rows = positions 8*(r/4) + 4*(l/32) + r%4 of the block,
+        // column = line l%32: registers rq*4 .. +3 of a lane are one block of its line).  Offsets
+        // into val are 32-bit (the host checks that val is smaller than 4 GiB).
+        constexpr int N = MODE;
+        const uint32_t *s_sel = (const uint32_t *)(smem + 256 * SD_PITCH);
+        const int j = lane & 31, h = lane >> 5;
+        int blk_base = (int)(p0 / 4) + wm * 32 + h;
+        asm volatile("" : "+v"(blk_base));   // computed afresh: nothing is kept in registers through the product for it
+        const uint32_t cg = (uint32_t)P.cg, nb = (uint32_t)P.nb;
+        const uint32_t g1_mask = P.g > 1 ? 0u : ~0u;   // inv_g is 0 for g == 1
+        unsigned char *vbase = (unsigned char *)P.val;
+        auto epilogue = [&](auto interior_tag) {
+            constexpr bool INTERIOR = decltype(interior_tag)::value;   // every line and block of the tile exists
+#pragma unroll
+            for (int y = 0; y < 4; y++) {
+                const uint32_t line = (uint32_t)l0 + wn * 128 + y * 32 + j;
+                const bool line_in = INTERIOR || line < (uint32_t)P.Gpad, line_ok = INTERIOR || line < (uint32_t)P.G;
+                const uint32_t rowbase = ((line / cg) * nb + (uint32_t)blk_base) * cg;
+#pragma unroll
+                for (int x = 0; x < 4; x++) {
+                    // the slots and selectors of the block's four quads first (LDS reads in flight together)
+                    uint32_t sl[4], sel[4], sel2[4];
+#pragma unroll
+                    for (int rq = 0; rq < 4; rq++) {
+                        sl[rq] = min((my_slot[(y * 4 + x) * 2 + (rq >> 1)] >> (16 * (rq & 1))) & 0x7fffu, cg - 1);
+                        const uint32_t pat = __umulhi(sl[rq], P.inv_g) + (sl[rq] & g1_mask);   // slot / g without a branch
+                        if constexpr (N < 4) sel[rq] = s_sel[pat & 7];
+                        if constexpr (N == 3) sel2[rq] = s_sel[8 + (pat & 7)];
+                    }
+#pragma unroll
+                    for (int rq = 0; rq < 4; rq++) {
+                        uint16_t hh[4];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) hh[e] = sd_bits16<T>(sd_from_acc(acc[x][y][rq * 4 + e]));
+                        uint32_t lo = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
+                        uint32_t hi = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
+                        if (!INTERIOR && !line_ok) lo = hi = 0;
+                        if (!INTERIOR && (!line_in || blk_base + x * 8 + rq * 2 >= (int)nb)) continue;
+                        unsigned char *dst =
+                            vbase + (size_t)((rowbase + (uint32_t)(x * 8 + rq * 2) * cg + sl[rq]) * (uint32_t)(2 * N));
+                        if constexpr (N == 4) {
+                            *(uint2 *)dst = uint2{lo, hi};
+                        } else {
+                            const uint32_t out = __builtin_amdgcn_perm(hi, lo, sel[rq]);
+                            if constexpr (N == 1) {
+                                *(uint16_t *)dst = (uint16_t)out;
+                            } else if constexpr (N == 2) {
+                                *(uint32_t *)dst = out;
+                            } else {   // 6-byte entries are 2-byte aligned only
+                                const uint32_t out2 = __builtin_amdgcn_perm(hi, lo, sel2[rq]);
+                                ((uint16_t *)dst)[0] = (uint16_t)out;
+                                ((uint16_t *)dst)[1] = (uint16_t)(out >> 16);
+                                ((uint16_t *)dst)[2] = (uint16_t)out2;
+                            }
+                        }
+                    }
+                    // an accumulator block at a time: its registers are read when it is stored
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        };
+        if (l0 + 256 <= P.G && p0 + 256 <= P.nb * 4)
+            epilogue(std::true_type{});
+        else
+            epilogue(std::false_type{});
+        return;
+    }
     asm volatile("s_barrier" ::: "memory");
 
-    // ---- epilogue: stage [line][position] in the output type (D rows = positions 8*(r/4) + 4*(l/32)
-    // + r%4 of the block, column = line l%32: a lane stores 4 consecutive positions of its line)
+    // ---- epilogue through LDS: stage [line][position] in the output type (D rows = positions
+    // 8*(r/4) + 4*(l/32) + r%4 of the block, column = line l%32: a lane stores 4 consecutive
+    // positions of its line)
     int8_t *s_ord = (int8_t *)(smem + 256 * SD_PITCH);
     for (int i = tid; i < P.order_bytes; i += 256) s_ord[i] = P.order[i];
     {
@@ -332,17 +456,15 @@ template <typename T> __global__ __launch_bounds__(256, 1) void sddmm_kernel(Sdd
     const bool line_ok = line < P.G;
     const int64_t chunk = line / P.cg;
     const unsigned char *row = smem + tid * SD_PITCH;
-    uint16_t *val = (uint16_t *)P.val;
-    const int n = P.n, m = P.m;
     const int64_t b_lo = p0 / m, b_hi = min(P.nb, (p0 + 256 + m - 1) / m);
     const int64_t pend = min(p0 + 256, P.S);
     const bool whole = (256 % m) == 0;   // blocks do not straddle tiles
-    constexpr int UB = 8;                // blocks in flight: their slots are loaded together
+    constexpr int UB = 32;               // blocks in flight: their slots are loaded together
     for (int64_t bb = b_lo; bb < b_hi; bb += UB) {
         int slot[UB];
 #pragma unroll
         for (int u = 0; u < UB; u++) slot[u] = bb + u < b_hi ? (int)P.slot[(bb + u) * P.Gpad + line] : 0;
-#pragma unroll
+#pragma unroll 4
         for (int u = 0; u < UB; u++) {
             const int64_t b = bb + u;
             if (b >= b_hi) break;
@@ -439,15 +561,32 @@ extern "C" int nmg_sddmm(const void *d_lines, int64_t ld_lines, const void *d_po
     NMG_REQUIRE((int64_t)P.tiles_p * P.tiles_l <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
     hipStream_t s = (hipStream_t)stream;
     dim3 grid((unsigned)(P.tiles_p * P.tiles_l));
-    if (dtype == NMG_F16) {
-        auto k = sddmm_kernel<__half>;
-        NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, SD_LDS));
-        hipLaunchKernelGGL(k, grid, dim3(256), SD_LDS, s, P);
-    } else {
-        auto k = sddmm_kernel<__hip_bfloat16>;
-        NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, SD_LDS));
-        hipLaunchKernelGGL(k, grid, dim3(256), SD_LDS, s, P);
+    // m == 4, val 8-byte aligned and smaller than 4 GiB: the epilogue that stays in registers
+    const int64_t val_bytes = ((G + cg - 1) / cg) * P.nb * cg * n * 2;
+    const bool in_regs = m == 4 && n >= 1 && ((uintptr_t)d_val % 8) == 0 && val_bytes < ((int64_t)1 << 32) &&
+                         P.Gpad < ((int64_t)1 << 31);
+    if (in_regs) {
+        const int8_t *ho = host_order(n, m);
+        for (int64_t p = 0; p < binom(m, n); p++)
+            for (int j = 0; j < n; j++) P.ord4 |= (uint64_t)(ho[p * n + j] & 3) << (8 * p + 2 * j);
     }
+    auto launch = [&](auto k) -> int {
+        NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, SD_LDS));
+        hipLaunchKernelGGL(k, grid, dim3(256), SD_LDS, s, P);
+        return NMG_OK;
+    };
+    auto launch_t = [&](auto tag) -> int {
+        using T = decltype(tag);
+        if (!in_regs) return launch(sddmm_kernel<T, 0>);
+        switch (n) {
+        case 1: return launch(sddmm_kernel<T, 1>);
+        case 2: return launch(sddmm_kernel<T, 2>);
+        case 3: return launch(sddmm_kernel<T, 3>);
+        default: return launch(sddmm_kernel<T, 4>);
+        }
+    };
+    const int rc = dtype == NMG_F16 ? launch_t(__half{}) : launch_t(__hip_bfloat16{});
+    if (rc) return rc;
     NMG_HIP_TRY(hipGetLastError());
     return NMG_OK;
 }
