@@ -1,9 +1,9 @@
 """Benchmark of the grouped n:m (nmg) hot path on one MI355X.
 
-Default workload (benchmark config 2): fp16 weight 4096x4096 ~ N(0, 0.02), grouped 2:4 (group 16)
-along the reduction dim; fp16 activations 2048 tokens x 4096 ~ N(0,1); forward only, fp32
-accumulate.  A "step" is one pass of the measured operation over that batch with every operand
-resident in HBM.
+Default (headline) workload: the north-star shape, fp16 weight 4096x11008 ~ N(0, 0.02), grouped
+2:4 (group 16) along the reduction dim; fp16 activations 2048 tokens x 11008 ~ N(0,1); forward
+only, fp32 accumulate.  A "step" is one pass of the measured operation over that batch with every
+operand resident in HBM.
 
 Prints one JSON line.  For the matmul workloads value = dense-equivalent TFLOP/s (2*M*K*N / step
 time) and roofline.achieved counts the effective (non-zero) flops 2*M*K*N*n/m per launch over the
@@ -11,11 +11,16 @@ kernel's average launch duration, measured with HIP events on the stream the ker
 on, against the dense fp16 MFMA peak -- i.e. the fraction of the density-scaled MFMA roofline.
 For the bandwidth-bound workloads (decode shapes, sparsifier) value = GB/s of algorithmic bytes
 (weight values + int16 indices + activations + output; dense input + val + idx for the
-sparsifier) and the roofline is HBM.  roofline.traffic is read from the committed rocprofv3 --pmc
-summary of the same command, when there is one.
-cpu_baseline (default workload) = the CPU restatement of the reference's AVX/OpenMP kernel
-(oracle/nmg_cpu_simd.cpp) on the host cores, same shape, fp32; for the sparsifier workloads the
-restatement of the reference's single-threaded sort-and-scan on a slab of the weight.
+sparsifier) and the roofline is HBM.  roofline.traffic is null: HBM traffic comes from rocprofv3
+counter runs, whose summaries are under profiles/ (config.traffic_profile names the file).
+With the default workload the same run also measures the other benchmark rows (config 2, config 3
+at 2:8, the decode shapes at 1 and 16 tokens, config 4 at 1 token, the config 2 sparsifier and the
+config 5 training step) with the same protocol and reports them under config.also as
+{us, value, unit, frac}; --no-also skips them.
+cpu_baseline (headline and config 2) = the CPU restatement of the reference's AVX/OpenMP kernel
+(oracle/nmg_cpu_simd.cpp) on the host cores, same shape, fp32, on a 1024-row slab of the weight;
+for the sparsifier workloads the restatement of the reference's single-threaded sort-and-scan on
+a slab of the weight.
 
 Other modes: --workload picks another benchmark shape; --calibrate-copy runs a plain device copy
 of known size (the counter calibration for FETCH_SIZE / WRITE_SIZE).
@@ -23,7 +28,6 @@ of known size (the counter calibration for FETCH_SIZE / WRITE_SIZE).
 import argparse
 import json
 import os
-import re
 import sys
 import time
 
@@ -72,6 +76,10 @@ PMC_SUMMARIES = {
     "c4_b1": "w4_linear_c4_b1_pmc.txt",
     "sparsify_c2": "sparsify_rounds_sparsify_c2_pmc.txt",
 }
+
+# measured beside the headline workload in the default run: (workload, steps, warm-up)
+ALSO = [("c2", 50, 10), ("c3_2_8", 20, 5), ("decode_1", 50, 10), ("decode_16", 50, 10), ("c4_b1", 50, 10),
+        ("sparsify_c2", 20, 5), ("c5_step", 10, 3)]
 
 
 def cpu_baseline(M, K, N, n, m, g, seconds=15.0):
@@ -130,19 +138,6 @@ def cpu_baseline_sparsify(M, K, n, m, g, seconds=10.0):
     }
 
 
-def committed_traffic(workload):
-    """HBM bytes per launch from profiles/ (FETCH_SIZE + WRITE_SIZE, calibrated), or None."""
-    name = PMC_SUMMARIES.get(workload)
-    if name is None:
-        return None
-    try:
-        text = open(os.path.join(ROOT, "profiles", name)).read()
-    except OSError:
-        return None
-    mt = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", text, re.M)
-    return float(mt.group(1)) if mt else None
-
-
 def calibrate_copy():
     import torch
     n = 64 * 1024 * 1024
@@ -154,34 +149,14 @@ def calibrate_copy():
     print(json.dumps({"calibration": "device copy", "bytes_read": n, "bytes_written": n}))
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
-    ap.add_argument("--kernel", default="auto")
-    ap.add_argument("--variant", type=int, default=-1)
-    ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--eager", action="store_true", help="launch every step from Python, decode shapes too")
-    ap.add_argument("--graph", action="store_true", help="replay the timed steps from a HIP graph, large shapes too")
-    ap.add_argument("--calibrate-copy", action="store_true")
-    ap.add_argument("--copies", type=int, default=0,
-                    help="decode shapes: separate copies of the weight that the steps take in turn "
-                         "(0: as many as exceed 512 MiB, so that no step finds its weight in a cache)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU; multi-GPU runs are not part of this build", file=sys.stderr)
-        sys.exit(2)
-    if args.calibrate_copy:
-        calibrate_copy()
-        return
-
+def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, graph_large=False, copies_arg=0):
+    """Run one workload: `warmup` untimed steps, then `steps` timed ones between two synchronisations.
+    Returns the row of that workload (times, value, roofline)."""
     import torch
     import sten_amd as sten
 
     dev = "cuda:0"
-    kind, M, K, N, n, m, g, desc = WORKLOADS[args.workload]
+    kind, M, K, N, n, m, g, desc = WORKLOADS[workload]
     # Decode shapes are bound by the stream of the weight from HBM, and a weight of 18-54 MB
     # would stay in the 256 MB memory-side cache between two steps: the steps take separate
     # copies of it in turn, more than 512 MiB in all.
@@ -220,7 +195,7 @@ def main():
     elif kind == "w4":
         # int4 kept values + 2-bit positions + fp16 scales + activations + output
         algo_bytes = M * K // 4 + M * K // 8 + (K // 128) * M * 2 + N * K * 2 + N * M * 2
-        copies = args.copies or -(-ROTATE_BYTES // algo_bytes)
+        copies = copies_arg or -(-ROTATE_BYTES // algo_bytes)
         ws = [sten.SparseMarlinTensor.from_dense(W) for _ in range(copies)]
         del W
         X = torch.randn(N, K).half().to(dev)
@@ -237,11 +212,11 @@ def main():
         # weight values + one int16 index per (line, block) + activations + output
         algo_bytes = M * K * n // m * 2 + M * K // m * 2 + N * K * 2 + N * M * 2
         if kind == "decode":
-            copies = args.copies or -(-ROTATE_BYTES // algo_bytes)
+            copies = copies_arg or -(-ROTATE_BYTES // algo_bytes)
         ws = [sten.GroupedNMTensor.from_dense(W, n, m, sparse_dim=1, group_size=g, group_dim=0)
               for _ in range(copies)]
         for w in ws:
-            w.spmm_opt["variant"] = args.variant
+            w.spmm_opt["variant"] = variant
         del W
         if kind == "grad_x":
             X = torch.randn(N, M).half().to(dev)      # upstream gradient dY [tokens, out features]
@@ -252,10 +227,10 @@ def main():
 
         def step():
             turn[0] += 1
-            return sten.spmm(ws[turn[0] % copies], X, reduce_dim=rd, kernel=args.kernel)
+            return sten.spmm(ws[turn[0] % copies], X, reduce_dim=rd, kernel=kernel)
 
     # every copy of the weight derives its kernel operands before anything is timed or captured
-    for _ in range(max(args.warmup, copies)):
+    for _ in range(max(warmup, copies)):
         step()
     torch.cuda.synchronize()
 
@@ -267,10 +242,10 @@ def main():
     # them too).
     graph = None
     short = kind in ("decode", "w4") or (kind == "fwd" and N <= 1024)
-    if (short and not args.eager) or (args.graph and kind not in ("step", "train", "sparsify")):
+    if (short and not eager) or (graph_large and kind not in ("step", "train", "sparsify")):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            for _ in range(args.steps):
+            for _ in range(steps):
                 step()
         graph.replay()
         torch.cuda.synchronize()
@@ -279,7 +254,7 @@ def main():
         if graph is not None:
             graph.replay()
         else:
-            for _ in range(args.steps):
+            for _ in range(steps):
                 step()
 
     # The timed region: K back-to-back steps between two synchronisations.  The average duration
@@ -292,41 +267,86 @@ def main():
     run_steps()
     e1.record(stream)
     torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / args.steps
-    kern_ms = e0.elapsed_time(e1) / args.steps
+    wall = (time.perf_counter() - t0) / steps
+    kern_ms = e0.elapsed_time(e1) / steps
     launch = "hip graph of the timed steps, replayed" if graph is not None else "eager"
 
-    out = {
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": wall * 1e3,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16", "data": "synthetic",
-    }
+    row = {"ms_per_step": wall * 1e3, "kernel_ms": kern_ms, "launch": launch, "desc": desc, "kind": kind,
+           "shape": (M, K, N, n, m, g), "traffic_profile": PMC_SUMMARIES.get(workload)}
     if kind in ("fwd", "grad_x", "step", "train"):
         dense_flops = 2.0 * M * K * N * (3 if kind in ("step", "train") else 1)
         eff_flops = dense_flops * n / m
         achieved = eff_flops / (kern_ms * 1e-3) / 1e12
-        out.update({
+        row.update({
             "metric": "nmg sparse x dense GEMM TFLOP/s (dense-equiv)",
             "value": dense_flops / wall / 1e12, "unit": "TFLOP/s",
-            "config": {"workload": desc, "kernel": args.kernel, "variant": args.variant, "launch": launch,
-                       "effective_tflops": eff_flops / wall / 1e12, "kernel_ms": kern_ms},
+            "effective_tflops": eff_flops / wall / 1e12,
             "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP16_TFLOPS,
-                         "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS,
-                         "traffic": committed_traffic(args.workload),
+                         "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS, "traffic": None,
                          "flops": "effective non-zero (2*M*K*N*n/m); dense-equivalent is m/n times this"},
         })
     else:
         achieved = algo_bytes / (kern_ms * 1e-3) / 1e9
-        out.update({
+        row.update({
             "metric": "nmg sparsifier GB/s" if kind == "sparsify" else "nmg sparse x dense decode GB/s",
             "value": algo_bytes / wall / 1e9, "unit": "GB/s",
-            "config": {"workload": desc, "kernel": args.kernel, "launch": launch, "kernel_ms": kern_ms,
-                       "algorithmic_bytes": algo_bytes, "weight_copies": copies},
+            "algorithmic_bytes": algo_bytes, "weight_copies": copies,
             "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": achieved / PEAK_HBM_GBS, "traffic": committed_traffic(args.workload)},
+                         "frac": achieved / PEAK_HBM_GBS, "traffic": None},
         })
-    if not args.no_cpu and args.workload == "c2":
+    del step
+    torch.cuda.empty_cache()
+    return row
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="target_2_4", choices=sorted(WORKLOADS))
+    ap.add_argument("--kernel", default="auto")
+    ap.add_argument("--variant", type=int, default=-1)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-also", action="store_true", help="headline workload only")
+    ap.add_argument("--eager", action="store_true", help="launch every step from Python, decode shapes too")
+    ap.add_argument("--graph", action="store_true", help="replay the timed steps from a HIP graph, large shapes too")
+    ap.add_argument("--calibrate-copy", action="store_true")
+    ap.add_argument("--copies", type=int, default=0,
+                    help="decode shapes: separate copies of the weight that the steps take in turn "
+                         "(0: as many as exceed 512 MiB, so that no step finds its weight in a cache)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU; multi-GPU runs are not part of this build", file=sys.stderr)
+        sys.exit(2)
+    if args.calibrate_copy:
+        calibrate_copy()
+        return
+
+    row = measure(args.workload, args.steps, args.warmup, args.kernel, args.variant, args.eager, args.graph,
+                  args.copies)
+    kind, M, K, N, n, m, g, desc = WORKLOADS[args.workload]
+    out = {
+        "metric": row["metric"], "value": row["value"], "unit": row["unit"],
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": row["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": desc, "kernel": args.kernel, "variant": args.variant, "launch": row["launch"],
+                   "kernel_ms": row["kernel_ms"], "traffic_profile": row["traffic_profile"]},
+        "roofline": row["roofline"],
+    }
+    for key in ("effective_tflops", "algorithmic_bytes", "weight_copies"):
+        if key in row:
+            out["config"][key] = row[key]
+    if args.workload == "target_2_4" and not args.no_also:
+        also = {}
+        for name, steps, warmup in ALSO:
+            r = measure(name, steps, warmup)
+            also[name] = {"us": r["kernel_ms"] * 1e3, "value": r["value"], "unit": r["unit"],
+                          "frac": r["roofline"]["frac"], "bound": r["roofline"]["bound"]}
+        out["config"]["also"] = also
+    if not args.no_cpu and args.workload in ("c2", "target_2_4"):
         out["cpu_baseline"] = cpu_baseline(M, K, N, n, m, g)
     if not args.no_cpu and kind == "sparsify":
         out["cpu_baseline"] = cpu_baseline_sparsify(M, K, n, m, g)

@@ -14,12 +14,14 @@ from .dispatch import (DISPATCH_RAISE, DISPATCH_WARN, DenseTensor, DispatchError
 from .impls import GroupedNMSparsifier, install
 from .layout import NMGLayout
 from .native import NmgError
-from .perfect import PerfectNMTensor, is_correct_nm
+from . import perfect
+from .perfect import PerfectNMSparsifier, PerfectNMTensor, is_correct_nm
 from .tensor import GroupedNMTensor, spmm
 from . import w4
 from .w4 import SparseMarlinSparsifier, SparseMarlinTensor
 
 install(dispatch)
 w4.install(dispatch)
+perfect.install(dispatch)
 
 __all__ = [n for n in dir() if not n.startswith("_")]

@@ -353,13 +353,39 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
         }
     };
 
+    // The counted wait.  Invariants it rests on:
+    //  (1) a wavefront's vector memory operations complete in issue order, and it issues exactly
+    //      OPS of them per K step (XL DMA loads, then 4 * FB weight fragments), all of step
+    //      kp+DD_D before the wait at the end of step kp; so at that wait the newest (DD_D-1) * OPS
+    //      operations are the steps kp+2 .. kp+DD_D and everything older -- step kp+1 -- has landed
+    //      once the counter is down to (DD_D-1) * OPS.  The barrier after it makes that true for
+    //      the DMA loads of the other wavefronts too.
+    //  (2) the weight set of step kp+1 is passed through the wait as in/out operands: whatever
+    //      uses those registers afterwards is ordered after the wait by the compiler as well.
+    //      (What it does with them *before* the wait is checked on the compiled code: no
+    //      instruction may touch a register with a load in flight, `python -m sten_amd.isa_check`.)
+    //  (3) LDS stage (kp+DD_D) % DD_NS is refilled during step kp; its last readers were the
+    //      fragment reads of step kp+DD_D-DD_NS <= kp-2, complete (lgkmcnt(0), same wait) before
+    //      the barrier that ended that step.  The two fragment sets alternate by phase; NP is
+    //      even, so the set read after the barrier (for phase 0 of the next step) is set 0.
+    static_assert(DD_NS > DD_D, "a stage must not be refilled while the step that reads it is in flight");
+    static_assert(NP % 2 == 0, "fragment sets alternate by phase across K steps");
+    static_assert(FB == 2, "the wait lists the registers of two fragment rows");
+    auto landed = [&](WSet &w) {
+        asm volatile("s_waitcnt vmcnt(%8) lgkmcnt(0)"
+                     : "+v"(w.a[0][0]), "+v"(w.a[0][1]), "+v"(w.a[0][2]), "+v"(w.a[0][3]),
+                       "+v"(w.a[1][0]), "+v"(w.a[1][1]), "+v"(w.a[1][2]), "+v"(w.a[1][3])
+                     : "n"((DD_D - 1) * OPS)
+                     : "memory");
+    };
+
     // prologue: steps 0 .. DD_D-1 in flight, then wait for step 0
 #pragma unroll
     for (int st = 0; st < DD_D; st++) {
         issue_x(st);
         issue_a(st, ws[st]);
     }
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DD_D - 1) * OPS) : "memory");
+    landed(ws[0]);
     asm volatile("s_barrier" ::: "memory");
     read_b(fr[0], smem, 0);
 
@@ -383,8 +409,8 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
                     for (int i = PH * OPS / NP; i < OPS; i++)
                         issue_one(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)], i);
                     __builtin_amdgcn_sched_barrier(0);
-                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // fragments of step kp are in registers
-                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DD_D - 1) * OPS) : "memory");  // my share of kp+1 landed
+                    // fragments of step kp are in registers, my share of step kp+1 has landed ...
+                    landed(ws[(u + 1) % (DD_D + 1)]);
                     asm volatile("s_barrier" ::: "memory");              // ... and everybody else's
                     __builtin_amdgcn_sched_barrier(0);
                     read_b(fr[(PH + 1) % 2], next, 0);
@@ -470,14 +496,11 @@ template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_
 
 template <typename T> static int launch_dense(DfParams &P, int variant, hipStream_t s)
 {
-    if (variant < 0) {
-        // 256 x 256 tiles move fewer bytes per flop through the vector caches but there are half
-        // as many of them to spread over the 256 CUs: compare rounds of tiles.
-        const int64_t tm = (P.O + 255) / 256;
-        const int64_t n128 = tm * ((P.T + 127) / 128), n256 = tm * ((P.T + 255) / 256);
-        const double cost128 = (double)((n128 + 255) / 256), cost256 = 1.7 * (double)((n256 + 255) / 256);
-        variant = cost256 < cost128 ? 1 : 0;
-    }
+    // 256 x 256 tiles (variant 1) move fewer bytes per flop through the vector caches and are 8 %
+    // faster on shapes with enough of them, but they are by request only: a sixteen-phase form of
+    // that tile once gave wrong values now and then and the cause was never found, so the automatic
+    // choice stays with the tile that has no such history.
+    if (variant < 0) variant = 0;
     if (variant == 1) return launch_dense_direct<T, 2, 8, 4, 1, 2>(P, s);
     return launch_dense_direct<T, 2, 4, 4, 1, 1>(P, s);
 }

@@ -693,12 +693,31 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
         }
     };
 
+    // The counted wait.  (1) A wavefront's vector memory operations complete in issue order and
+    // it issues exactly OPS of them per K step, all of step kp+DR_D before the wait at the end of
+    // step kp: when the counter is down to (DR_D-1) * OPS, step kp+1 has landed; the barrier after
+    // it extends that to the DMA loads of the other wavefronts.  (2) The weight set of step kp+1
+    // passes through the wait as in/out operands, so its later uses are ordered after the wait by
+    // the compiler as well; that nothing touches a register with a load in flight *before* the
+    // wait is checked on the compiled code (`python -m sten_amd.isa_check`).  (3) LDS stage
+    // (kp+DR_D) % DR_NS is refilled during step kp; its last readers, the fragment reads of step
+    // kp+DR_D-DR_NS < kp, completed (lgkmcnt(0), same wait) before the barrier of their step.
+    static_assert(DR_NS > DR_D, "a stage must not be refilled while the step that reads it is in flight");
+    static_assert(NP % 2 == 0, "fragment sets alternate by phase across K steps");
+    static_assert(FB == 2, "the wait lists the registers of two fragment rows");
+    auto landed = [&](WSet &w) {
+        asm volatile("s_waitcnt vmcnt(%6) lgkmcnt(0)"
+                     : "+a"(w.a[0][0]), "+a"(w.a[0][1]), "+v"(w.ix[0]), "+a"(w.a[1][0]), "+a"(w.a[1][1]), "+v"(w.ix[1])
+                     : "n"((DR_D - 1) * OPS)
+                     : "memory");
+    };
+
     // prologue: steps 0 .. DR_D-1 in flight, then wait for step 0
 #pragma unroll
     for (int st = 0; st < DR_D; st++) {
         issue_step(st, ws[st]);
     }
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DR_D - 1) * OPS) : "memory");
+    landed(ws[0]);
     asm volatile("s_barrier" ::: "memory");
     read_b(fr[0], smem, 0);
 
@@ -722,8 +741,8 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
                     for (int i = PH * OPS / NP; i < OPS; i++)
                         issue_one(kp + DR_D, ws[(u + DR_D) % (DR_D + 1)], i);
                     __builtin_amdgcn_sched_barrier(0);
-                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // fragments of step kp are in registers
-                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DR_D - 1) * OPS) : "memory");  // my share of kp+1 landed
+                    // fragments of step kp are in registers, my share of step kp+1 has landed ...
+                    landed(ws[(u + 1) % (DR_D + 1)]);
                     asm volatile("s_barrier" ::: "memory");              // ... and everybody else's
                     __builtin_amdgcn_sched_barrier(0);
                     read_b(fr[(PH + 1) % 2], next, 0);

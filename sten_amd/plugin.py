@@ -10,7 +10,7 @@ registration of a sparsifier key (sten.py:1096-1100), so existing keys are remov
 """
 import torch
 
-from . import impls, w4
+from . import impls, perfect, w4
 from .tensor import GroupedNMTensor
 
 
@@ -33,3 +33,8 @@ def register(sten_module):
     w4_key = (w4.SparseMarlinSparsifier, torch.Tensor, w4.SparseMarlinTensor)
     if reg is None or w4_key not in reg:
         w4.install(sten_module)
+    pf_key = (perfect.PerfectNMSparsifier, torch.Tensor, perfect.PerfectNMTensor)
+    if reg is None or pf_key not in reg:
+        perfect.install(sten_module)
+    sten_module.PerfectNMTensor = perfect.PerfectNMTensor
+    sten_module.PerfectNMSparsifier = perfect.PerfectNMSparsifier

@@ -233,15 +233,20 @@ class GroupedNMTensor:
 
     def densefrag(self, reduce_dim):
         """The weight as the A operand of the dense matrix cores, [outputs, reduction] in
-        fragment order, expanded from the rowpack operand into fresh scratch.  It is as large as
-        the dense weight, so it is rebuilt per call unless ``spmm_opt["cache_dense"]`` is set
-        (inference on a frozen weight: trades the memory saving for one pass less per call)."""
+        fragment order, expanded from the rowpack operand.  It is as large as the dense weight.
+        It is kept until ``val`` changes (one copy per reduction direction), so a frozen weight,
+        or the forward and backward of one training step, pay the expansion once;
+        ``spmm_opt["cache_dense"] = False`` rebuilds it per call instead and keeps the memory of
+        the compressed format."""
         lay = self.layout
         lib = native.load()
-        key = (self.val.data_ptr(), self.val._version, self.idx.data_ptr(), reduce_dim)
-        cached = getattr(self, "_densefrag", None)
-        if self.spmm_opt.get("cache_dense") and cached is not None and cached[0] == key:
-            return cached[1]
+        key = (self.val.data_ptr(), self.val._version, self.idx.data_ptr())
+        keep = self.spmm_opt.get("cache_dense", True)
+        cache = getattr(self, "_densefrag", None)
+        if cache is None or cache.get("key") != key or not keep:
+            cache = self._densefrag = {"key": key}
+        if reduce_dim in cache:
+            return cache[reduce_dim]
         pk_val, pk_pat = self.rowpack()
         O, K = lay.dense_shape[1 - reduce_dim], lay.dense_shape[reduce_dim]
         elems = ctypes.c_int64(0)
@@ -252,7 +257,8 @@ class GroupedNMTensor:
             native.check(lib.nmg_densefrag(
                 native.ptr(pk_val), native.ptr(pk_pat), lay.G, lay.S, transpose, native.ptr(df),
                 lay.n, lay.m, native.dtype_code(df.dtype), native.stream_ptr(df.device)))
-        self._densefrag = (key, df) if self.spmm_opt.get("cache_dense") else None
+        if keep:
+            cache[reduce_dim] = df
         return df
 
     def dense_operand(self, reduce_dim):

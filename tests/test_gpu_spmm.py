@@ -289,6 +289,41 @@ def test_split_reduction_on_the_target_weight_at_intermediate_batches():
         assert rel_l2(to_np(y), to_np(x.double() @ Wd.t())) <= TOL[torch.float16]
 
 
+def test_target_weight_against_the_oracle_at_decode_and_large_batches():
+    # the north-star weight 4096 x 11008 2:4:16 compressed by the CPU oracle (val / idx compared
+    # bit for bit), then the product at 1 and 16 tokens (decode kernel) and 2048 tokens (direct
+    # kernel of the sparse matrix cores) against the fp64 product with the oracle's dense form
+    print("case target weight 4096x11008 vs oracle, T = 1, 16, 2048", flush=True)
+    W = seeded((4096, 11008), torch.float16, seed=11, std=0.02)
+    Wd, (val, idx, lay) = dense_ref(W, 2, 4, 16, 1)
+    w = make(W, 2, 4, 16, 1)
+    assert np.array_equal(to_np(w.idx), idx)
+    assert np.array_equal(to_np(w.val).view(np.uint16), val.view(np.uint16))
+    for T in (1, 16, 2048):
+        x = seeded((T, 11008), torch.float16, seed=12 + T)
+        y = sten.spmm(w, x.to(DEV), reduce_dim=1)
+        assert y.shape == (T, 4096)
+        assert rel_l2(to_np(y), to_np(x).astype(np.float64) @ Wd.T) <= TOL[torch.float16], f"T={T}"
+
+
+@pytest.mark.parametrize("T", [3, 16, 300])
+def test_one_of_eight_with_group_32_against_the_oracle(T):
+    # benchmark config 3's sparsest pattern (1:8, group 32: chunks of 256 lines) at a size the
+    # oracle compresses in seconds: decode kernel, split reduction and direct kernel
+    print(f"case 1:8:32 T={T}", flush=True)
+    W = seeded((1024, 1536), torch.float16, seed=21, std=0.05)
+    Wd, (val, idx, lay) = dense_ref(W, 1, 8, 32, 1)
+    w = make(W, 1, 8, 32, 1)
+    assert np.array_equal(to_np(w.idx), idx)
+    assert np.array_equal(to_np(w.val).view(np.uint16), val.view(np.uint16))
+    x = seeded((T, 1536), torch.float16, seed=22)
+    y = sten.spmm(w, x.to(DEV), reduce_dim=1)
+    assert rel_l2(to_np(y), to_np(x).astype(np.float64) @ Wd.T) <= TOL[torch.float16]
+    gy = seeded((T, 1024), torch.float16, seed=23)
+    gx = sten.spmm(w, gy.to(DEV), reduce_dim=0)
+    assert rel_l2(to_np(gx), to_np(gy).astype(np.float64) @ Wd) <= TOL[torch.float16]
+
+
 def test_sparse_matrix_cores_refuse_incompatible_patterns():
     w = make(seeded((64, 64), torch.float16, 1), 4, 8, 1, 1)     # 4:8 can keep 3 of an aligned 4
     with pytest.raises(sten.NmgError):
@@ -439,7 +474,7 @@ def _check_structure(w, n, m):
     return d
 
 
-@pytest.mark.parametrize("n,m", [(2, 8), (4, 8)])
+@pytest.mark.parametrize("n,m", [(1, 8), (2, 8), (4, 8)])
 def test_full_size_config3_forward(n, m):
     # benchmark config 3 at full size (8192 x 8192, group 32, 4096 tokens): structure of the
     # compressed weight, the product against the dense product of its own dense form, linearity

@@ -1,0 +1,99 @@
+"""The static check of hand-tracked loads (sten_amd/isa_check.py) on small synthetic kernels:
+it must see a register touched while its load is in flight, honour counted waits, carry the state
+of a loop into its next iteration, and tell spills inside a streaming loop from spills outside."""
+from sten_amd import isa_check as C
+
+
+def run(body):
+    C.notes.clear()
+    return C.check_kernel("_Zk", body.strip("\n").split("\n"))
+
+
+def test_touch_before_wait_is_found():
+    p = run("""
+\tglobal_load_dwordx4 v[4:7], v1, s[2:3]
+\tv_mov_b32_e32 v9, v5
+\ts_waitcnt vmcnt(0)
+""")
+    assert len(p) == 1 and "v_mov_b32_e32 v9, v5" in p[0]
+
+
+def test_wait_clears_and_counts_in_order():
+    clean = run("""
+\tglobal_load_dwordx4 v[4:7], v1, s[2:3]
+\tglobal_load_dwordx4 v[8:11], v1, s[2:3] offset:1024
+\ts_waitcnt vmcnt(1)
+\tv_mov_b32_e32 v20, v5
+\ts_waitcnt vmcnt(0)
+\tv_mov_b32_e32 v21, v9
+""")
+    assert clean == []
+    early = run("""
+\tglobal_load_dwordx4 v[4:7], v1, s[2:3]
+\tglobal_load_dwordx4 v[8:11], v1, s[2:3] offset:1024
+\ts_waitcnt vmcnt(1)
+\tv_mov_b32_e32 v21, v9
+""")
+    assert len(early) == 1
+
+
+def test_dma_loads_count_but_write_no_register():
+    p = run("""
+\tglobal_load_dwordx4 v[4:7], v1, s[2:3]
+\tglobal_load_lds_dwordx4 v2, s[4:5]
+\ts_waitcnt vmcnt(1)
+\tv_add_u32_e32 v2, 1, v2
+\tv_mov_b32_e32 v20, v4
+""")
+    assert p == []
+
+
+def test_state_carried_around_a_loop():
+    # the load at the end of the body is consumed at its top: fine with a wait there, a hazard without
+    good = run("""
+\tglobal_load_dword v4, v1, s[2:3]
+.LBB0_1:
+\ts_waitcnt vmcnt(0)
+\tv_mov_b32_e32 v9, v4
+\tglobal_load_dword v4, v1, s[2:3]
+\ts_cbranch_scc1 .LBB0_1
+\ts_waitcnt vmcnt(0)
+""")
+    assert good == []
+    bad = run("""
+\tglobal_load_dword v4, v1, s[2:3]
+\ts_waitcnt vmcnt(0)
+.LBB0_1:
+\tv_mov_b32_e32 v9, v4
+\tglobal_load_dword v4, v1, s[2:3]
+\ts_cbranch_scc1 .LBB0_1
+\ts_waitcnt vmcnt(0)
+""")
+    assert len(bad) == 1 and "second iteration" in bad[0]
+
+
+def test_spill_of_a_register_in_flight_and_spill_in_a_streaming_loop():
+    p = run("""
+\tglobal_load_dword v4, v1, s[2:3]
+\tscratch_store_dword off, v4, off
+\ts_waitcnt vmcnt(0)
+""")
+    assert len(p) == 1 and "scratch_store_dword" in p[0]
+    p = run("""
+.LBB0_1:
+\tglobal_load_dword v4, v1, s[2:3]
+\tscratch_store_dword off, v30, off
+\ts_waitcnt vmcnt(0)
+\ts_cbranch_scc1 .LBB0_1
+""")
+    assert len(p) == 1 and "inside a loop" in p[0]
+    p = run("""
+\tscratch_store_dword off, v30, off
+.LBB0_1:
+\tglobal_load_dword v4, v1, s[2:3]
+\ts_waitcnt vmcnt(0)
+\ts_cbranch_scc1 .LBB0_1
+\tscratch_load_dword v30, off, off
+\ts_waitcnt vmcnt(0)
+""")
+    assert p == [] and len(C.notes) == 2

@@ -77,6 +77,29 @@ def test_hip_linear_matches_dequantised_matmul(M, K, T):
 
 
 @pytest.mark.gpu
+def test_full_size_config4():
+    # benchmark config 4 at its real size: 11008 x 4096 pruned 2:4 along K, int4 with one scale per
+    # 128 positions; packing bit-exact against the restatement, the product at 1, 4 and 16 tokens
+    # against the dequantised fp64 matmul.  (Parity against the reference is unpinned: see above.)
+    import sten_amd as sten
+    print("case w4 full size 11008x4096, T = 1, 4, 16", flush=True)
+    M, K = 11008, 4096
+    w = seeded((M, K), torch.float16, seed=44, std=0.02)
+    t = sten.SparseMarlinTensor.from_dense(w.to("cuda:0"))
+    pos, q, s = W.prune_quantise(to_np(w))
+    B, meta, sc = W.pack(pos, q, s, M, K)
+    assert np.array_equal(to_np(t.B), B)
+    assert np.array_equal(to_np(t.meta).view(np.uint32), meta)
+    assert np.array_equal(to_np(t.s).view(np.uint16), sc.view(np.uint16))
+    wd = W.dequantise(pos, q, s, K)
+    for T in (1, 4, 16):
+        x = seeded((T, K), torch.float16, seed=45 + T)
+        y = t.linear(x.to("cuda:0"))
+        assert y.shape == (T, M)
+        assert rel_l2(to_np(y), W.linear(wd, to_np(x))) <= 1e-3, f"T={T}"
+
+
+@pytest.mark.gpu
 def test_registered_linear_like_the_reference_test():
     # tests/test_sparse_marlin.py:119-133 sparsifies every MLP weight of a model and runs it; here
     # a local two-layer MLP stands in for the hub model
