@@ -274,3 +274,38 @@ def linear(x, val, idx, lay, bias=None):
     if bias is not None:
         y = y + bias
     return y
+
+
+def perfect_nm(x, n, m, sparse_dim):
+    """Ungrouped n:m, restating PerfectNMTensor.from_dense (grouped_nm_tensor.py:1018-1046): pad the
+    sparse dim to a multiple of m, split it into (blocks, m), sort the magnitudes of a block in
+    descending order and keep the first n.  Returns (val, idx) with the sparse dim replaced by
+    (blocks, n).  The reference's argsort is unstable, so it leaves the order of equal magnitudes
+    open; here equal magnitudes keep the lower position first (a stable sort) and NaN sorts first."""
+    sparse_dim %= x.ndim
+    S = x.shape[sparse_dim]
+    blocks = -(-S // m)
+    pad = [(0, 0)] * x.ndim
+    pad[sparse_dim] = (0, blocks * m - S)
+    y = np.moveaxis(np.pad(x, pad), sparse_dim, -1)
+    y = y.reshape(*y.shape[:-1], blocks, m)
+    mag = np.abs(y.astype(np.float64))
+    mag = np.where(np.isnan(mag), np.inf, mag)
+    order = np.argsort(-mag, axis=-1, kind="stable")[..., :n]
+    val = np.take_along_axis(y, order, axis=-1)
+    nd = val.ndim
+    perm = list(range(sparse_dim)) + [nd - 2, nd - 1] + list(range(sparse_dim, nd - 2))
+    return np.ascontiguousarray(np.transpose(val, perm)), np.ascontiguousarray(np.transpose(order, perm)).astype(np.int64)
+
+
+def perfect_nm_to_dense(val, idx, m, sparse_dim, size):
+    """Inverse scatter (grouped_nm_tensor.py:1048-1065)."""
+    full = list(val.shape)
+    full[sparse_dim + 1] = m
+    dense = np.zeros(full, dtype=val.dtype)
+    np.put_along_axis(dense, idx, val, axis=sparse_dim + 1)
+    merged = full[:sparse_dim] + [full[sparse_dim] * m] + full[sparse_dim + 2:]
+    dense = dense.reshape(merged)
+    sl = [slice(None)] * dense.ndim
+    sl[sparse_dim] = slice(0, size)
+    return np.ascontiguousarray(dense[tuple(sl)])
