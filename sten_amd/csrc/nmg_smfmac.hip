@@ -19,6 +19,9 @@
 // A fragments go global -> registers (already in lane order, fully coalesced); the activation
 // tile goes global -> registers -> LDS (double buffered), one barrier per 64-wide K step.
 #include "nmg_common.h"
+
+#include <map>
+#include <mutex>
 #include "nmg_tile.h"
 
 #include <algorithm>
@@ -1431,3 +1434,61 @@ extern "C" int nmg_spmm_smfmac_splitk(const void *d_fp_val, const void *d_fp_idx
     return dtype == NMG_F16 ? launch_smfmac_direct<__half, 2, 4, 4, 1, 2>(P, s)
                             : launch_smfmac_direct<__hip_bfloat16, 2, 4, 4, 1, 2>(P, s);
 }
+
+// ---- the split reduction for callers that cannot allocate -----------------------------------
+// Same kernels as nmg_spmm_smfmac_splitk; the single-precision partial sums of the slices go to a
+// file-scope array of this library instead of a workspace the caller brings.  Each GPU holds its
+// own copy of the array (until the process ends) at its own address, looked up once per device.
+// Every call on a GPU uses that GPU's array: calls that overlap on one GPU (two streams) race.
+// Nothing in it has to start at zero -- a call reads only what its own slices wrote -- so it is
+// never cleared, and a call may follow a larger one.
+namespace nmg {
+constexpr int64_t kSplitkScratchBytes = (int64_t)32 << 20;
+static __device__ __align__(256) unsigned char g_splitk_scratch[kSplitkScratchBytes];
+static std::mutex g_scratch_mu;
+static std::map<int, void *> g_scratch_ptr;   // device -> address of its copy
+
+static int splitk_scratch(void **ptr)
+{
+    int dev = 0;
+    NMG_HIP_TRY(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    auto it = g_scratch_ptr.find(dev);
+    if (it == g_scratch_ptr.end()) {
+        void *p = nullptr;
+        NMG_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(g_splitk_scratch)));
+        it = g_scratch_ptr.emplace(dev, p).first;
+    }
+    *ptr = it->second;
+    return NMG_OK;
+}
+}  // namespace nmg
+
+extern "C" int64_t nmg_noalloc_scratch_bytes(void) { return kSplitkScratchBytes; }
+
+extern "C" int nmg_noalloc_prepare(void)
+{
+    void *p = nullptr;
+    return splitk_scratch(&p);
+}
+
+extern "C" int nmg_spmm_smfmac_splitk_noalloc(const void *d_fp_val, const void *d_fp_idx, int64_t M, int64_t K,
+                                              const void *d_x, int64_t ldx, void *d_y, int64_t ldy,
+                                              const void *d_bias, int64_t T, int dtype, int slices, void *stream)
+{
+    NMG_REQUIRE(M >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
+    if (slices > 1) {
+        const int64_t tiles_m = (M + 255) / 256;
+        const int64_t need = (int64_t)slices * T * tiles_m * 256 * 4;
+        NMG_REQUIRE(need <= kSplitkScratchBytes, NMG_ERR_UNSUPPORTED,
+                    "%d slices of %lld tokens x %lld features need %lld bytes of partial sums; the built-in "
+                    "scratch holds %lld (use nmg_spmm_smfmac_splitk with a workspace of your own)",
+                    slices, (long long)T, (long long)(tiles_m * 256), (long long)need,
+                    (long long)kSplitkScratchBytes);
+    }
+    void *ws = nullptr;
+    if (int rc = splitk_scratch(&ws)) return rc;
+    return nmg_spmm_smfmac_splitk(d_fp_val, d_fp_idx, M, K, d_x, ldx, d_y, ldy, d_bias, T, dtype, slices, ws,
+                                  kSplitkScratchBytes, stream);
+}
+
