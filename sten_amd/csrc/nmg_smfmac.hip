@@ -527,7 +527,14 @@ template <typename T> static int launch_smfmac_pipe(SmfParams &P, hipStream_t s)
 constexpr int DR_D = 3;                 // K steps in flight
 constexpr int DR_NS = 4;                // activation stages in LDS (>= DR_D + 1)
 
-template <typename T, int FB, int TB, int WM, int WN, int NH>
+//
+// XT = true is the product with both dense operands transposed, C[M, T] = W * B for B [K, T]
+// (what torch.mm(W, B) asks for): the activation tile of a K step is then 64 reduction rows x TT
+// tokens, fetched as it lies in memory, and an activation fragment -- a lane wants 16 consecutive
+// reduction positions of its token -- is four LDS transpose reads (DS_READ_B64_TR_B16: in every
+// group of 16 lanes, lane i receives as element j the 16-bit element i%4 of the 8 bytes addressed
+// by lane 4j + i/4); the epilogue stages [feature][token] and stores token-contiguous rows.
+template <typename T, int FB, int TB, int WM, int WN, int NH, bool XT = false>
 __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
 {
     using S = Smf<T>;
@@ -577,16 +584,30 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
         ai_base[fb] = (const unsigned char *)P.fp_idx + ((int64_t)(mb0 + fb) * KPT + kp_lo) * 256;
     }
     const uint32_t lane16 = lane * 16, lane4 = lane * 4;
-    const unsigned char *x_base = (const unsigned char *)P.x + (int64_t)kp_lo * 128;
+    // K step kp of the activations starts kp * XSTEP bytes into the operand
+    const int64_t XSTEP = XT ? 64 * P.ldx * 2 : 128;
+    const unsigned char *x_base = (const unsigned char *)P.x + (int64_t)kp_lo * XSTEP;
     uint32_t x_off[XL];
 #pragma unroll
     for (int i = 0; i < XL; i++) {
-        const int row = (wave * XL + i) * 8 + (lane >> 3);
-        const int piece = lane & 7;
-        const int q = piece ^ ((row >> 1) & 7);
-        int64_t tok = t0 + row;
-        if (tok >= P.T) tok = P.T - 1;
-        x_off[i] = (uint32_t)((tok * P.ldx + q * 8) * 2);
+        if constexpr (XT) {
+            // a DMA load fills 1 KiB = 1024 / (TT * 2) reduction rows of the tile; piece p (8 tokens)
+            // of row k holds the logical chunk p ^ 4*(k%4), which spreads the transpose reads
+            // of four consecutive rows over all banks
+            constexpr int PPR = TT / 8;                       // 16-byte pieces per row
+            const int row = (wave * XL + i) * (64 / PPR) + lane / PPR;
+            const int chunk = (lane % PPR) ^ ((row & 3) << 2);
+            int64_t tok = t0 + chunk * 8;
+            if (tok > P.T - 8) tok = (P.T - 1) / 8 * 8;       // clamped columns are computed, never stored
+            x_off[i] = (uint32_t)((row * P.ldx + tok) * 2);
+        } else {
+            const int row = (wave * XL + i) * 8 + (lane >> 3);
+            const int piece = lane & 7;
+            const int q = piece ^ ((row >> 1) & 7);
+            int64_t tok = t0 + row;
+            if (tok >= P.T) tok = P.T - 1;
+            x_off[i] = (uint32_t)((tok * P.ldx + q * 8) * 2);
+        }
     }
 
     struct WSet {
@@ -601,7 +622,7 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
         if (kp >= KP) kp = KP - 1;
         if (i < XL) {
             unsigned char *base = smem + (kp & (DR_NS - 1)) * STAGE;
-            const unsigned char *xb = x_base + (int64_t)kp * 128;
+            const unsigned char *xb = x_base + (int64_t)kp * XSTEP;
 #pragma unroll
             for (int q = 0; q < XL; q++)
                 if (q == i)
@@ -664,12 +685,39 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
         u32x4 b[BT][2];
     };
     BFrags fr[2];
+    // XT: lane (g = l/16, i = l%16) of a transpose read supplies the 8 bytes at reduction row
+    // 16*(g/2) + i/4 (+ 32*ks + 4*r), tokens 16*(g%2) + 4*(i%4) .. +3 of the 32-token block, and
+    // receives token l%32 at rows 16*(l/32) + 4r + 0..3: reads r = 0..3 are the lane's 16 positions.
+    int t_off[TB];
+    if constexpr (XT) {
+        const int g = lane >> 4, i16 = lane & 15, a = i16 >> 2;
+#pragma unroll
+        for (int tb = 0; tb < TB; tb++) {
+            const int chunk = (wn * TB + tb) * 4 + 2 * (g & 1) + ((i16 & 3) >> 1);   // 8-token chunk of the row
+            t_off[tb] = (16 * (g >> 1) + a) * (TT * 2) + ((chunk ^ (a << 2)) << 4) + (i16 & 1) * 8;
+        }
+    }
     auto read_b = [&](BFrags &f, const unsigned char *base, int ph) {
         const int ks = ph / NH, hh = ph % NH;
 #pragma unroll
         for (int t = 0; t < BT; t++) {
-            f.b[t][0] = *(const u32x4 *)(base + b_off[ks][0] + (hh * BT + t) * 32 * 128);
-            f.b[t][1] = *(const u32x4 *)(base + b_off[ks][1] + (hh * BT + t) * 32 * 128);
+            if constexpr (XT) {
+                typedef short i16x4 __attribute__((ext_vector_type(4)));
+                typedef __attribute__((address_space(3))) i16x4 *lds_i16x4;
+                union {
+                    i16x4 h[4];
+                    u32x4 u[2];
+                } c;
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    c.h[r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (lds_i16x4)(base + t_off[hh * BT + t] + (32 * ks + 4 * r) * (TT * 2)));
+                f.b[t][0] = c.u[0];
+                f.b[t][1] = c.u[1];
+            } else {
+                f.b[t][0] = *(const u32x4 *)(base + b_off[ks][0] + (hh * BT + t) * 32 * 128);
+                f.b[t][1] = *(const u32x4 *)(base + b_off[ks][1] + (hh * BT + t) * 32 * 128);
+            }
         }
     };
     // MFMAs lo..hi-1 of phase PH, numbered fb * BT + t
@@ -800,11 +848,16 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
         return;
     }
     const TileOut out{P.y, P.bias, P.M, P.T, P.ldy};
-    smf_store_tile<T, FB, TB>(acc, smem + wave * (TB * 32 * (FB * 64 + 16)), lane, f0 + wm * FB * 32,
-                              t0 + wn * TB * 32, out);
+    if constexpr (XT)
+        smf_store_tile_t<T, FB, TB>(acc, smem + wave * (FB * 32 * (TB * 64 + 16)), lane, f0 + wm * FB * 32,
+                                    t0 + wn * TB * 32, out);
+    else
+        smf_store_tile<T, FB, TB>(acc, smem + wave * (TB * 32 * (FB * 64 + 16)), lane, f0 + wm * FB * 32,
+                                  t0 + wn * TB * 32, out);
 }
 
-template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_smfmac_direct(SmfParams &P, hipStream_t s)
+template <typename T, int FB, int TB, int WM, int WN, int NH, bool XT = false>
+static int launch_smfmac_direct(SmfParams &P, hipStream_t s)
 {
     constexpr int TF = WM * FB * 32, TT = WN * TB * 32;
     static_assert(TF == 256, "the operand is padded to 256 lines");
@@ -812,10 +865,12 @@ template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_
     P.tiles_n = (int)((P.T + TT - 1) / TT);
     const int slices = P.ksplit > 1 ? P.ksplit : 1;
     dim3 grid((unsigned)(P.tiles_m * P.tiles_n * slices));
-    constexpr size_t ring = (size_t)DR_NS * TT * 128, stg = (size_t)4 * TB * 32 * (FB * 64 + 16);
+    constexpr size_t ring = (size_t)DR_NS * TT * 128;
+    constexpr size_t stg = XT ? (size_t)4 * FB * 32 * (TB * 64 + 16) : (size_t)4 * TB * 32 * (FB * 64 + 16);
     constexpr size_t lds = ring > stg ? ring : stg;
     static_assert(lds <= 160 * 1024, "LDS");
-    auto k = spmm_smfmac_direct_kernel<T, FB, TB, WM, WN, NH>;
+    static_assert(!XT || (TT == 128 && WN == 1), "the transposed tile is 64 rows of 128 tokens");
+    auto k = spmm_smfmac_direct_kernel<T, FB, TB, WM, WN, NH, XT>;
     NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(k, grid, dim3(256), lds, s, P);
     NMG_HIP_TRY(hipGetLastError());
@@ -1433,6 +1488,38 @@ extern "C" int nmg_spmm_smfmac_splitk(const void *d_fp_val, const void *d_fp_idx
     hipStream_t s = (hipStream_t)stream;
     return dtype == NMG_F16 ? launch_smfmac_direct<__half, 2, 4, 4, 1, 2>(P, s)
                             : launch_smfmac_direct<__hip_bfloat16, 2, 4, 4, 1, 2>(P, s);
+}
+
+// ---- both dense operands transposed: C[M, T] = W * B (+ bias per row), B [K, T] ------------------
+extern "C" int nmg_spmm_smfmac_tt(const void *d_fp_val, const void *d_fp_idx, int64_t M, int64_t K,
+                                  const void *d_b, int64_t ldb, void *d_c, int64_t ldc, const void *d_bias,
+                                  int64_t T, int dtype, void *stream)
+{
+    NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED,
+                "the sparse matrix cores take f16/bf16 only");
+    NMG_REQUIRE(M >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
+    NMG_REQUIRE(ldb >= T && ldc >= T, NMG_ERR_ARG, "leading dimension smaller than row length");
+    NMG_REQUIRE((K % 64) == 0 && K > 0 && (ldb % 8) == 0 && ((uintptr_t)d_b % 16) == 0, NMG_ERR_UNSUPPORTED,
+                "the transposed product needs K %% 64 == 0, ldb %% 8 == 0 and a 16-byte aligned B");
+    NMG_REQUIRE(ldb < ((int64_t)1 << 24), NMG_ERR_UNSUPPORTED, "leading dimension too large");
+    if (M == 0 || T == 0) return NMG_OK;
+    NMG_REQUIRE(d_fp_val && d_fp_idx && d_b && d_c, NMG_ERR_ARG, "null device pointer");
+    SmfParams P{};
+    P.fp_val = d_fp_val;
+    P.fp_idx = (const uint32_t *)d_fp_idx;
+    P.x = d_b;
+    P.y = d_c;
+    P.bias = d_bias;
+    P.M = M;
+    P.K = K;
+    P.T = T;
+    P.ldx = ldb;
+    P.ldy = ldc;
+    P.MB = (int)((M + 255) / 256 * 8);
+    P.KP = (int)(K / 64);
+    hipStream_t s = (hipStream_t)stream;
+    return dtype == NMG_F16 ? launch_smfmac_direct<__half, 2, 4, 4, 1, 2, true>(P, s)
+                            : launch_smfmac_direct<__hip_bfloat16, 2, 4, 4, 1, 2, true>(P, s);
 }
 
 // ---- the split reduction for callers that cannot allocate -----------------------------------

@@ -91,6 +91,65 @@ __device__ __forceinline__ void smf_store_tile(const f32x16 (&acc)[FB][TB], unsi
     }
 }
 
+// The same epilogue for a transposed output, Y[M, T] row-major (tokens contiguous): the
+// wavefront's FB*32 features x TB*32 tokens are staged as [feature][token], so that a lane stores
+// 16 bytes = 8 tokens of one feature row and TB*64 bytes per row are contiguous.  The bias of a
+// feature is added to its whole row.
+template <typename T, int FB, int TB>
+__device__ __forceinline__ void smf_store_tile_t(const f32x16 (&acc)[FB][TB], unsigned char *stg, int lane,
+                                                 int64_t fw, int64_t tw, const TileOut &P)
+{
+    constexpr int ROW = TB * 64 + 16;       // bytes per staged feature row
+    constexpr int CPR = TB * 4;             // 16-byte chunks per row
+    constexpr int RPP = 64 / CPR;           // feature rows per pass of the wavefront
+    const int j = lane & 31, h = lane >> 5;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int tb = 0; tb < TB; tb++)
+#pragma unroll
+        for (int fb = 0; fb < FB; fb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int f = fb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                *(uint16_t *)(stg + f * ROW + (tb * 32 + j) * 2) = f32_to_bits16(acc[fb][tb][r], (T *)nullptr);
+            }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    uint16_t *Y = (uint16_t *)P.y;
+    const T *bias = (const T *)P.bias;
+    const bool vec_ok = (P.ldy & 7) == 0 && ((uintptr_t)P.y & 15) == 0;
+    const int tc = lane % CPR;                      // 8-token chunk of the row
+    const int64_t tok = tw + tc * 8;
+#pragma unroll 4
+    for (int it = 0; it < FB * 32 / RPP; it++) {
+        const int fl = it * RPP + lane / CPR;
+        const int64_t f = fw + fl;
+        u32x4 v = *(const u32x4 *)(stg + fl * ROW + tc * 16);
+        if (f >= P.M || tok >= P.T) continue;
+        if (bias) {
+            const float bv = to_f32(bias[f]);
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint16_t lo = (uint16_t)(w[i] & 0xFFFF), hi = (uint16_t)(w[i] >> 16);
+                T tlo = *reinterpret_cast<T *>(&lo), thi = *reinterpret_cast<T *>(&hi);
+                lo = f32_to_bits16(to_f32(tlo) + bv, (T *)nullptr);
+                hi = f32_to_bits16(to_f32(thi) + bv, (T *)nullptr);
+                w[i] = (uint32_t)lo | ((uint32_t)hi << 16);
+            }
+            v.x = w[0]; v.y = w[1]; v.z = w[2]; v.w = w[3];
+        }
+        uint16_t *dst = Y + f * P.ldy + tok;
+        if (vec_ok && tok + 7 < P.T) {
+            *(u32x4 *)dst = v;
+        } else {
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                if (tok + i < P.T) dst[i] = (uint16_t)(w[i >> 1] >> ((i & 1) * 16));
+        }
+    }
+}
+
 // ---- reductions cut into slices (products with fewer tiles than the GPU has CUs) ----
 // Slice s of a tile stores its sums in single precision at part[s][token][feature] (part_ld
 // features per token, a multiple of 256: the padded features of the last tile are stored too);

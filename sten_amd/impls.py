@@ -8,7 +8,7 @@ functions: this package's own ``dispatch`` module, or a real ``sten``.
 """
 import torch
 
-from .tensor import GroupedNMTensor, spmm
+from .tensor import GroupedNMTensor, spmm, spmm_tt
 
 
 class GroupedNMSparsifier:
@@ -111,7 +111,7 @@ def install(api):
     def mm_fwd(ctx, inputs, output_sparsifiers):
         weight, b = inputs
         ctx.save_for_backward(weight, b)
-        return spmm(weight.wrapped_tensor, b.t().contiguous(), reduce_dim=1).t()
+        return spmm_tt(weight.wrapped_tensor, b)
 
     def mm_bwd_common(ctx, grad_outputs, compressed):
         weight, b = ctx.saved_tensors

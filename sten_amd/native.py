@@ -73,6 +73,7 @@ SIGNATURES = {
     "nmg_noalloc_scratch_bytes": (_I64, []),
     "nmg_noalloc_prepare": (_I, []),
     "nmg_spmm_smfmac_splitk_noalloc": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _P]),
+    "nmg_spmm_smfmac_tt": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _P]),
     "nmg_gemm_nt": (_I, [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I, _P]),
 }
 

@@ -354,6 +354,36 @@ class GroupedNMTensor:
                 f"device={self.val.device})")
 
 
+def spmm_tt(weight, b):
+    """C = W @ B for a 2-D ``GroupedNMTensor`` W [R, C] and a dense B [C, N] (``torch.mm``), without
+    transposing copies when the sparse matrix cores can take it (16-bit, 2-of-4 compatible pattern
+    along dim 1, C % 64 == 0, more than 16 columns, B row-contiguous with a row pitch that is a
+    multiple of 8); otherwise through ``spmm`` on the transposed operands."""
+    lay = weight.layout
+    native.require_gpu(b, weight.val)
+    R, C = lay.dense_shape
+    if b.dim() != 2 or b.shape[0] != C:
+        raise native.NmgError(f"B must be [{C}, N], got {tuple(b.shape)}")
+    if b.dtype != weight.val.dtype:
+        raise native.NmgError(f"dtype mismatch: B {b.dtype}, weight {weight.val.dtype}")
+    N = b.shape[1]
+    direct = (lay.sparse_dim == 1 and b.dtype in (torch.float16, torch.bfloat16) and C % 64 == 0 and N > 16
+              and weight.spmm_opt.get("kernel", "auto") in ("auto", "smfmac"))
+    if direct and b.stride(1) != 1:
+        b = b.contiguous()
+    if direct and (b.stride(0) % 8 != 0 or b.data_ptr() % 16 != 0):
+        direct = False
+    packed = weight.fragpack() if direct else None
+    if packed is None:
+        return spmm(weight, b.t().contiguous(), reduce_dim=1).t()
+    c = torch.empty((R, N), dtype=b.dtype, device=b.device)
+    with torch.cuda.device(b.device):
+        native.check(native.load().nmg_spmm_smfmac_tt(
+            native.ptr(packed[0]), native.ptr(packed[1]), R, C, native.ptr(b), b.stride(0), native.ptr(c), N,
+            None, N, native.dtype_code(b.dtype), native.stream_ptr(b.device)))
+    return c
+
+
 def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
     """Y = X @ op(W) for a 2-D ``GroupedNMTensor`` W of shape [R, C].
 

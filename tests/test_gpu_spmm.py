@@ -324,6 +324,65 @@ def test_one_of_eight_with_group_32_against_the_oracle(T):
     assert rel_l2(to_np(gx), to_np(gy).astype(np.float64) @ Wd) <= TOL[torch.float16]
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("R,C,N,n,m,g", [
+    (256, 256, 128, 2, 4, 16),      # one tile
+    (300, 192, 100, 2, 4, 4),       # ragged rows and columns (N % 8 != 0 goes through a padded pitch)
+    (520, 448, 264, 1, 8, 2),       # several tiles both ways
+    (1024, 1024, 1000, 2, 8, 4),
+    (768, 3072, 4096, 2, 4, 16),    # the shape of the reference's own matmul test (dace_gnm_mult.py:1183)
+])
+def test_product_with_both_dense_operands_transposed(dtype, R, C, N, n, m, g):
+    # torch.mm(W, B): C[R, N] = W @ B with B [C, N] as it lies in memory (no transposing copies),
+    # against the fp64 product with the oracle's dense form, and against the copying route
+    print(f"case spmm_tt {dtype} R={R} C={C} N={N} {n}:{m}:{g}", flush=True)
+    W = seeded((R, C), dtype, seed=R + C, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, 1)
+    w = make(W, n, m, g, 1)
+    b = seeded((C, N), dtype, seed=9)
+    ref = Wd @ to_np(b).astype(np.float64)
+    pitch = -(-N // 8) * 8
+    bb = torch.zeros(C, pitch, dtype=dtype, device=DEV)[:, :N]
+    bb.copy_(b)
+    c = sten.spmm_tt(w, bb)
+    assert c.shape == (R, N) and c.is_contiguous()
+    assert rel_l2(to_np(c), ref) <= TOL[dtype]
+    c2 = sten.spmm(w, b.to(DEV).t().contiguous(), reduce_dim=1).t()
+    assert rel_l2(to_np(c), to_np(c2)) <= 2 * TOL[dtype]
+    # the C ABI with a bias per row and a padded output pitch
+    lib = native.load()
+    fp_val, fp_idx = w.fragpack()
+    bias = seeded((R,), dtype, seed=10).to(DEV)
+    out = torch.full((R, pitch + 8), 7.0, dtype=dtype, device=DEV)
+    native.check(lib.nmg_spmm_smfmac_tt(native.ptr(fp_val), native.ptr(fp_idx), R, C, native.ptr(bb), pitch,
+                                        native.ptr(out), pitch + 8, native.ptr(bias), N, native.dtype_code(dtype),
+                                        None))
+    torch.cuda.synchronize()
+    assert rel_l2(to_np(out[:, :N]), ref + to_np(bias).astype(np.float64)[:, None]) <= TOL[dtype]
+    assert bool((out[:, N:] == 7.0).all()), "columns beyond N must stay untouched"
+
+
+def test_transposed_product_argument_errors():
+    lib = native.load()
+    w = make(seeded((64, 128), torch.float16, 1), 2, 4, 4, 1)
+    fp_val, fp_idx = w.fragpack()
+    b = torch.zeros(128, 40, dtype=torch.float16, device=DEV)
+    c = torch.zeros(64, 40, dtype=torch.float16, device=DEV)
+    args = lambda K, ldb, dt: (native.ptr(fp_val), native.ptr(fp_idx), 64, K, native.ptr(b), ldb, native.ptr(c), 40,
+                               None, 40, dt, None)
+    assert lib.nmg_spmm_smfmac_tt(*args(128, 40, native.NMG_F16)) == 0
+    assert lib.nmg_spmm_smfmac_tt(*args(100, 40, native.NMG_F16)) == 2      # K % 64
+    assert lib.nmg_spmm_smfmac_tt(*args(128, 36, native.NMG_F16)) == 1      # ldb < T
+    assert lib.nmg_spmm_smfmac_tt(*args(128, 44, native.NMG_F16)) == 2      # ldb % 8
+    assert lib.nmg_spmm_smfmac_tt(*args(128, 40, native.NMG_F32)) == 2
+    torch.cuda.synchronize()
+    # torch.mm through the dispatcher takes this route and matches the dense product
+    sp = sten.SparseTensorWrapper.wrapped_from_dense(w, w.to_dense(), None)
+    bm = torch.randn(128, 96, device=DEV).half()
+    got = torch.mm(sp, bm)
+    assert rel_l2(to_np(got), to_np(w.to_dense().double() @ bm.double())) <= TOL[torch.float16]
+
+
 def test_sparse_matrix_cores_refuse_incompatible_patterns():
     w = make(seeded((64, 64), torch.float16, 1), 4, 8, 1, 1)     # 4:8 can keep 3 of an aligned 4
     with pytest.raises(sten.NmgError):
