@@ -258,248 +258,6 @@ __global__ __launch_bounds__(64 * WM * WN, MINW) void spmm_smfmac_kernel(SmfPara
     }
 }
 
-constexpr int PIPE_OUT_ROW = 128 * 2 + 16;  // epilogue staging: one token row of a matrix wavefront
-
-// ------------------------------------------------------------------------ pipelined kernel
-// Same math, deeper memory pipeline and specialised wavefronts.
-//
-// Weight fragments, index words and the activation tile all travel global -> LDS with the
-// LDS-DMA form of global_load (no registers involved) into a ring of PIPE_NS stages, so
-// PIPE_NS-1 K steps of loads are in flight while one is being multiplied: HBM / fabric latency
-// is several K steps long, which a one-step register prefetch cannot cover.
-//
-// A workgroup has 8 wavefronts: 4 "matrix" wavefronts (one per SIMD, 128 features x 64 tokens
-// each) that only read fragments from LDS and issue MFMAs, and 4 "loader" wavefronts that only
-// issue the DMA loads and track their completion (s_waitcnt vmcnt is per wavefront).  A single
-// wavefront per SIMD is issue-bound: the DMA instructions, their address arithmetic and M0
-// updates do not fit in the shadow of its own MFMAs; a second wavefront on the SIMD issues them
-// in parallel.  One s_barrier per K step: loaders arrive when step kp+1 has landed, matrix
-// wavefronts when they hold all of step kp in registers; after it the loaders refill slot kp
-// and the matrix wavefronts start on step kp+1.
-//
-// Stage layout (bytes): [8 feature blocks x 2 k-steps x 1024] weight values in lane order,
-// [8 x 256] index words, [128 token rows x 128] activations.  A DMA load writes 64 lanes x 16 B
-// contiguously, so the activation rows cannot be padded; instead the 16-byte chunks of a row
-// are XOR-swizzled with (row/2)%8, chosen on the global side, which makes the fragment reads
-// (32 rows x 16 B at one logical chunk) conflict-free.
-// Requires K % 64 == 0 and activations smaller than 2 GiB (32-bit lane offsets).
-// Workgroup tile 256 features x 128 tokens.
-constexpr int PIPE_NS = 4;
-constexpr int PIPE_AVAL = 8 * 2 * 1024;
-constexpr int PIPE_AIDX = 8 * 256;
-constexpr int PIPE_X = 128 * 128;
-constexpr int PIPE_STAGE = PIPE_AVAL + PIPE_AIDX + PIPE_X;
-constexpr int PIPE_LPT = 10;  // DMA loads per loader thread per stage: 4 weight + 2 index + 4 activation
-
-
-template <typename T>
-__global__ __launch_bounds__(512, 2) void spmm_smfmac_pipe_kernel(SmfParams P)
-{
-    using S = Smf<T>;
-    constexpr int FB = 4, TB = 2;
-    extern __shared__ __align__(16) unsigned char smem[];
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-
-    // Workgroup -> tile.  Consecutive ids are dealt round-robin to the 8 XCDs; give each XCD a
-    // contiguous run of ids, and walk the tile grid in bands of 4 feature tiles so that a run
-    // covers a compact block of tiles (weight rows and activation rows both reused from that
-    // XCD's L2).
-    int id = blockIdx.x;
-    const int ntiles = P.tiles_m * P.tiles_n;
-    if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
-    constexpr int GH = 4;
-    const int band = id / (GH * P.tiles_n);
-    const int band_h = min(P.tiles_m - band * GH, GH);
-    const int in_band = id - band * GH * P.tiles_n;
-    const int tile_m = band * GH + in_band % band_h, tile_n = in_band / band_h;
-    const int64_t f0 = (int64_t)tile_m * 256, t0 = (int64_t)tile_n * 128;
-    const int KP = P.KP, KS = KP * 2;
-    const int mbT = (int)(f0 / 32);
-
-    if (wave >= 4) {
-        // ============================== loader wavefronts ==============================
-        const int lw = wave - 4;
-        const unsigned char *av_base = (const unsigned char *)P.fp_val + (int64_t)mbT * KS * 1024;
-        const unsigned char *ai_base = (const unsigned char *)P.fp_idx + (int64_t)mbT * KP * 256;
-        const unsigned char *x_base = (const unsigned char *)P.x;
-        // weight values: loader lw moves fragments fi = 4lw..4lw+3 (fi = fb*2 + ks) of every stage
-        uint32_t av_off[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int fi = lw * 4 + i, fb = fi >> 1, ks = fi & 1;
-            av_off[i] = (uint32_t)(((fb * KS + ks) * 64 + lane) * 16);
-        }
-        // index words: loader lw moves feature blocks 2lw, 2lw+1
-        uint32_t ai_off[2];
-#pragma unroll
-        for (int i = 0; i < 2; i++) ai_off[i] = (uint32_t)((((lw * 2 + i) * KP) * 64 + lane) * 4);
-        // activations: loader lw moves row groups 4lw..4lw+3 (8 rows each); lane -> (row, piece)
-        uint32_t x_off[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int row = (lw * 4 + i) * 8 + (lane >> 3);
-            const int piece = lane & 7;
-            const int q = piece ^ ((row >> 1) & 7);   // logical chunk stored at this piece
-            int64_t tok = t0 + row;
-            if (tok >= P.T) tok = P.T - 1;            // clamped rows are computed, never stored
-            x_off[i] = (uint32_t)((tok * P.ldx + q * 8) * 2);
-        }
-        auto issue = [&](int kp, int stage) {
-            unsigned char *base = smem + stage * PIPE_STAGE;
-            const unsigned char *avb = av_base + (int64_t)kp * 2048;  // two k-steps of a feature block
-            const unsigned char *aib = ai_base + (int64_t)kp * 256;
-            const unsigned char *xb = x_base + (int64_t)kp * 128;
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                __builtin_amdgcn_global_load_lds((glb_ptr_t)(avb + av_off[i]),
-                                                 (lds_ptr_t)(base + (lw * 4 + i) * 1024), 16, 0, 0);
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-                __builtin_amdgcn_global_load_lds((glb_ptr_t)(aib + ai_off[i]),
-                                                 (lds_ptr_t)(base + PIPE_AVAL + (lw * 2 + i) * 256), 4, 0, 0);
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                __builtin_amdgcn_global_load_lds(
-                    (glb_ptr_t)(xb + x_off[i]),
-                    (lds_ptr_t)(base + PIPE_AVAL + PIPE_AIDX + (lw * 4 + i) * 1024), 16, 0, 0);
-        };
-        // Fill the ring (steps beyond KP-1 repeat the last one so the load count stays uniform).
-#pragma unroll
-        for (int st = 0; st < PIPE_NS; st++) issue(st < KP ? st : KP - 1, st);
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((PIPE_NS - 1) * PIPE_LPT) : "memory");
-        asm volatile("s_barrier" ::: "memory");
-        for (int kp = 0; kp < KP; kp++) {
-            if (kp + PIPE_NS <= KP) {
-                // steps kp+1 .. kp+NS-1 are in flight; kp+1 has landed once NS-2 remain
-                asm volatile("s_waitcnt vmcnt(%0)" ::"n"((PIPE_NS - 2) * PIPE_LPT) : "memory");
-            } else {
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            }
-            asm volatile("s_barrier" ::: "memory");
-            if (kp + PIPE_NS < KP) issue(kp + PIPE_NS, kp & (PIPE_NS - 1));
-        }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        return;
-    }
-
-    // ================================ matrix wavefronts ================================
-    const int wm = wave >> 1, wn = wave & 1;
-    f32x16 acc[FB][TB];
-#pragma unroll
-    for (int i = 0; i < FB; i++)
-#pragma unroll
-        for (int j = 0; j < TB; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
-
-    // ---- fragment read offsets inside a stage ----
-    const int a_off = (wm * FB) * 2 * 1024 + lane * 16;
-    const int i_off = PIPE_AVAL + (wm * FB) * 256 + lane * 4;
-    const int j = lane & 31, h = lane >> 5, sw = (j >> 1) & 7;
-    int b_off[2][2];  // [ks][c]
-#pragma unroll
-    for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-        for (int c = 0; c < 2; c++)
-            b_off[ks][c] = PIPE_AVAL + PIPE_AIDX + (wn * 64 + j) * 128 + (((ks * 4 + h * 2 + c) ^ sw) << 4);
-
-    // Fragment registers of one k-step: 4 weight fragments, their index words, 2 activation
-    // fragments.  Set 0 serves the even k-step of a stage, set 1 the odd one.
-    struct Frags {
-        u32x4 a[FB];
-        uint32_t ix[FB];
-        u32x4 b[TB][2];
-    };
-    Frags fr0, fr1;
-    auto read_frags = [&](Frags &f, const unsigned char *base, int ks) {
-#pragma unroll
-        for (int fb = 0; fb < FB; fb++) {
-            f.a[fb] = *(const u32x4 *)(base + a_off + (fb * 2 + ks) * 1024);
-            f.ix[fb] = *(const uint32_t *)(base + i_off + fb * 256);
-        }
-#pragma unroll
-        for (int tb = 0; tb < TB; tb++) {
-            f.b[tb][0] = *(const u32x4 *)(base + b_off[ks][0] + tb * 32 * 128);
-            f.b[tb][1] = *(const u32x4 *)(base + b_off[ks][1] + tb * 32 * 128);
-        }
-    };
-    auto mma = [&](const Frags &f, auto abid_tag, auto lo_tag, auto hi_tag) {
-        constexpr int ABID = decltype(abid_tag)::value;
-#pragma unroll
-        for (int fb = decltype(lo_tag)::value; fb < decltype(hi_tag)::value; fb++) {
-            union {
-                u32x4 u;
-                typename S::A v;
-            } ca;
-            ca.u = f.a[fb];
-#pragma unroll
-            for (int tb = 0; tb < TB; tb++) {
-                union {
-                    u32x4 u[2];
-                    typename S::B v;
-                } cb;
-                cb.u[0] = f.b[tb][0];
-                cb.u[1] = f.b[tb][1];
-                acc[fb][tb] = S::template run<ABID>(ca.v, cb.v, acc[fb][tb], (int)f.ix[fb]);
-            }
-        }
-    };
-
-    asm volatile("s_barrier" ::: "memory");  // step 0 has landed
-    read_frags(fr0, smem, 0);
-
-    using I0 = std::integral_constant<int, 0>;
-    using I1 = std::integral_constant<int, 1>;
-    using IFB = std::integral_constant<int, FB>;
-    // Instruction-group masks of the scheduler: 0x008 MFMA, 0x100 LDS read.  One MFMA occupies
-    // the matrix pipe for ~32 cycles during which the wavefront can issue a few other
-    // instructions for free, so the LDS reads are dealt out two per MFMA instead of in bursts.
-    for (int kp = 0; kp < KP; kp++) {
-        const unsigned char *base = smem + (kp & (PIPE_NS - 1)) * PIPE_STAGE;
-        // ---- even k-step: MFMAs on set 0, fetch set 1 of the same stage ----
-        read_frags(fr1, base, 1);
-        mma(fr0, I0{}, I0{}, IFB{});
-#pragma unroll
-        for (int i = 0; i < FB * TB; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i < 5) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // ---- odd k-step: two MFMAs, then hand the stage back ----
-        mma(fr1, I1{}, I0{}, I1{});
-        __builtin_amdgcn_sched_barrier(0);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // all of stage kp is in registers
-        asm volatile("s_barrier" ::: "memory");             // ... and step kp+1 has landed
-        __builtin_amdgcn_sched_barrier(0);
-        read_frags(fr0, smem + ((kp + 1) & (PIPE_NS - 1)) * PIPE_STAGE, 0);
-        mma(fr1, I1{}, I1{}, IFB{});
-#pragma unroll
-        for (int i = 0; i < (FB - 1) * TB; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i < 5) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    }
-
-    const TileOut out{P.y, P.bias, P.M, P.T, P.ldy};
-    smf_store_tile<T, FB, TB>(acc, smem + wave * (64 * PIPE_OUT_ROW), lane, f0 + wm * 128, t0 + wn * 64, out);
-}
-
-template <typename T> static int launch_smfmac_pipe(SmfParams &P, hipStream_t s)
-{
-    P.tiles_m = (int)((P.M + 255) / 256);
-    P.tiles_n = (int)((P.T + 127) / 128);
-    dim3 grid((unsigned)(P.tiles_m * P.tiles_n));
-    const size_t lds = (size_t)PIPE_NS * PIPE_STAGE;
-    static_assert(PIPE_NS * PIPE_STAGE >= 4 * 64 * PIPE_OUT_ROW, "epilogue staging must fit in the ring");
-    auto k = spmm_smfmac_pipe_kernel<T>;
-    NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(k, grid, dim3(512), lds, s, P);
-    NMG_HIP_TRY(hipGetLastError());
-    return NMG_OK;
-}
 
 // ------------------------------------------------------------- pipelined kernel, direct weights
 // The fragpack operand is already in the register order of the instruction, so the weight
@@ -518,7 +276,10 @@ template <typename T> static int launch_smfmac_pipe(SmfParams &P, hipStream_t s)
 // itself; each also issues its quarter of the activation tile's DMA loads.  Every K step a
 // wavefront issues XL DMA loads and 3*FB register loads for step kp+DR_D, so "step kp+1 has
 // landed" is vmcnt <= OPS*(DR_D-1); the barrier that follows publishes the activation rows of
-// all four wavefronts.  Tile order, swizzle and preconditions as in the kernel above.
+// all four wavefronts.  A DMA load writes 64 lanes x 16 B contiguously, so the activation rows
+// cannot be padded; instead the 16-byte chunks of a row are XOR-swizzled with (row/2)%8, chosen on
+// the global side, which makes the fragment reads (32 rows x 16 B at one logical chunk)
+// conflict-free.  Requires K % 64 == 0 and activations smaller than 2 GiB (32-bit lane offsets).
 //
 // A K step is cut into 2 * NH phases (k-step of 32 x a part of the wavefront's token blocks): the
 // MFMAs of a phase run while the activation fragments of the next one are read from LDS into a
@@ -1357,10 +1118,7 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
         variant = 6;
     }
     switch (variant) {
-    case 0: return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);  // 256 lines x 128 tokens, 1 wave/SIMD
-    case 1: return launch_smfmac_cfg<T, 2, 2, 2, 2, 2>(P, s);  // 128 x 128, 2 waves/SIMD
-    case 2: return launch_smfmac_cfg<T, 2, 2, 2, 4, 2>(P, s);  // 128 x 256
-    case 3: return launch_smfmac_cfg<T, 4, 1, 2, 4, 2>(P, s);  // 256 x 128, waves stacked on lines
+    case 0: return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);  // register-prefetch kernel, 256 lines x 128 tokens: any K
     case 5:                                                     // decode shapes, T <= 16
         if (P.T > 16) return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
         // few line blocks: many wavefronts per workgroup keep enough loads in flight per CU;
@@ -1378,10 +1136,6 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
         }
         if ((P.M + 31) / 32 >= 256) return launch_smfmac_skinny<T, 4, 4>(P, s);
         return launch_smfmac_skinny<T, 16, 1>(P, s);
-    case 4:                                                     // 256 x 128, LDS-DMA ring
-        if (P.K % 64 != 0 || P.T * P.ldx * 2 >= (int64_t)1 << 31)
-            return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
-        return launch_smfmac_pipe<T>(P, s);
     case 6:                                                     // 256 x 128, weights straight to registers
     case 8:                                                     // 256 x 256
         if (P.K % 64 != 0 || P.T * P.ldx * 2 >= (int64_t)1 << 31)
@@ -1399,7 +1153,8 @@ extern "C" int nmg_spmm_smfmac(const void *d_fp_val, const void *d_fp_idx, int64
     NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED,
                 "the sparse matrix cores take f16/bf16 only");
     NMG_REQUIRE(M >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
-    NMG_REQUIRE(variant >= -1 && variant <= 8 && variant != 7, NMG_ERR_ARG, "unknown tile variant %d", variant);
+    NMG_REQUIRE(variant == -1 || variant == 0 || variant == 5 || variant == 6 || variant == 8, NMG_ERR_ARG,
+                "unknown tile variant %d", variant);
     NMG_REQUIRE(ldx >= K && ldy >= M, NMG_ERR_ARG, "leading dimension smaller than row length");
     NMG_REQUIRE((K % 8) == 0 && (ldx % 8) == 0 && ((uintptr_t)d_x % 16) == 0, NMG_ERR_UNSUPPORTED,
                 "activations must be 16-byte aligned with K and ldx multiples of 8");

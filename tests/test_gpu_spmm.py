@@ -192,7 +192,7 @@ def test_unregistered_op_raises_in_raise_mode():
         torch.relu(w)
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 6, 8])
+@pytest.mark.parametrize("variant", [-1, 0, 6, 8])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M,K,T,n,m,g", [
     (768, 768, 256, 2, 4, 16),
