@@ -71,6 +71,8 @@ WORKLOADS = {
 
 # committed rocprofv3 --pmc summaries (FETCH_SIZE / WRITE_SIZE) of the workloads that have one
 PMC_SUMMARIES = {
+    "target_2_4": "spmm_target_2_4_pmc.txt",
+    "c5_step": "train_step_c5_kernel_trace_pmc.txt",
     "c2": "spmm_c2_pmc.txt",
     "decode_1": "spmm_decode_1_pmc.txt",
     "c4_b1": "w4_linear_c4_b1_pmc.txt",
