@@ -184,6 +184,31 @@ def test_optimizer_steps_keep_pattern():
     assert lin.weight.requires_grad
 
 
+def test_in_place_updates_with_an_independently_sparsified_tensor():
+    # Two tensors of the same layout, compressed independently, keep different columns in the same
+    # slots: add_ / mul_ / copy_ must combine them position by position (through the dense form and
+    # this tensor's pattern), not slot by slot; tensors that share the pattern take the direct path.
+    a = make(seeded((96, 64), torch.float32, seed=1), 2, 4, 4, 1)
+    b = make(seeded((96, 64), torch.float32, seed=2), 2, 4, 4, 1)
+    assert a.layout == b.layout and not torch.equal(a.idx, b.idx)
+    da, db = a.to_dense().clone(), b.to_dense().clone()
+    mask = a.clone_layout(torch.ones(96, 64, device=DEV)).to_dense() != 0
+    a.add_(b, alpha=0.5)
+    assert torch.equal(a.to_dense(), torch.where(mask, da + 0.5 * db, torch.zeros_like(da)))
+    a.mul_(b)
+    want = torch.where(mask, (da + 0.5 * db) * db, torch.zeros_like(da))
+    assert torch.equal(a.to_dense(), want)
+    a.copy_(b)
+    assert torch.equal(a.to_dense(), torch.where(mask, db, torch.zeros_like(db)))
+    # same pattern (clone_layout shares idx; an equal copy of idx counts too): slot by slot
+    c = a.clone_layout(torch.full((96, 64), 2.0, device=DEV))
+    d = sten.GroupedNMTensor(c.val.clone(), a.idx.clone(), a.layout)
+    before = a.val.clone()
+    a.add_(c)
+    a.add_(d)
+    assert torch.equal(a.val, (before + 2.0) + 2.0)
+
+
 def test_unregistered_op_raises_in_raise_mode():
     sten.set_dispatch_failure("raise")
     w = sten.SparseTensorWrapper.wrapped_from_dense(
