@@ -14,8 +14,9 @@ For the bandwidth-bound workloads (decode shapes, sparsifier) value = GB/s of al
 sparsifier) and the roofline is HBM.  roofline.traffic is null: HBM traffic comes from rocprofv3
 counter runs, whose summaries are under profiles/ (config.traffic_profile names the file).
 With the default workload the same run also measures the other benchmark rows (config 2, config 3
-at 2:8, the decode shapes at 1 and 16 tokens, config 4 at 1 token, the config 2 sparsifier and the
-config 5 training step) with the same protocol and reports them under config.also as
+at 1:8 / 2:8 / 4:8, the decode shapes at 1, 4, 8 and 16 tokens, config 4 at 1, 4 and 16 tokens, the
+config 2 sparsifier and the config 5 training step without and with the optimizer update) with the
+same protocol and reports them under config.also as
 {us, value, unit, frac}; --no-also skips them.
 cpu_baseline (headline and config 2) = the CPU restatement of the reference's AVX/OpenMP kernel
 (oracle/nmg_cpu_simd.cpp) on the host cores, same shape, fp32, on a 1024-row slab of the weight;
@@ -80,8 +81,10 @@ PMC_SUMMARIES = {
 }
 
 # measured beside the headline workload in the default run: (workload, steps, warm-up)
-ALSO = [("c2", 50, 10), ("c3_2_8", 20, 5), ("decode_1", 50, 10), ("decode_16", 50, 10), ("c4_b1", 50, 10),
-        ("sparsify_c2", 20, 5), ("c5_step", 10, 3)]
+ALSO = [("c2", 50, 10), ("c3_1_8", 20, 5), ("c3_2_8", 20, 5), ("c3_4_8", 20, 5),
+        ("decode_1", 50, 10), ("decode_4", 50, 10), ("decode_8", 50, 10), ("decode_16", 50, 10),
+        ("c4_b1", 50, 10), ("c4_b4", 50, 10), ("c4_b16", 50, 10),
+        ("sparsify_c2", 20, 5), ("c5_step", 10, 3), ("c5_train", 10, 3)]
 
 
 def cpu_baseline(M, K, N, n, m, g, seconds=15.0):
