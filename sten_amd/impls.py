@@ -17,9 +17,15 @@ class GroupedNMSparsifier:
     ``sparse_dim`` / ``group_dim`` select another one, e.g. ``sparse_dim=-1, group_dim=-2`` puts
     the n:m blocks along the reduction dim of ``F.linear``."""
 
-    def __init__(self, n, m, g, sparse_dim=-2, group_dim=-1):
+    # orientation used when the caller names none: the reference's.  `plugin.register(sten,
+    # nm_along_reduction=True)` switches it to (-1, -2) for unchanged user code that wants the
+    # n:m blocks along the reduction dim of F.linear, where the sparse matrix cores can use them.
+    default_dims = (-2, -1)
+
+    def __init__(self, n, m, g, sparse_dim=None, group_dim=None):
         self.n, self.m, self.g = n, m, g
-        self.sparse_dim, self.group_dim = sparse_dim, group_dim
+        self.sparse_dim = type(self).default_dims[0] if sparse_dim is None else sparse_dim
+        self.group_dim = type(self).default_dims[1] if group_dim is None else group_dim
 
 
 def _masked_weight_grad(weight, lhs_t, rhs):

@@ -14,7 +14,13 @@ from . import impls, perfect, w4
 from .tensor import GroupedNMTensor
 
 
-def register(sten_module):
+def register(sten_module, nm_along_reduction=False):
+    """Install the implementations into ``sten_module``.  ``nm_along_reduction=True`` also makes
+    ``GroupedNMSparsifier(n, m, g)`` (no dims given) put the n:m blocks along the last dim -- the
+    reduction dim of ``F.linear`` -- instead of the reference's dim -2: unchanged user code then
+    reaches the sparse matrix cores in forward, at the price of a pattern that differs from the one
+    the reference would choose for the same call."""
+    impls.GroupedNMSparsifier.default_dims = (-1, -2) if nm_along_reduction else (-2, -1)
     reg = getattr(sten_module, "SPARSIFIER_IMPLEMENTATIONS", None)
     if reg is None and hasattr(sten_module, "sten"):
         reg = sten_module.sten.SPARSIFIER_IMPLEMENTATIONS
