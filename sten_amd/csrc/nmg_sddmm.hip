@@ -116,6 +116,7 @@ static_assert(SD_LDS <= 160 * 1024, "LDS of a CU");
 static_assert(SD_D < SD_NS, "a stage is refilled only after the barrier that ends its last read");
 static_assert(SD_D * SD_LPW < 64, "vmcnt is a 6-bit counter");
 
+// MODE 8 + n (n = 1, 2, 4): m == 8, the same after an exchange between the two lanes that hold a block.
 // MODE 1 .. 4: m == 4 and n == MODE.  The 4 consecutive positions a lane holds of its line are one
 // block, so the kept values are picked in registers (one byte permute with a per-pattern selector)
 // and stored by the lane itself; the slots of the lane's 64 (line, block) pairs are fetched when the
@@ -145,8 +146,8 @@ template <typename T, int MODE> __global__ __launch_bounds__(256, 1) void sddmm_
 
     // ---- MODE 1: the lane's slots.  Accumulator block (x, y), register quad rq: line
     // l0 + wn*128 + y*32 + l%32, block (p0 + wm*128 + x*32 + rq*8 + (l/32)*4) / 4.
-    uint32_t my_slot[MODE >= 1 ? 32 : 1];   // two slots per register: rq even | rq odd << 16
-    if constexpr (MODE >= 1) {
+    uint32_t my_slot[MODE >= 1 ? (MODE <= 4 ? 32 : 16) : 1];   // two slots per register
+    if constexpr (MODE >= 1 && MODE <= 4) {
         // byte selectors of V_PERM_B32 per pattern: kept halves 0, 1 (and 2, 3) out of the 8 bytes
         // {positions 0, 1 | positions 2, 3} of a block, from the packed order table
         uint32_t *s_sel = (uint32_t *)(smem + 256 * SD_PITCH);
@@ -169,6 +170,43 @@ template <typename T, int MODE> __global__ __launch_bounds__(256, 1) void sddmm_
                     my_slot[(y * 4 + x) * 2 + rp] = (uint32_t)(uint16_t)P.slot[blk0 * P.Gpad + line] |
                                                     ((uint32_t)(uint16_t)P.slot[blk1 * P.Gpad + line] << 16);
                 }
+        }
+    }
+
+    if constexpr (MODE > 8) {
+        // ---- MODE 8 + n: m == 8.  A block of a line lies in two lanes (positions 0..3 in lane
+        // l%32, 4..7 in lane l%32 + 32); after the exchange in the epilogue lane l owns the blocks
+        // (p0 + wm*128 + x*32) / 8 + 2k + l/32, k = 0, 1, of its line: their slots, k = 1 in the
+        // high half.  Selector table: per pattern and output word two V_PERM_B32 selectors, one for
+        // the positions 0..3, one for 4..7 (bytes that come from the other half select zero).
+        constexpr int N = MODE - 8, ND = (N + 1) / 2;
+        uint32_t *s_sel = (uint32_t *)(smem + 256 * SD_PITCH);
+        for (int e = tid; e < P.order_bytes / N * ND; e += 256) {
+            const int pat = e / ND, w = e - pat * ND;
+            uint32_t sa = 0x0c0c0c0cu, sb = 0x0c0c0c0cu;
+#pragma unroll
+            for (int jj = 0; jj < 2; jj++) {
+                const int j = 2 * w + jj;
+                if (j >= N) break;
+                const uint32_t q = (uint32_t)P.order[pat * N + j] & 7u;
+                const uint32_t two = (2 * (q & 3)) | ((2 * (q & 3) + 1) << 8);
+                if (q < 4) sa = (sa & ~(0xffffu << (16 * jj))) | (two << (16 * jj));
+                else sb = (sb & ~(0xffffu << (16 * jj))) | (two << (16 * jj));
+            }
+            s_sel[2 * e] = sa;
+            s_sel[2 * e + 1] = sb;
+        }
+        const int j = lane & 31, h = lane >> 5;
+#pragma unroll
+        for (int y = 0; y < 4; y++) {
+            const int64_t line = min(l0 + wn * 128 + y * 32 + j, P.Gpad - 1);
+#pragma unroll
+            for (int x = 0; x < 4; x++) {
+                const int blk0 = min((int)(p0 / 8) + wm * 16 + x * 4 + h, (int)P.nb - 1);
+                const int blk1 = min((int)(p0 / 8) + wm * 16 + x * 4 + 2 + h, (int)P.nb - 1);
+                my_slot[y * 4 + x] = (uint32_t)(uint16_t)P.slot[blk0 * P.Gpad + line] |
+                                     ((uint32_t)(uint16_t)P.slot[blk1 * P.Gpad + line] << 16);
+            }
         }
     }
 
@@ -356,7 +394,87 @@ template <typename T, int MODE> __global__ __launch_bounds__(256, 1) void sddmm_
     uint16_t *val = (uint16_t *)P.val;
     const int n = P.n, m = P.m;
 
-    if constexpr (MODE >= 1) {
+    if constexpr (MODE > 8) {
+        // ---- epilogue in registers, m == 8 (D rows = positions 8*(r/4) + 4*(l/32) + r%4 of the
+        // 32-position block: register quad rq of lanes l%32 and l%32 + 32 is block rq, low and
+        // high half).  The quads 2k and 2k+1 are rounded, packed and exchanged between the two
+        // lanes (V_PERMLANE32_SWAP), after which the low lane holds block 2k and the high lane
+        // block 2k+1 as four words; the kept values are picked with two byte permutes per word.
+        constexpr int N = MODE - 8, ND = (N + 1) / 2;
+        const uint32_t *s_sel = (const uint32_t *)(smem + 256 * SD_PITCH);
+        asm volatile("s_barrier" ::: "memory");   // the selector table was written by other wavefronts
+        const int j = lane & 31, h = lane >> 5;
+        int blk_base = (int)(p0 / 8) + wm * 16 + h;
+        asm volatile("" : "+v"(blk_base));
+        const uint32_t cg = (uint32_t)P.cg, nb = (uint32_t)P.nb;
+        const uint32_t g1_mask = P.g > 1 ? 0u : ~0u;
+        unsigned char *vbase = (unsigned char *)P.val;
+        auto epilogue = [&](auto interior_tag) {
+            constexpr bool INTERIOR = decltype(interior_tag)::value;
+#pragma unroll
+            for (int y = 0; y < 4; y++) {
+                const uint32_t line = (uint32_t)l0 + wn * 128 + y * 32 + j;
+                const bool line_in = INTERIOR || line < (uint32_t)P.Gpad, line_ok = INTERIOR || line < (uint32_t)P.G;
+                const uint32_t rowbase = ((line / cg) * nb + (uint32_t)blk_base) * cg;
+#pragma unroll
+                for (int x = 0; x < 4; x++) {
+#pragma unroll
+                    for (int k = 0; k < 2; k++) {
+                        const uint32_t sl = min((my_slot[y * 4 + x] >> (16 * k)) & 0x7fffu, cg - 1);
+                        const uint32_t pat = __umulhi(sl, P.inv_g) + (sl & g1_mask);
+                        uint32_t sel[ND][2];
+#pragma unroll
+                        for (int w = 0; w < ND; w++) {
+                            sel[w][0] = s_sel[(pat * ND + w) * 2];
+                            sel[w][1] = s_sel[(pat * ND + w) * 2 + 1];
+                        }
+                        uint32_t d[4];   // before the exchange: quad 2k words 0, 1, quad 2k+1 words 0, 1
+#pragma unroll
+                        for (int qd = 0; qd < 2; qd++)
+#pragma unroll
+                            for (int w = 0; w < 2; w++) {
+                                const uint16_t lo16 = sd_bits16<T>(sd_from_acc(acc[x][y][(2 * k + qd) * 4 + 2 * w]));
+                                const uint16_t hi16 = sd_bits16<T>(sd_from_acc(acc[x][y][(2 * k + qd) * 4 + 2 * w + 1]));
+                                d[qd * 2 + w] = (uint32_t)lo16 | ((uint32_t)hi16 << 16);
+                            }
+                        // words of (quad 2k, quad 2k+1): low lanes keep quad 2k and receive its
+                        // high half from the lane 32 up, which receives the low half of quad 2k+1
+                        uint32_t blkw[4];   // positions 0,1 | 2,3 | 4,5 | 6,7 of the lane's block
+#pragma unroll
+                        for (int w = 0; w < 2; w++) {
+                            const auto sw = __builtin_amdgcn_permlane32_swap(d[w], d[2 + w], false, false);
+                            blkw[w] = sw[0];
+                            blkw[2 + w] = sw[1];
+                        }
+                        if (!INTERIOR && !line_ok) blkw[0] = blkw[1] = blkw[2] = blkw[3] = 0;
+                        if (!INTERIOR && (!line_in || blk_base + x * 4 + 2 * k >= (int)nb)) continue;
+                        unsigned char *dst =
+                            vbase + (size_t)((rowbase + (uint32_t)(x * 4 + 2 * k) * cg + sl) * (uint32_t)(2 * N));
+                        uint32_t out[ND];
+#pragma unroll
+                        for (int w = 0; w < ND; w++)
+                            out[w] = __builtin_amdgcn_perm(blkw[1], blkw[0], sel[w][0]) |
+                                     __builtin_amdgcn_perm(blkw[3], blkw[2], sel[w][1]);
+                        if constexpr (N == 1) {
+                            *(uint16_t *)dst = (uint16_t)out[0];
+                        } else if constexpr (N == 2) {
+                            *(uint32_t *)dst = out[0];
+                        } else {
+                            static_assert(N == 4, "m == 8 is built for n = 1, 2, 4");
+                            *(uint2 *)dst = uint2{out[0], out[1]};
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        };
+        if (l0 + 256 <= P.G && p0 + 256 <= P.nb * 8)
+            epilogue(std::true_type{});
+        else
+            epilogue(std::false_type{});
+        return;
+    }
+    if constexpr (MODE >= 1 && MODE <= 4) {
         // ---- epilogue in registers (D rows = positions 8*(r/4) + 4*(l/32) + r%4 of the block,
         // column = line l%32: registers rq*4 .. +3 of a lane are one block of its line).  Offsets
         // into val are 32-bit (the host checks that val is smaller than 4 GiB).
@@ -564,8 +682,9 @@ extern "C" int nmg_sddmm(const void *d_lines, int64_t ld_lines, const void *d_po
     dim3 grid((unsigned)(P.tiles_p * P.tiles_l));
     // m == 4, val 8-byte aligned and smaller than 4 GiB: the epilogue that stays in registers
     const int64_t val_bytes = ((G + cg - 1) / cg) * P.nb * cg * n * 2;
-    const bool in_regs = m == 4 && n >= 1 && ((uintptr_t)d_val % 8) == 0 && val_bytes < ((int64_t)1 << 32) &&
-                         P.Gpad < ((int64_t)1 << 31);
+    const bool small = ((uintptr_t)d_val % 8) == 0 && val_bytes < ((int64_t)1 << 32) && P.Gpad < ((int64_t)1 << 31);
+    const bool in_regs = m == 4 && n >= 1 && small;
+    const bool in_regs8 = m == 8 && (n == 1 || n == 2 || n == 4) && small;
     if (in_regs) {
         const int8_t *ho = host_order(n, m);
         for (int64_t p = 0; p < binom(m, n); p++)
@@ -578,6 +697,11 @@ extern "C" int nmg_sddmm(const void *d_lines, int64_t ld_lines, const void *d_po
     };
     auto launch_t = [&](auto tag) -> int {
         using T = decltype(tag);
+        if (in_regs8) {
+            if (n == 1) return launch(sddmm_kernel<T, 9>);
+            if (n == 2) return launch(sddmm_kernel<T, 10>);
+            return launch(sddmm_kernel<T, 12>);
+        }
         if (!in_regs) return launch(sddmm_kernel<T, 0>);
         switch (n) {
         case 1: return launch(sddmm_kernel<T, 1>);
