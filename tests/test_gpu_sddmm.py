@@ -40,6 +40,9 @@ def oracle_masked_grad(gy, x, idx, lay):
     (528, 96, 31, 3, 6, 2, 0),
     (64, 48, 7, 1, 1, 8, 1),            # n == m: nothing dropped
     (768, 1024, 160, 2, 4, 1, 1),       # group size 1
+    (1800, 512, 96, 2, 8, 32, 1),       # config 3's patterns: chunks of 896 / 2240 lines span several tiles
+    (2240, 264, 64, 4, 8, 32, 0),
+    (520, 512, 40, 1, 8, 32, 1),
 ])
 def test_masked_product_matches_oracle(dtype, R, C, T, n, m, g, sd):
     print(f"case sddmm {dtype} R={R} C={C} T={T} {n}:{m}:{g} sd={sd}", flush=True)
