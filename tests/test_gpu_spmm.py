@@ -732,3 +732,18 @@ def test_direct_kernels_on_a_full_chip_with_a_long_reduction():
         for _ in range(4):
             got = sten.spmm(w, g, reduce_dim=0, kernel="densefrag").float()
             assert float((got - want).norm() / want.norm()) <= 1e-4, f"dense variant {dense_variant}"
+
+
+def test_matrix_rate_probe_runs_every_instruction():
+    # measurement aid of bench.py: launches and finishes for every kind, refuses a bad one
+    lib = native.load()
+    src = torch.randn(512 * 1024, device=DEV).half()
+    out = torch.empty(256 * 1024, dtype=torch.float32, device=DEV)
+    for kind in range(4):
+        print(f"case matrix rate probe kind {kind}", flush=True)
+        assert lib.nmg_probe_matrix_rate_flops(kind, 10) == 2 * 128 * 128 * 64 * 10 * 4096
+        native.check(lib.nmg_probe_matrix_rate(kind, native.ptr(src), native.ptr(out), 10, None))
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())
+    assert lib.nmg_probe_matrix_rate(7, native.ptr(src), native.ptr(out), 10, None) == 1
+    assert lib.nmg_probe_matrix_rate_flops(7, 10) == -1
