@@ -496,11 +496,17 @@ template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_
 
 template <typename T> static int launch_dense(DfParams &P, int variant, hipStream_t s)
 {
-    // 256 x 256 tiles (variant 1) move fewer bytes per flop through the vector caches and are 8 %
-    // faster on shapes with enough of them, but they are by request only: a sixteen-phase form of
-    // that tile once gave wrong values now and then and the cause was never found, so the automatic
-    // choice stays with the tile that has no such history.
-    if (variant < 0) variant = 0;
+    // 256 x 256 tiles (variant 1) move fewer bytes per flop through the vector caches and are 5-6 %
+    // faster per flop in steady state (8192^2 x 4096 tokens: 414 against 439 us); one workgroup per
+    // CU either way, so what decides is how full the last round of tiles is.  (A sixteen-phase form
+    // of the 256 x 256 tile once gave wrong values now and then; that form is gone, the eight-phase
+    // form here passes the static check of its hand-tracked loads and the repeated full-chip test.)
+    if (variant < 0) {
+        const int64_t tm = (P.O + 255) / 256, t256 = tm * ((P.T + 255) / 256), t128 = tm * ((P.T + 127) / 128);
+        const double fill256 = (double)t256 / (double)((t256 + 255) / 256 * 256);
+        const double fill128 = (double)t128 / (double)((t128 + 255) / 256 * 256);
+        variant = (P.ksplit <= 1 && t256 >= 256 && fill256 * 1.055 >= fill128) ? 1 : 0;
+    }
     if (variant == 1) return launch_dense_direct<T, 2, 8, 4, 1, 2>(P, s);
     return launch_dense_direct<T, 2, 4, 4, 1, 1>(P, s);
 }
