@@ -325,10 +325,14 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
         u32x4 b[BT];
     };
     BFrags fr[2];
-    auto read_b = [&](BFrags &f, const unsigned char *base, int ph) {
+    // part 0 / 1: the first / second half of the phase's reads (part < 0: all of them)
+    auto read_b = [&](BFrags &f, const unsigned char *base, int ph, int part = -1) {
         const int k16 = ph / NH, hh = ph % NH;
 #pragma unroll
-        for (int t = 0; t < BT; t++) f.b[t] = *(const u32x4 *)(base + b_off[k16] + (hh * BT + t) * 32 * 128);
+        for (int t = 0; t < BT; t++) {
+            if (part >= 0 && t / ((BT + 1) / 2) != part) continue;
+            f.b[t] = *(const u32x4 *)(base + b_off[k16] + (hh * BT + t) * 32 * 128);
+        }
     };
     // MFMAs lo..hi-1 of phase PH, numbered fb * BT + t
     auto mma = [&](const WSet &w, const BFrags &f, auto ph_tag, int lo, int hi) {
@@ -402,37 +406,61 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
             // instruction statements fence the scheduler, so this is also the issue order.
             auto phase = [&](auto ph_tag) {
                 constexpr int PH = decltype(ph_tag)::value;
-                mma(ws[u], fr[PH % 2], ph_tag, 0, 2);
-                __builtin_amdgcn_sched_barrier(0);
+                constexpr int L0 = PH * OPS / NP, L1 = (PH + 1) * OPS / NP;   // this phase's loads
+                // One memory instruction (or two LDS reads) goes into the shadow of one MFMA: a load
+                // holds the wavefront's issue for about 20 clocks, an LDS read for 7, an MFMA runs 32.
+                constexpr bool SPLIT = BT >= 2 && NM >= 6;
                 if (PH == NP - 1) {
+                    mma(ws[u], fr[PH % 2], ph_tag, 0, 2);
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int i = PH * OPS / NP; i < OPS; i++)
-                        issue_one(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)], i);
+                    for (int i = L0; i < OPS; i++) issue_one(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)], i);
                     __builtin_amdgcn_sched_barrier(0);
                     // fragments of step kp are in registers, my share of step kp+1 has landed ...
                     landed(ws[(u + 1) % (DD_D + 1)]);
                     asm volatile("s_barrier" ::: "memory");              // ... and everybody else's
                     __builtin_amdgcn_sched_barrier(0);
-                    read_b(fr[(PH + 1) % 2], next, 0);
+                    if constexpr (SPLIT) {
+                        mma(ws[u], fr[PH % 2], ph_tag, 2, 3);
+                        __builtin_amdgcn_sched_barrier(0);
+                        read_b(fr[(PH + 1) % 2], next, 0, 0);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma(ws[u], fr[PH % 2], ph_tag, 3, 4);
+                        __builtin_amdgcn_sched_barrier(0);
+                        read_b(fr[(PH + 1) % 2], next, 0, 1);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma(ws[u], fr[PH % 2], ph_tag, 4, NM);
+                    } else {
+                        read_b(fr[(PH + 1) % 2], next, 0);
+                        mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
+                    }
                 } else {
-                    read_b(fr[(PH + 1) % 2], base, PH + 1);
-                }
-                // The step's OPS loads are dealt out evenly over its phases, one at a time between
-                // MFMAs: a burst would find the CU's vector memory path busy (16 clocks per 1 KiB
-                // instruction, shared by the four wavefronts) and stall with its MFMAs unissued.
-                // (In the last phase the loads come before the counted wait, which assumes them.)
-                constexpr int L0 = PH * OPS / NP, L1 = (PH + 1) * OPS / NP;   // this phase's loads
-                if (PH != NP - 1) {
+                    if constexpr (SPLIT) {
+                        mma(ws[u], fr[PH % 2], ph_tag, 0, 1);
+                        __builtin_amdgcn_sched_barrier(0);
+                        read_b(fr[(PH + 1) % 2], base, PH + 1, 0);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma(ws[u], fr[PH % 2], ph_tag, 1, 2);
+                        __builtin_amdgcn_sched_barrier(0);
+                        read_b(fr[(PH + 1) % 2], base, PH + 1, 1);
+                    } else {
+                        mma(ws[u], fr[PH % 2], ph_tag, 0, 2);
+                        __builtin_amdgcn_sched_barrier(0);
+                        read_b(fr[(PH + 1) % 2], base, PH + 1);
+                    }
+                    // The step's OPS loads are dealt out evenly over its phases, one at a time behind
+                    // an MFMA: a burst would find the CU's vector memory path busy and stall with
+                    // its MFMAs unissued.  (In the last phase the loads come before the counted
+                    // wait, which assumes them.)
 #pragma unroll
                     for (int i = L0; i < L1; i++) {
                         __builtin_amdgcn_sched_barrier(0);
-                        issue_one(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)], i);
-                        __builtin_amdgcn_sched_barrier(0);
                         if (2 + i - L0 < NM) mma(ws[u], fr[PH % 2], ph_tag, 2 + i - L0, 3 + i - L0);
+                        __builtin_amdgcn_sched_barrier(0);
+                        issue_one(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)], i);
                     }
+                    __builtin_amdgcn_sched_barrier(0);
                     if (2 + L1 - L0 < NM) mma(ws[u], fr[PH % 2], ph_tag, 2 + L1 - L0, NM);
-                } else {
-                    mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             };

@@ -459,10 +459,12 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
             t_off[tb] = (16 * (g >> 1) + a) * (TT * 2) + ((chunk ^ (a << 2)) << 4) + (i16 & 1) * 8;
         }
     }
-    auto read_b = [&](BFrags &f, const unsigned char *base, int ph) {
+    // part 0 / 1: the first / second half of the phase's reads (part < 0: all of them)
+    auto read_b = [&](BFrags &f, const unsigned char *base, int ph, int part = -1) {
         const int ks = ph / NH, hh = ph % NH;
 #pragma unroll
         for (int t = 0; t < BT; t++) {
+            if (BT >= 2 && part >= 0 && t / (BT / 2) != part) continue;
             if constexpr (XT) {
                 typedef short i16x4 __attribute__((ext_vector_type(4)));
                 typedef __attribute__((address_space(3))) i16x4 *lds_i16x4;
@@ -477,8 +479,8 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
                 f.b[t][0] = c.u[0];
                 f.b[t][1] = c.u[1];
             } else {
-                f.b[t][0] = *(const u32x4 *)(base + b_off[ks][0] + (hh * BT + t) * 32 * 128);
-                f.b[t][1] = *(const u32x4 *)(base + b_off[ks][1] + (hh * BT + t) * 32 * 128);
+                if (BT >= 2 || part != 1) f.b[t][0] = *(const u32x4 *)(base + b_off[ks][0] + (hh * BT + t) * 32 * 128);
+                if (BT >= 2 || part != 0) f.b[t][1] = *(const u32x4 *)(base + b_off[ks][1] + (hh * BT + t) * 32 * 128);
             }
         }
     };
@@ -547,42 +549,64 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
             // instruction statements fence the scheduler, so this is also the issue order.
             auto phase = [&](auto ph_tag) {
                 constexpr int PH = decltype(ph_tag)::value;
-                mma(ws[u], fr[PH % 2], ph_tag, 0, 2);
-                __builtin_amdgcn_sched_barrier(0);
+                constexpr int L0 = PH * OPS / NP, L1 = (PH + 1) * OPS / NP;
+                // One memory instruction (or two LDS reads) goes into the shadow of one MFMA: a load
+                // holds the wavefront's issue for about 20 clocks, an LDS read for 7, an MFMA runs 32.
+                // (XT: the transposing reads of a block stay together.)
+                constexpr bool SPLIT = !XT && TB == 8;   // measured: -3..6 % on the 256 x 256 tile, +5 % where two 256 x 128 workgroups share a CU
                 if (PH == NP - 1) {
+                    mma(ws[u], fr[PH % 2], ph_tag, 0, 2);
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int i = PH * OPS / NP; i < OPS; i++)
-                        issue_one(kp + DR_D, ws[(u + DR_D) % (DR_D + 1)], i);
+                    for (int i = L0; i < OPS; i++) issue_one(kp + DR_D, ws[(u + DR_D) % (DR_D + 1)], i);
                     __builtin_amdgcn_sched_barrier(0);
                     // fragments of step kp are in registers, my share of step kp+1 has landed ...
                     landed(ws[(u + 1) % (DR_D + 1)]);
                     asm volatile("s_barrier" ::: "memory");              // ... and everybody else's
                     __builtin_amdgcn_sched_barrier(0);
-                    read_b(fr[(PH + 1) % 2], next, 0);
+                    if constexpr (SPLIT) {
+                        mma(ws[u], fr[PH % 2], ph_tag, 2, 3);
+                        __builtin_amdgcn_sched_barrier(0);
+                        read_b(fr[(PH + 1) % 2], next, 0, 0);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma(ws[u], fr[PH % 2], ph_tag, 3, 4);
+                        __builtin_amdgcn_sched_barrier(0);
+                        read_b(fr[(PH + 1) % 2], next, 0, 1);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma(ws[u], fr[PH % 2], ph_tag, 4, NM);
+                    } else {
+                        read_b(fr[(PH + 1) % 2], next, 0);
+                        mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
+#pragma unroll
+                        for (int i = 0; i < BT; i++) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                        }
+                    }
                 } else {
-                    read_b(fr[(PH + 1) % 2], base, PH + 1);
-                }
-                // The step's OPS loads are dealt out over its phases, one at a time between MFMAs
-                // (a burst finds the CU's vector memory path busy and stalls with its MFMAs
-                // unissued: 5 % on the 256 x 128 tile); in the last phase they come before the
-                // counted wait, which assumes them.
-                constexpr int L0 = PH * OPS / NP, L1 = (PH + 1) * OPS / NP;
-                if (PH != NP - 1) {
+                    if constexpr (SPLIT) {
+                        mma(ws[u], fr[PH % 2], ph_tag, 0, 1);
+                        __builtin_amdgcn_sched_barrier(0);
+                        read_b(fr[(PH + 1) % 2], base, PH + 1, 0);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma(ws[u], fr[PH % 2], ph_tag, 1, 2);
+                        __builtin_amdgcn_sched_barrier(0);
+                        read_b(fr[(PH + 1) % 2], base, PH + 1, 1);
+                    } else {
+                        mma(ws[u], fr[PH % 2], ph_tag, 0, 2);
+                        __builtin_amdgcn_sched_barrier(0);
+                        read_b(fr[(PH + 1) % 2], base, PH + 1);
+                    }
+                    // the step's OPS loads are dealt out over its phases, one at a time between MFMAs
 #pragma unroll
                     for (int i = L0; i < L1; i++) {
                         __builtin_amdgcn_sched_barrier(0);
-                        issue_one(kp + DR_D, ws[(u + DR_D) % (DR_D + 1)], i);
-                        __builtin_amdgcn_sched_barrier(0);
                         if (2 + i - L0 < NM) mma(ws[u], fr[PH % 2], ph_tag, 2 + i - L0, 3 + i - L0);
+                        __builtin_amdgcn_sched_barrier(0);
+                        issue_one(kp + DR_D, ws[(u + DR_D) % (DR_D + 1)], i);
                     }
+                    __builtin_amdgcn_sched_barrier(0);
                     if (2 + L1 - L0 < NM) mma(ws[u], fr[PH % 2], ph_tag, 2 + L1 - L0, NM);
-                } else {
-                    mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
-#pragma unroll
-                    for (int i = 0; i < BT; i++) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             };
@@ -1112,11 +1136,14 @@ static int launch_smfmac_cfg(SmfParams &P, hipStream_t s)
 template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStream_t s)
 {
     if (variant < 0) {
-        // Large-batch default.  The 256 x 256 tile moves a quarter fewer bytes per flop through
-        // the vector caches, but with its K step split in four phases (LDS reads of one phase
-        // behind the MFMAs of the other) the 256 x 128 tile runs as fast per flop on shapes with
-        // many tiles (8192^2 x 4096: 267 us both) and fills the CUs better on shapes with few.
-        variant = 6;
+        // Large-batch default.  The 256 x 256 tile moves a quarter fewer bytes per flop through the
+        // vector caches and is 2-4 % faster per flop in steady state (16384 x 4096 x 4096 tokens:
+        // 267 against 273 us; 8192^2 x 4096, 2:8: 250 against 260); what decides is how the tiles
+        // fill the chip: rounds of 256 tiles, a 256 x 256 tile taking twice the time of a 256 x 128
+        // one (two of which share a CU when there are more than 256).
+        const int64_t tm = (P.M + 255) / 256, t256 = tm * ((P.T + 255) / 256), t128 = tm * ((P.T + 127) / 128);
+        const double cost128 = (double)((t128 + 255) / 256), cost256 = (double)((t256 + 255) / 256) * 2.0 / 1.025;
+        variant = (P.ksplit <= 1 && cost256 < cost128) ? 8 : 6;
     }
     switch (variant) {
     case 0: return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);  // register-prefetch kernel, 256 lines x 128 tokens: any K
