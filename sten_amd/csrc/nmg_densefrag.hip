@@ -488,7 +488,19 @@ __global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
         }
     }
     pin_acc();
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // The loads of the steps beyond the last are still in flight and nothing reads what they bring:
+    // every register of the ring passes through the final wait, so that none of them is given to
+    // the epilogue while a load may still land in it.
+    static_assert(DD_D == 2 && FB == 2, "the final wait lists three weight sets of two fragment rows");
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(ws[0].a[0][0]), "+v"(ws[0].a[0][1]), "+v"(ws[0].a[0][2]), "+v"(ws[0].a[0][3]),
+                   "+v"(ws[0].a[1][0]), "+v"(ws[0].a[1][1]), "+v"(ws[0].a[1][2]), "+v"(ws[0].a[1][3]),
+                   "+v"(ws[1].a[0][0]), "+v"(ws[1].a[0][1]), "+v"(ws[1].a[0][2]), "+v"(ws[1].a[0][3]),
+                   "+v"(ws[1].a[1][0]), "+v"(ws[1].a[1][1]), "+v"(ws[1].a[1][2]), "+v"(ws[1].a[1][3]),
+                   "+v"(ws[2].a[0][0]), "+v"(ws[2].a[0][1]), "+v"(ws[2].a[0][2]), "+v"(ws[2].a[0][3]),
+                   "+v"(ws[2].a[1][0]), "+v"(ws[2].a[1][1]), "+v"(ws[2].a[1][2]), "+v"(ws[2].a[1][3])
+                 :
+                 : "memory");
     asm volatile("s_barrier" ::: "memory");
     if (P.ksplit > 1) {
         store_partial_tile<FB, TB>(acc, P.part + (int64_t)slice * P.T * P.part_ld, P.part_ld, lane,

@@ -626,7 +626,17 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
         }
     }
     pin_acc();
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // The loads of the steps beyond the last are still in flight and nothing reads what they bring:
+    // every register of the ring passes through the final wait, so that none of them is given to
+    // the epilogue while a load may still land in it.
+    static_assert(DR_D == 3 && FB == 2, "the final wait lists four weight sets of two fragment rows");
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+a"(ws[0].a[0][0]), "+a"(ws[0].a[0][1]), "+a"(ws[0].a[1][0]), "+a"(ws[0].a[1][1]), "+v"(ws[0].ix[0]), "+v"(ws[0].ix[1]),
+                   "+a"(ws[1].a[0][0]), "+a"(ws[1].a[0][1]), "+a"(ws[1].a[1][0]), "+a"(ws[1].a[1][1]), "+v"(ws[1].ix[0]), "+v"(ws[1].ix[1]),
+                   "+a"(ws[2].a[0][0]), "+a"(ws[2].a[0][1]), "+a"(ws[2].a[1][0]), "+a"(ws[2].a[1][1]), "+v"(ws[2].ix[0]), "+v"(ws[2].ix[1]),
+                   "+a"(ws[3].a[0][0]), "+a"(ws[3].a[0][1]), "+a"(ws[3].a[1][0]), "+a"(ws[3].a[1][1]), "+v"(ws[3].ix[0]), "+v"(ws[3].ix[1])
+                 :
+                 : "memory");
     asm volatile("s_barrier" ::: "memory");
     if (P.ksplit > 1) {
         store_partial_tile<FB, TB>(acc, P.part + (int64_t)slice * P.T * P.part_ld, P.part_ld, lane,
@@ -924,7 +934,13 @@ __global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_decode_staged_kernel(S
             __builtin_amdgcn_sched_barrier(0);
         }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // the last loads (beyond the wavefront's range) are in flight and unused: their registers pass
+    // through the final wait, so that none is reused while a load may still land in it
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(as[0].a[0][0]), "+v"(as[0].a[0][1]), "+v"(as[0].a[1][0]), "+v"(as[0].a[1][1]), "+v"(as[0].ix[0]), "+v"(as[0].ix[1]),
+                   "+v"(as[1].a[0][0]), "+v"(as[1].a[0][1]), "+v"(as[1].a[1][0]), "+v"(as[1].a[1][1]), "+v"(as[1].ix[0]), "+v"(as[1].ix[1])
+                 :
+                 : "memory");
     __syncthreads();   // every wavefront is done with its staging area: reuse it for the reduction
     float(*red)[32][17] = (float(*)[32][17])smem;
     // D[row = line][col = token]: lane holds token j, lines 8*(r/4) + 4*h + r%4

@@ -396,7 +396,12 @@ __global__ __launch_bounds__(64 * NW) void w4_linear_staged_kernel(W4Params P)
             __builtin_amdgcn_sched_barrier(0);
         }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // the last loads (beyond the wavefront's range) are in flight and unused: their registers pass
+    // through the final wait, so that none is reused while a load may still land in it
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(ws[0].a), "+v"(ws[0].ix), "+v"(ws[0].s), "+v"(ws[1].a), "+v"(ws[1].ix), "+v"(ws[1].s)
+                 :
+                 : "memory");
     __syncthreads();
     float(*red)[32][17] = (float(*)[32][17])w4_smem;
     if (j < 16) {

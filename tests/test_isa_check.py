@@ -97,3 +97,21 @@ def test_spill_of_a_register_in_flight_and_spill_in_a_streaming_loop():
 \ts_waitcnt vmcnt(0)
 """)
     assert p == [] and len(C.notes) == 2
+
+
+def test_register_of_an_unused_load_reused_before_the_wait():
+    # a load whose result nobody reads (a prefetch beyond the last step) still lands: its
+    # destination must not be given to other values before the wait that covers it
+    p = run("""
+\tglobal_load_dwordx4 v[4:7], v1, s[2:3]
+\tv_accvgpr_read_b32 v5, a32
+\ts_waitcnt vmcnt(0)
+\tv_cvt_f16_f32_e32 v9, v5
+""")
+    assert len(p) == 1 and "v_accvgpr_read_b32 v5, a32" in p[0]
+    ok = run("""
+\tglobal_load_dwordx4 v[4:7], v1, s[2:3]
+\ts_waitcnt vmcnt(0)
+\tv_accvgpr_read_b32 v5, a32
+""")
+    assert ok == []
