@@ -39,15 +39,7 @@ const int8_t *host_order(int n, int m);
 int device_order(int n, int m, const int8_t **d_order);
 // 256 bytes of zeros on the current device (file-scope array, never written).
 int device_zero_page(const void **d_zero);
-// Workgroups that start together run their K loops in lock step: every CU of an XCD issues its
-// loads, then its matrix instructions, in the same clocks.  A start delay of 0 .. 3 x 512 clocks,
-// by the workgroup's place in its XCD (consecutive blockIdx.x / 8), puts them in four phases
-// (measured: 3-6 % on the masked weight gradient and the sparse product, nothing on the dense one).
-__device__ __forceinline__ void skew_start()
-{
-    const int sk = ((blockIdx.x >> 3) & 3) * 8;
-    for (int i = 0; i < sk; i++) __builtin_amdgcn_s_sleep(1);
-}
+
 
 inline size_t dtype_size(int dtype)
 {

@@ -131,7 +131,6 @@ template <typename T, int MODE> __global__ __launch_bounds__(256, 1) void sddmm_
     // Workgroup -> tile.  Consecutive ids are dealt round-robin to the 8 XCDs: give each XCD a
     // contiguous run of ids, and walk the grid in bands of 4 position tiles, so that a run covers
     // a compact block of tiles whose operands stay in that XCD's L2.
-    skew_start();
     int id = blockIdx.x;
     const int ntiles = P.tiles_p * P.tiles_l;
     if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);

@@ -315,7 +315,6 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    skew_start();
     int id = blockIdx.x;
     const int ntiles = P.tiles_m * P.tiles_n;
     // slices of the reduction: the slices of a tile are workgroups ntiles apart
