@@ -37,12 +37,14 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
+PEAK_FP32_TFLOPS = 157.3    # MI355X dense fp32 MFMA
 ROTATE_BYTES = 512 * 1024 * 1024
 PEAK_HBM_GBS = 8000.0
 SETTLE_S = 0.08                # untimed load before the timed steps (see measure())
 
 WORKLOADS = {
     # name: (kind, M, K, tokens, n, m, g, description)
+    "c1": ("fwd", 768, 768, 256, 2, 4, 16, "configs[0]: W 768x768 fp32 2:4:16 x 256 tokens, forward (the reference's own CPU-runnable case; fp32 matrix cores)"),
     "c2": ("fwd", 4096, 4096, 2048, 2, 4, 16, "configs[1]: W 4096x4096 fp16 2:4:16 along K x 2048 tokens, forward"),
     "target_2_4": ("fwd", 4096, 11008, 2048, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 2048 tokens, forward"),
     "target_2_4_4k": ("fwd", 4096, 11008, 4096, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 4096 tokens, forward"),
@@ -82,7 +84,7 @@ PMC_SUMMARIES = {
 }
 
 # measured beside the headline workload in the default run: (workload, steps, warm-up)
-ALSO = [("c2", 50, 10), ("c3_1_8", 20, 5), ("c3_2_8", 20, 5), ("c3_4_8", 20, 5),
+ALSO = [("c1", 50, 10), ("c2", 50, 10), ("c3_1_8", 20, 5), ("c3_2_8", 20, 5), ("c3_4_8", 20, 5),
         ("decode_1", 50, 10), ("decode_4", 50, 10), ("decode_8", 50, 10), ("decode_16", 50, 10),
         ("c4_b1", 50, 10), ("c4_b4", 50, 10), ("c4_b16", 50, 10),
         ("sparsify_c2", 20, 5), ("c5_step", 10, 3), ("c5_train", 10, 3)]
@@ -207,7 +209,8 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
     # copies of it in turn, more than 512 MiB in all.
     copies, turn = 1, [0]
     torch.manual_seed(0)
-    W = (torch.randn(M, K) * 0.02).half().to(dev)
+    dt = torch.float32 if workload == "c1" else torch.float16
+    W = (torch.randn(M, K) * 0.02).to(dt).to(dev)
 
     if kind in ("step", "train"):
         # the registered F.linear through the dispatch layer, compressed weight gradient
@@ -267,7 +270,7 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
             X = torch.randn(N, M).half().to(dev)      # upstream gradient dY [tokens, out features]
             rd = 0
         else:
-            X = torch.randn(N, K).half().to(dev)
+            X = torch.randn(N, K).to(dt).to(dev)
             rd = 1
 
         def step():
@@ -335,12 +338,13 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
         dense_flops = 2.0 * M * K * N * (3 if kind in ("step", "train") else 1)
         eff_flops = dense_flops * n / m
         achieved = eff_flops / (kern_ms * 1e-3) / 1e12
+        peak = PEAK_FP32_TFLOPS if workload == "c1" else PEAK_FP16_TFLOPS
         row.update({
             "metric": "nmg sparse x dense GEMM TFLOP/s (dense-equiv)",
             "value": dense_flops / wall / 1e12, "unit": "TFLOP/s",
             "effective_tflops": eff_flops / wall / 1e12,
-            "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP16_TFLOPS,
-                         "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS, "traffic": None,
+            "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak,
+                         "unit": "TFLOP/s", "frac": achieved / peak, "traffic": None,
                          "flops": "effective non-zero (2*M*K*N*n/m); dense-equivalent is m/n times this"},
         })
     else:
@@ -395,7 +399,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": row["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16", "data": "synthetic",
+        "dtype": "f32" if args.workload == "c1" else "f16", "data": "synthetic",
         "config": {"workload": desc, "kernel": args.kernel, "variant": args.variant, "launch": row["launch"],
                    "settle": f"{row['settle_steps']} more untimed steps ({SETTLE_S * 1e3:.0f} ms of load) between the "
                              "warm-up and the timed steps: the clocks dip for 10-60 ms after an idle spell",
@@ -405,7 +409,7 @@ def main():
     for key in ("effective_tflops", "algorithmic_bytes", "weight_copies"):
         if key in row:
             out["config"][key] = row[key]
-    if kind in ("fwd", "grad_x") and not args.no_ceiling:
+    if kind in ("fwd", "grad_x") and not args.no_ceiling and args.workload != "c1":
         # The instruction of the dominant kernel, issued from registers with nothing else going on:
         # the 2.5 PFLOP/s behind `peak` assume 2.4 GHz, which random operands do not sustain, and the
         # 32x32x32 sparse instruction stays below its nominal rate even on zeros.
@@ -425,7 +429,7 @@ def main():
             also[name] = {"us": r["kernel_ms"] * 1e3, "value": r["value"], "unit": r["unit"],
                           "frac": r["roofline"]["frac"], "bound": r["roofline"]["bound"]}
         out["config"]["also"] = also
-    if not args.no_cpu and args.workload in ("c2", "target_2_4"):
+    if not args.no_cpu and args.workload in ("c1", "c2", "target_2_4"):
         out["cpu_baseline"] = cpu_baseline(M, K, N, n, m, g)
     if not args.no_cpu and kind == "sparsify":
         out["cpu_baseline"] = cpu_baseline_sparsify(M, K, n, m, g)

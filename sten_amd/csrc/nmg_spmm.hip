@@ -62,12 +62,14 @@ struct SpmmParams {
     int n, m, c, pat_bytes;
 };
 
-constexpr int BM = 128, BN = 128;
-
-template <typename T, bool REDUCE_SPARSE>
+// Tile BM tokens x BN outputs per workgroup of 2 x 2 wavefronts: 128 x 128, or 64 x 64 for products
+// whose 128 x 128 tiles would leave most of the CUs without work.
+template <typename T, bool REDUCE_SPARSE, int BM, int BN>
 __global__ __launch_bounds__(256) void spmm_mfma_kernel(SpmmParams P)
 {
     using M = Mma<T>;
+    constexpr int WMT = BM / 2, WNT = BN / 2;   // tokens x outputs per wavefront
+    constexpr int MI = WMT / 32, NJ = WNT / 32; // 32 x 32 accumulator blocks per wavefront
     constexpr int BK = M::BK, LDSW = BK + M::PAD;
     __shared__ __align__(16) T As[BM * LDSW];
     __shared__ __align__(16) T Bs[BN * LDSW];
@@ -85,11 +87,11 @@ __global__ __launch_bounds__(256) void spmm_mfma_kernel(SpmmParams P)
     const T *X = (const T *)P.x;
     const T *pkv = (const T *)P.pk_val;
 
-    f32x16 acc[2][2];
+    f32x16 acc[MI][NJ];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < NJ; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
@@ -140,19 +142,18 @@ __global__ __launch_bounds__(256) void spmm_mfma_kernel(SpmmParams P)
         // ---- MFMA ----
 #pragma unroll
         for (int kk = 0; kk < BK; kk += M::KPI) {
-            typename M::Frag a[2], b[2];
+            typename M::Frag a[MI], b[NJ];
             const int koff = kk + (lane >> 5) * M::EPL;
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const T *pa = &As[(wm * 64 + i * 32 + (lane & 31)) * LDSW + koff];
-                const T *pb = &Bs[(wn * 64 + i * 32 + (lane & 31)) * LDSW + koff];
-                a[i] = *(const typename M::Frag *)pa;
-                b[i] = *(const typename M::Frag *)pb;
-            }
+            for (int i = 0; i < MI; i++)
+                a[i] = *(const typename M::Frag *)&As[(wm * WMT + i * 32 + (lane & 31)) * LDSW + koff];
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int j = 0; j < NJ; j++)
+                b[j] = *(const typename M::Frag *)&Bs[(wn * WNT + j * 32 + (lane & 31)) * LDSW + koff];
 #pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = M::run(a[i], b[j], acc[i][j]);
+            for (int i = 0; i < MI; i++)
+#pragma unroll
+                for (int j = 0; j < NJ; j++) acc[i][j] = M::run(a[i], b[j], acc[i][j]);
         }
     }
 
@@ -161,15 +162,15 @@ __global__ __launch_bounds__(256) void spmm_mfma_kernel(SpmmParams P)
     T *Y = (T *)P.y;
     const T *bias = (const T *)P.bias;
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int64_t o = o0 + wn * 64 + j * 32 + (lane & 31);
+    for (int j = 0; j < NJ; j++) {
+        const int64_t o = o0 + wn * WNT + j * 32 + (lane & 31);
         if (o >= P.O) continue;
         const float bv = bias ? to_f32(bias[o]) : 0.f;
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (int i = 0; i < MI; i++) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int64_t tok = tok0 + wm * 64 + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                const int64_t tok = tok0 + wm * WMT + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
                 if (tok < P.T) {
                     T out;
                     from_f32(acc[i][j][r] + bv, out);
@@ -252,11 +253,20 @@ template <typename T> static int launch_spmm(SpmmParams &P, int reduce_sparse, i
         else
             hipLaunchKernelGGL((spmm_skinny_kernel<T, 16>), grid, dim3(256), 0, s, P);
     } else {
-        dim3 grid((unsigned)((P.O + BN - 1) / BN), (unsigned)((P.T + BM - 1) / BM));
-        if (reduce_sparse)
-            hipLaunchKernelGGL((spmm_mfma_kernel<T, true>), grid, dim3(256), 0, s, P);
-        else
-            hipLaunchKernelGGL((spmm_mfma_kernel<T, false>), grid, dim3(256), 0, s, P);
+        const int64_t big = ((P.O + 127) / 128) * ((P.T + 127) / 128);
+        if (big >= 128) {
+            dim3 grid((unsigned)((P.O + 127) / 128), (unsigned)((P.T + 127) / 128));
+            if (reduce_sparse)
+                hipLaunchKernelGGL((spmm_mfma_kernel<T, true, 128, 128>), grid, dim3(256), 0, s, P);
+            else
+                hipLaunchKernelGGL((spmm_mfma_kernel<T, false, 128, 128>), grid, dim3(256), 0, s, P);
+        } else {
+            dim3 grid((unsigned)((P.O + 63) / 64), (unsigned)((P.T + 63) / 64));
+            if (reduce_sparse)
+                hipLaunchKernelGGL((spmm_mfma_kernel<T, true, 64, 64>), grid, dim3(256), 0, s, P);
+            else
+                hipLaunchKernelGGL((spmm_mfma_kernel<T, false, 64, 64>), grid, dim3(256), 0, s, P);
+        }
     }
     NMG_HIP_TRY(hipGetLastError());
     return NMG_OK;
