@@ -121,7 +121,13 @@ static_assert(SD_D * SD_LPW < 64, "vmcnt is a 6-bit counter");
 // block, so the kept values are picked in registers (one byte permute with a per-pattern selector)
 // and stored by the lane itself; the slots of the lane's 64 (line, block) pairs are fetched when the
 // kernel starts and wait in registers through the product.  MODE 0: any n:m, through the staged tile.
-template <typename T, int MODE> __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
+// NT = true: the operands are given with the reduction (tokens) as their fast dim, L^T [G, T] and
+// P^T [S, T] (the weight gradient of torch.mm(W, B): grad_out [R, N] and B [C, N] as they lie in
+// memory).  An operand tile of a K step is then 256 feature rows of 64 bytes; a fragment -- the
+// lane's 8 consecutive tokens of its feature -- is one 16-byte LDS read, and the 16-byte pieces of
+// a row are XOR-swizzled with (row/4)%4 on the global side so that the reads hit every bank once.
+template <typename T, int MODE, bool NT = false>
+__global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
 {
     using Mm = SdMma<T>;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -219,13 +225,24 @@ template <typename T, int MODE> __global__ __launch_bounds__(256, 1) void sddmm_
     uint32_t g_off[SD_LPW];
 #pragma unroll
     for (int i = 0; i < SD_LPW; i++) {
-        const int tok = (((wave & 1) * 8 + i) << 1) + (lane >> 5);
-        const int chunk = (lane & 31) ^ ((tok & 3) << 2);
-        int64_t feat = f0 + chunk * 8;
-        if (feat > ext - 8) feat = ext - 8;   // columns beyond the extent feed outputs that are never stored
-        g_off[i] = (uint32_t)((tok * ld + feat) * 2);
+        if constexpr (NT) {
+            // load i fills feature rows (wave & 1) * 128 + 16 i + l/4, slot l%4 <- logical piece
+            // (l%4) ^ (row/4)%4 (8 tokens); rows beyond the extent repeat the last one (never stored)
+            const int row = (wave & 1) * 128 + 16 * i + (lane >> 2);
+            const int piece = (lane & 3) ^ ((row >> 2) & 3);
+            int64_t feat = f0 + row;
+            if (feat > ext - 1) feat = ext - 1;
+            g_off[i] = (uint32_t)(((feat - min(f0, ext - 1)) * ld + piece * 8) * 2);
+        } else {
+            const int tok = (((wave & 1) * 8 + i) << 1) + (lane >> 5);
+            const int chunk = (lane & 31) ^ ((tok & 3) << 2);
+            int64_t feat = f0 + chunk * 8;
+            if (feat > ext - 8) feat = ext - 8;   // columns beyond the extent feed outputs that are never stored
+            g_off[i] = (uint32_t)((tok * ld + feat) * 2);
+        }
     }
     const int tok_hi = lane >> 5;
+    const int nt_tok = ((lane & 3) ^ ((lane >> 4) & 3)) * 8;   // NT: first token of the lane's piece (the same in every load)
     const unsigned char *zero = (const unsigned char *)P.zero;
     // The DMA loads are written as instructions: they have no destination registers, so nothing
     // the compiler does with registers can race with them, and the compiler -- which would make
@@ -241,7 +258,7 @@ template <typename T, int MODE> __global__ __launch_bounds__(256, 1) void sddmm_
     auto step_of = [&](int kp) {
         const int kq = kp < KP ? kp : KP - 1;
         Step st;
-        st.b = gsrc + (int64_t)kq * SD_KS * ld * 2;
+        st.b = NT ? gsrc + (min(f0, ext - 1) * ld + (int64_t)kq * SD_KS) * 2 : gsrc + (int64_t)kq * SD_KS * ld * 2;
         st.dst = (uint32_t)(uintptr_t)(lds_ptr_t)(smem + (kp & (SD_NS - 1)) * SD_STAGE + (is_l ? SD_OP : 0) +
                                                   (wave & 1) * 8 * 1024);
         st.rem = (int)min((int64_t)SD_KS, P.T - (int64_t)kq * SD_KS);
@@ -252,7 +269,7 @@ template <typename T, int MODE> __global__ __launch_bounds__(256, 1) void sddmm_
     // scalar base + 32-bit lane offset form.
     auto issue_one = [&](const Step &st, int i, auto tail_tag) {
         if constexpr (decltype(tail_tag)::value) {
-            const int tok = (((wave & 1) * 8 + i) << 1) + tok_hi;
+            const int tok = NT ? nt_tok : (((wave & 1) * 8 + i) << 1) + tok_hi;
             const unsigned char *src = tok < st.rem ? st.b + g_off[i] : zero;
             asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                          :: "v"(src), "s"(st.dst + i * 1024) : "memory");
@@ -281,9 +298,28 @@ template <typename T, int MODE> __global__ __launch_bounds__(256, 1) void sddmm_
     };
     Frags fr[2];
     // fragment number w in the order the MFMAs first need them: a0, b0, b1, b2, b3, a1, a2, a3
+    // NT: lane (i = l%32, h = l/32) reads the 16 bytes of feature row 32*blk + i, piece 2*kk + h
+    // (stored at slot piece ^ (row/4)%4): its 8 tokens of k-step kk.
+    const int nt_row = (lane & 31) * 64, nt_sw = (lane >> 2) & 3, nt_h = lane >> 5;
     auto read_one = [&](Frags &f, const unsigned char *stage, int kk, int w) {
         const bool is_a = w == 0 || w >= 5;
         const int x = w == 0 ? 0 : (w >= 5 ? w - 4 : w - 1);
+        if constexpr (NT) {
+            const int at = ((is_a ? wm : wn) * 4 + x) * 32 * 64 + nt_row + (((2 * kk + nt_h) ^ nt_sw) << 4) + (is_a ? 0 : SD_OP);
+            union {
+                u32x4 u;
+                sd_i16x4 h[2];
+            } c;
+            c.u = *(const u32x4 *)(stage + at);
+            if (is_a) {
+                f.a[x][0] = c.h[0];
+                f.a[x][1] = c.h[1];
+            } else {
+                f.b[x][0] = c.h[0];
+                f.b[x][1] = c.h[1];
+            }
+            return;
+        }
 #pragma unroll
         for (int r = 0; r < 2; r++) {
             if (is_a)
@@ -635,23 +671,25 @@ extern "C" int nmg_slotmap(const int16_t *d_idx, int64_t G, int64_t S, int16_t *
     return NMG_OK;
 }
 
-extern "C" int nmg_sddmm(const void *d_lines, int64_t ld_lines, const void *d_pos, int64_t ld_pos, int64_t T,
-                         const int16_t *d_slot, int64_t G, int64_t S, void *d_val, int n, int m, int g,
-                         int dtype, void *stream)
+static int sddmm_impl(bool nt, const void *d_lines, int64_t ld_lines, const void *d_pos, int64_t ld_pos, int64_t T,
+                      const int16_t *d_slot, int64_t G, int64_t S, void *d_val, int n, int m, int g, int dtype,
+                      void *stream)
 {
     NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED, "the masked product takes f16/bf16");
     NMG_REQUIRE(host_order(n, m) != nullptr && g >= 1, NMG_ERR_ARG, "invalid n:m:g = %d:%d:%d", n, m, g);
     NMG_REQUIRE(G >= 0 && S >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
     const int64_t cg = binom(m, n) * g;
     NMG_REQUIRE(cg < 32768, NMG_ERR_ARG, "c*g must be below 2^15");
-    NMG_REQUIRE(ld_lines >= G && ld_pos >= S, NMG_ERR_ARG, "leading dimension smaller than row length");
+    NMG_REQUIRE(nt ? (ld_lines >= T && ld_pos >= T) : (ld_lines >= G && ld_pos >= S), NMG_ERR_ARG,
+                "leading dimension smaller than row length");
     if (G == 0 || S == 0 || n == 0) return NMG_OK;
     NMG_REQUIRE(T > 0, NMG_ERR_UNSUPPORTED, "no tokens: clear val instead");
-    NMG_REQUIRE(G % 8 == 0 && S % 8 == 0 && ld_lines % 8 == 0 && ld_pos % 8 == 0 &&
+    NMG_REQUIRE((nt || (G % 8 == 0 && S % 8 == 0)) && ld_lines % 8 == 0 && ld_pos % 8 == 0 &&
                     ((uintptr_t)d_lines % 16) == 0 && ((uintptr_t)d_pos % 16) == 0,
                 NMG_ERR_UNSUPPORTED, "needs extents and leading dimensions that are multiples of 8 and 16-byte aligned operands");
-    NMG_REQUIRE(ld_lines < ((int64_t)1 << 25) && ld_pos < ((int64_t)1 << 25), NMG_ERR_UNSUPPORTED,
+    NMG_REQUIRE(ld_lines < ((int64_t)1 << (nt ? 22 : 25)) && ld_pos < ((int64_t)1 << (nt ? 22 : 25)), NMG_ERR_UNSUPPORTED,
                 "leading dimension too large");
+    NMG_REQUIRE(!nt || T % 8 == 0, NMG_ERR_UNSUPPORTED, "reduction-contiguous operands need a token count that is a multiple of 8");
     NMG_REQUIRE(d_lines && d_pos && d_slot && d_val, NMG_ERR_ARG, "null device pointer");
     SddmmParams P{};
     if (int rc = device_order(n, m, &P.order)) return rc;
@@ -696,6 +734,10 @@ extern "C" int nmg_sddmm(const void *d_lines, int64_t ld_lines, const void *d_po
     };
     auto launch_t = [&](auto tag) -> int {
         using T = decltype(tag);
+        if (nt) {   // reduction-contiguous operands: 2:4 in registers, every other pattern through the staged tile
+            if (in_regs && n == 2 && S % 4 == 0) return launch(sddmm_kernel<T, 2, true>);   // (no padded positions)
+            return launch(sddmm_kernel<T, 0, true>);
+        }
         if (in_regs8) {
             if (n == 1) return launch(sddmm_kernel<T, 9>);
             if (n == 2) return launch(sddmm_kernel<T, 10>);
@@ -713,4 +755,18 @@ extern "C" int nmg_sddmm(const void *d_lines, int64_t ld_lines, const void *d_po
     if (rc) return rc;
     NMG_HIP_TRY(hipGetLastError());
     return NMG_OK;
+}
+
+extern "C" int nmg_sddmm(const void *d_lines, int64_t ld_lines, const void *d_pos, int64_t ld_pos, int64_t T,
+                         const int16_t *d_slot, int64_t G, int64_t S, void *d_val, int n, int m, int g,
+                         int dtype, void *stream)
+{
+    return sddmm_impl(false, d_lines, ld_lines, d_pos, ld_pos, T, d_slot, G, S, d_val, n, m, g, dtype, stream);
+}
+
+extern "C" int nmg_sddmm_nt(const void *d_lines_t, int64_t ld_lines, const void *d_pos_t, int64_t ld_pos, int64_t T,
+                            const int16_t *d_slot, int64_t G, int64_t S, void *d_val, int n, int m, int g,
+                            int dtype, void *stream)
+{
+    return sddmm_impl(true, d_lines_t, ld_lines, d_pos_t, ld_pos, T, d_slot, G, S, d_val, n, m, g, dtype, stream);
 }

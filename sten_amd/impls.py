@@ -126,7 +126,11 @@ def install(api):
         gc = gc.to(w.dtype)
         gb = spmm(w, gc.t().contiguous(), reduce_dim=0).t()
         if compressed:
-            gw = wrap(_masked_weight_grad(w, gc.t(), b.t()), gc)
+            # grad_out [R, N] and B [C, N] are reduction-contiguous as they lie: no transposing copies
+            if w.masked_product_supported(gc, b, reduction_last=True):
+                gw = wrap(w.masked_product(gc, b, reduction_last=True), gc)
+            else:
+                gw = wrap(_masked_weight_grad(w, gc.t(), b.t()), gc)
         else:
             gw = torch.mm(gc, b.t())
         return gw, gb

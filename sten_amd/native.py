@@ -68,6 +68,7 @@ SIGNATURES = {
     "nmg_spmm_smfmac_splitk": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _P, _I64, _P]),
     "nmg_slotmap": (_I, [_P, _I64, _I64, _P, _I, _I, _I, _P]),
     "nmg_sddmm": (_I, [_P, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _I, _I, _I, _I, _P]),
+    "nmg_sddmm_nt": (_I, [_P, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _I, _I, _I, _I, _P]),
     "nmg_perfect_nm": (_I, [_P, _I64, _I64, _I64, _P, _P, _I, _I, _I, _P]),
     "nmg_perfect_nm_to_dense": (_I, [_P, _P, _I64, _I64, _I64, _P, _I, _I, _I, _P]),
     "nmg_noalloc_scratch_bytes": (_I64, []),

@@ -296,18 +296,22 @@ class GroupedNMTensor:
         self._slotmap = (key, slot)
         return slot
 
-    def masked_product(self, rows_op, cols_op):
+    def masked_product(self, rows_op, cols_op, reduction_last=False):
         """New tensor with this tensor's pattern whose kept entries are those of
         ``rows_op^T @ cols_op`` (``rows_op`` [T, R], ``cols_op`` [T, C] for a weight [R, C]): the
         weight gradient of a linear layer, accumulated in fp32 and written straight into the
-        ``val`` layout.  16-bit types; extents that are multiples of 8."""
+        ``val`` layout.  16-bit types; extents that are multiples of 8.
+        ``reduction_last=True`` takes the operands transposed, ``rows_op`` [R, T] and ``cols_op``
+        [C, T] (the product ``rows_op @ cols_op^T``, as the weight gradient of ``torch.mm(W, B)``
+        finds them: grad_out and B); T must then be a multiple of 8, R and C may be anything."""
         lay = self.layout
         R, C = lay.dense_shape
         native.require_gpu(rows_op, cols_op, self.val)
-        if rows_op.dim() != 2 or cols_op.dim() != 2 or rows_op.shape[0] != cols_op.shape[0] \
-                or rows_op.shape[1] != R or cols_op.shape[1] != C:
-            raise native.NmgError(
-                f"operands must be [T, {R}] and [T, {C}], got {tuple(rows_op.shape)} and {tuple(cols_op.shape)}")
+        td, fd = (1, 0) if reduction_last else (0, 1)     # token dim / feature dim of the operands
+        if rows_op.dim() != 2 or cols_op.dim() != 2 or rows_op.shape[td] != cols_op.shape[td] \
+                or rows_op.shape[fd] != R or cols_op.shape[fd] != C:
+            want = f"[{R}, T] and [{C}, T]" if reduction_last else f"[T, {R}] and [T, {C}]"
+            raise native.NmgError(f"operands must be {want}, got {tuple(rows_op.shape)} and {tuple(cols_op.shape)}")
         dt = self.val.dtype
         if rows_op.dtype != dt or cols_op.dtype != dt:
             raise native.NmgError(f"dtype mismatch: operands {rows_op.dtype} / {cols_op.dtype}, weight {dt}")
@@ -317,13 +321,14 @@ class GroupedNMTensor:
             cols_op = cols_op.contiguous()
         lines, pos = (rows_op, cols_op) if lay.group_dim == 0 else (cols_op, rows_op)
         val = torch.empty_like(self.val)
-        T = rows_op.shape[0]
+        T = rows_op.shape[td]
         if T == 0:
             val.zero_()
         else:
             slot = self.slotmap()
+            entry = native.load().nmg_sddmm_nt if reduction_last else native.load().nmg_sddmm
             with torch.cuda.device(val.device):
-                native.check(native.load().nmg_sddmm(
+                native.check(entry(
                     native.ptr(lines), lines.stride(0), native.ptr(pos), pos.stride(0), T, native.ptr(slot),
                     lay.G, lay.S, native.ptr(val), lay.n, lay.m, lay.group_size, native.dtype_code(dt),
                     native.stream_ptr(val.device)))
@@ -331,13 +336,15 @@ class GroupedNMTensor:
         out.spmm_opt = dict(self.spmm_opt)
         return out
 
-    def masked_product_supported(self, rows_op, cols_op):
+    def masked_product_supported(self, rows_op, cols_op, reduction_last=False):
         lay = self.layout
-        return (len(lay.dense_shape) == 2 and self.val.dtype in (torch.float16, torch.bfloat16)
-                and rows_op.dtype == self.val.dtype and cols_op.dtype == self.val.dtype
-                and lay.dense_shape[0] % 8 == 0 and lay.dense_shape[1] % 8 == 0
-                and all(t.stride(1) != 1 or (t.stride(0) % 8 == 0 and t.data_ptr() % 16 == 0)
-                        for t in (rows_op, cols_op)))
+        ok = (len(lay.dense_shape) == 2 and self.val.dtype in (torch.float16, torch.bfloat16)
+              and rows_op.dtype == self.val.dtype and cols_op.dtype == self.val.dtype
+              and all(t.stride(1) != 1 or (t.stride(0) % 8 == 0 and t.data_ptr() % 16 == 0)
+                      for t in (rows_op, cols_op)))
+        if reduction_last:
+            return ok and rows_op.shape[1] % 8 == 0 and max(rows_op.stride(0), cols_op.stride(0)) < 2 ** 22
+        return ok and lay.dense_shape[0] % 8 == 0 and lay.dense_shape[1] % 8 == 0
 
     def fragpack(self):
         """Operand of the sparse-matrix-core kernel (values + 2-bit positions in instruction

@@ -165,3 +165,59 @@ def test_training_step_uses_the_fused_kernel():
     w = sp.weight.wrapped_tensor
     ref = w.clone_layout((gy.double().t() @ x.detach().double()).half())
     assert float((g.val.float() - ref.val.float()).norm() / ref.val.float().norm()) <= 1e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("R,C,T,n,m,g,sd", [
+    (256, 256, 64, 2, 4, 16, 1),
+    (200, 136, 40, 2, 4, 4, 1),          # ragged lines and positions, tokens end inside a K step
+    (203, 131, 24, 2, 4, 4, 0),          # extents that are no multiples of 8: fine in this form
+    (520, 264, 104, 1, 8, 2, 1),         # patterns outside 2:4 go through the staged epilogue
+    (264, 776, 136, 4, 8, 2, 0),
+    (96, 528, 200, 3, 6, 2, 1),
+    (768, 1024, 160, 2, 4, 1, 1),
+])
+def test_masked_product_reduction_contiguous_operands(dtype, R, C, T, n, m, g, sd):
+    # operands given as [R, T] and [C, T] (the weight gradient of torch.mm(W, B)): same values as
+    # the token-major form on the transposed copies, and the oracle's gather of the fp64 product
+    print(f"case sddmm nt {dtype} R={R} C={C} T={T} {n}:{m}:{g} sd={sd}", flush=True)
+    W = seeded((R, C), dtype, seed=R + C, std=0.5)
+    gy = seeded((R, T), dtype, seed=5)
+    b = seeded((C, T), dtype, seed=6)
+    _, idx, lay = oracle_sparsify(W, n, m, sd, g, 1 - sd)
+    ref, real = oracle_masked_grad(gy.t(), b.t(), idx, lay)
+    w = sten.GroupedNMTensor.from_dense(W.to(DEV), n, m, sparse_dim=sd, group_size=g, group_dim=1 - sd)
+    gw = w.masked_product(gy.to(DEV), b.to(DEV), reduction_last=True)
+    got = to_np(gw.val).astype(np.float64)
+    assert not got[~real].any()
+    assert rel_l2(got, ref) <= TOL[dtype]
+    if R % 8 == 0 and C % 8 == 0:
+        other = w.masked_product(gy.t().contiguous().to(DEV), b.t().contiguous().to(DEV))
+        assert torch.equal(gw.val, other.val)      # same products in the same order
+    # strided operands (row pitch larger than T)
+    big = torch.zeros((R, T + 24), dtype=dtype)
+    big[:, 8:8 + T] = gy
+    gw2 = w.masked_product(big.to(DEV)[:, 8:8 + T], b.to(DEV), reduction_last=True)
+    assert torch.equal(gw2.val, gw.val)
+
+
+def test_masked_product_reduction_contiguous_argument_errors():
+    W = torch.randn(64, 64).half().to(DEV)
+    w = sten.GroupedNMTensor.from_dense(W, 2, 4, sparse_dim=1, group_size=4, group_dim=0)
+    with pytest.raises(native.NmgError):   # token counts differ
+        w.masked_product(torch.randn(64, 16, device=DEV).half(), torch.randn(64, 24, device=DEV).half(), reduction_last=True)
+    with pytest.raises(native.NmgError):   # 12 tokens: not a multiple of 8
+        w.masked_product(torch.randn(64, 12, device=DEV).half(), torch.randn(64, 12, device=DEV).half(), reduction_last=True)
+
+
+def test_weight_gradient_of_torch_mm_from_its_operands_as_they_lie():
+    print("case sddmm nt on the operands of a torch.mm backward", flush=True)
+    torch.manual_seed(3)
+    R, C, N = 192, 256, 72
+    W = (torch.randn(R, C) * 0.1).half().to(DEV)
+    w = sten.GroupedNMTensor.from_dense(W, 2, 4, sparse_dim=1, group_size=8, group_dim=0)
+    B = torch.randn(C, N, device=DEV).half()
+    gc = torch.randn(R, N, device=DEV).half()
+    got = w.masked_product(gc, B, reduction_last=True)
+    ref = w.clone_layout((gc.double() @ B.double().t()).half())
+    assert float((got.val.float() - ref.val.float()).norm() / ref.val.float().norm()) <= 1e-3
