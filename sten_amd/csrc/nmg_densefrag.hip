@@ -534,20 +534,295 @@ template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_
     return NMG_OK;
 }
 
+// ------------------------------------------------- the same product with V_MFMA_F32_16X16X32
+// The 16 x 16 x 32 form of the instruction draws less power per flop than the 32 x 32 x 16 form
+// (from registers, random operands: 1.76-1.97 against 1.61-1.71 PFLOP/s), and with this skeleton
+// around it the difference stays.  Same operand, same ring, same counted waits as
+// dense_direct_kernel; what changes is who holds what:
+//   A fragment (16 outputs x 32 k): lane (r = l%16, kq = l/16) wants the 8 weights of output
+//     16*ab + r at k = 32*k32 + 8*kq + 0..7, which the densefrag operand stores in fragment
+//     (ob = ab/2, k16 = 2*k32 + kq/2) at lane 32*(kq%2) + 16*(ab%2) + r: a load still covers four
+//     runs of 256 contiguous bytes.
+//   B fragment (16 tokens x 32 k): lane (j = l%16, kq) reads the 16-byte chunk 4*k32 + kq of token
+//     row 16*tb + j; with the chunks XOR-swizzled by (row/2)%8 sixteen consecutive rows cover all
+//     banks.
+//   D: lane holds token l%16, outputs 4*(l/16) + 0..3 of the 16 x 16 block.
+// A wavefront owns 64 outputs x TB*16 tokens: 4 x TB accumulator blocks of 4 registers, all of
+// them in the accumulation registers.  A K step of 64 is two k-steps of 32; a phase is one
+// (k-step, token part) pair of 4 * TB / NH MFMAs.
+template <typename T> struct DfMma16;
+template <> struct DfMma16<__half> {
+    using F = df_f16x8;
+    __device__ static f32x4 run(F a, F b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+};
+template <> struct DfMma16<__hip_bfloat16> {
+    using F = df_bf16x8;
+    __device__ static f32x4 run(F a, F b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+};
+
+template <typename T, int TB, int NH>
+__global__ __launch_bounds__(256, 1) void dense16_direct_kernel(DfParams P)
+{
+    using Mm = DfMma16<T>;
+    constexpr int AB = 4;                                 // blocks of 16 outputs per wavefront
+    constexpr int TF = 256, TT = TB * 16;                 // workgroup tile: outputs x tokens
+    constexpr int STAGE = TT * 128;                       // activation bytes per K step
+    constexpr int XL = TT / 32;                           // DMA loads per wavefront per K step
+    constexpr int OPS = XL + 2 * AB;                      // memory operations per wavefront per K step
+    constexpr int BT = TB / NH;                           // token blocks per phase
+    constexpr int NP = 2 * NH;                            // phases per K step
+    constexpr int NM = AB * BT;                           // MFMAs per phase
+    static_assert(TB % NH == 0, "token blocks split evenly into phases");
+    static_assert(OPS * DD_D < 64, "vmcnt is a 6-bit counter");
+    static_assert(NP >= 2 && NP % 2 == 0, "fragment sets alternate by phase across K steps");
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    // workgroup -> tile as in dense_direct_kernel
+    int id = blockIdx.x;
+    const int ntiles = P.tiles_m * P.tiles_n;
+    if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
+    constexpr int GH = 4;
+    const int band = id / (GH * P.tiles_n);
+    const int band_h = min(P.tiles_m - band * GH, GH);
+    const int in_band = id - band * GH * P.tiles_n;
+    const int tile_m = band * GH + in_band % band_h, tile_n = in_band / band_h;
+    const int64_t f0 = (int64_t)tile_m * TF, t0 = (int64_t)tile_n * TT;
+    const int KP = P.KP;
+    const int ob0 = (int)(f0 / 32) + wave * 2;
+
+    const unsigned char *av_base[2];
+#pragma unroll
+    for (int o = 0; o < 2; o++) av_base[o] = (const unsigned char *)P.df + ((int64_t)(ob0 + o) * KP * 4) * 1024;
+    const int r16 = lane & 15, kq = lane >> 4;
+    const uint32_t lane_a = (uint32_t)((kq >> 1) * 1024 + ((kq & 1) * 32 + r16) * 16);
+    const unsigned char *x_base = (const unsigned char *)P.x;
+    uint32_t x_off[XL];
+#pragma unroll
+    for (int i = 0; i < XL; i++) {
+        const int row = (wave * XL + i) * 8 + (lane >> 3);
+        const int piece = lane & 7;
+        const int q = piece ^ ((row >> 1) & 7);   // logical 16-byte chunk stored at this piece
+        int64_t tok = t0 + row;
+        if (tok >= P.T) tok = P.T - 1;            // clamped rows are computed, never stored
+        x_off[i] = (uint32_t)((tok * P.ldx + q * 8) * 2);
+    }
+
+    struct WSet {
+        u32x4 a[AB][2];   // [block of 16 outputs][k-step of 32]
+    };
+    WSet ws[DD_D + 1];
+    // load number i (0 .. OPS-1) of K step kp: first the XL activation DMA loads, then the 2 * AB
+    // weight fragments.  Steps beyond the last repeat it: the operation count stays uniform, the
+    // data is unused.
+    auto issue_one = [&](int kp, WSet &w, int i) {
+        if (kp >= KP) kp = KP - 1;
+        if (i < XL) {
+            unsigned char *base = smem + (kp & (DD_NS - 1)) * STAGE;
+            const unsigned char *xb = x_base + (int64_t)kp * 128;
+#pragma unroll
+            for (int q = 0; q < XL; q++)
+                if (q == i)
+                    __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[q]),
+                                                     (lds_ptr_t)(base + (wave * XL + q) * 1024), 16, 0, 0);
+        } else {
+            // Written as instructions so that their completion is tracked by the explicit vmcnt
+            // waits below and by nothing else.
+#pragma unroll
+            for (int ab = 0; ab < AB; ab++)
+#pragma unroll
+                for (int k32 = 0; k32 < 2; k32++)
+                    if (XL + ab * 2 + k32 == i) {
+                        const unsigned char *av = av_base[ab >> 1] + (int64_t)kp * 4096;
+                        asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3"
+                                     : "=v"(w.a[ab][k32])
+                                     : "v"(lane_a), "s"(av), "n"(k32 * 2048 + (ab & 1) * 256)
+                                     : "memory");
+                    }
+        }
+    };
+
+    f32x4 acc[AB][TB];
+#pragma unroll
+    for (int i = 0; i < AB; i++)
+#pragma unroll
+        for (int t = 0; t < TB; t++) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    auto pin_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < AB; i++)
+#pragma unroll
+            for (int t = 0; t < TB; t++) asm volatile("" : "+a"(acc[i][t]));
+    };
+    pin_acc();
+
+    const int sw = (r16 >> 1) & 7;
+    int b_off[2];
+#pragma unroll
+    for (int k32 = 0; k32 < 2; k32++) b_off[k32] = r16 * 128 + (((k32 * 4 + kq) ^ sw) << 4);
+
+    struct BFrags {
+        u32x4 b[BT];
+    };
+    BFrags fr[2];
+    auto read_one = [&](BFrags &f, const unsigned char *base, int ph, int t) {
+        const int k32 = ph / NH, hh = ph % NH;
+        f.b[t] = *(const u32x4 *)(base + b_off[k32] + (hh * BT + t) * 16 * 128);
+    };
+    // MFMA number i of phase PH (i = ab * BT + t)
+    auto mma = [&](const WSet &w, const BFrags &f, auto ph_tag, int i) {
+        constexpr int PH = decltype(ph_tag)::value, K32 = PH / NH, HH = PH % NH;
+        const int ab = i / BT, t = i % BT;
+        union {
+            u32x4 u;
+            typename Mm::F v;
+        } ca, cb;
+        ca.u = w.a[ab][K32];
+        cb.u = f.b[t];
+        acc[ab][HH * BT + t] = Mm::run(ca.v, cb.v, acc[ab][HH * BT + t]);
+    };
+
+    // The counted wait: as in dense_direct_kernel -- OPS memory operations per K step, issued in
+    // order, all of step kp+DD_D before the wait of step kp; the set of step kp+1 passes through
+    // the wait as in/out operands.
+    static_assert(DD_NS > DD_D, "a stage must not be refilled while the step that reads it is in flight");
+    auto landed = [&](WSet &w) {
+        asm volatile("s_waitcnt vmcnt(%8) lgkmcnt(0)"
+                     : "+v"(w.a[0][0]), "+v"(w.a[0][1]), "+v"(w.a[1][0]), "+v"(w.a[1][1]),
+                       "+v"(w.a[2][0]), "+v"(w.a[2][1]), "+v"(w.a[3][0]), "+v"(w.a[3][1])
+                     : "n"((DD_D - 1) * OPS)
+                     : "memory");
+    };
+
+    // prologue: steps 0 .. DD_D-1 in flight, then wait for step 0
+#pragma unroll
+    for (int st = 0; st < DD_D; st++)
+#pragma unroll
+        for (int i = 0; i < OPS; i++) issue_one(st, ws[st], i);
+    landed(ws[0]);
+    asm volatile("s_barrier" ::: "memory");
+#pragma unroll
+    for (int t = 0; t < BT; t++) read_one(fr[0], smem, 0, t);
+
+    for (int kp0 = 0; kp0 < KP; kp0 += DD_D + 1) {
+#pragma unroll
+        for (int u = 0; u <= DD_D; u++) {
+            const int kp = kp0 + u;
+            if (kp >= KP) break;
+            const unsigned char *base = smem + (kp & (DD_NS - 1)) * STAGE;
+            const unsigned char *next = smem + ((kp + 1) & (DD_NS - 1)) * STAGE;
+            // A phase: its MFMAs, and behind one MFMA each the fragment reads of the next phase and
+            // this phase's share of the loads of step kp+DD_D (dealt out over all phases but the
+            // last).  The last phase waits for step kp+1 after two MFMAs, meets the other
+            // wavefronts and reads the first fragments of the next stage behind the rest.
+            auto phase = [&](auto ph_tag) {
+                constexpr int PH = decltype(ph_tag)::value;
+                if constexpr (PH == NP - 1) {
+                    mma(ws[u], fr[PH % 2], ph_tag, 0);
+                    mma(ws[u], fr[PH % 2], ph_tag, 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    landed(ws[(u + 1) % (DD_D + 1)]);
+                    asm volatile("s_barrier" ::: "memory");
+                    __builtin_amdgcn_sched_barrier(0);
+                    constexpr int SP = (NM - 2) / BT;
+#pragma unroll
+                    for (int i = 2; i < NM; i++) {
+                        mma(ws[u], fr[PH % 2], ph_tag, i);
+                        __builtin_amdgcn_sched_barrier(0);
+                        if ((i - 2) % SP == 0 && (i - 2) / SP < BT) read_one(fr[(PH + 1) % 2], next, 0, (i - 2) / SP);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                } else {
+                    constexpr int L0 = PH * OPS / (NP - 1), L1 = (PH + 1) * OPS / (NP - 1);
+                    constexpr int NOPS = BT + L1 - L0;
+                    constexpr int SP = NM / NOPS > 0 ? NM / NOPS : 1;
+                    static_assert(NOPS <= NM, "one memory instruction behind one MFMA");
+#pragma unroll
+                    for (int i = 0; i < NM; i++) {
+                        mma(ws[u], fr[PH % 2], ph_tag, i);
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (i % SP == 0 && i / SP < NOPS) {
+                            const int op = i / SP;
+                            if (op < BT)
+                                read_one(fr[(PH + 1) % 2], base, PH + 1, op);
+                            else
+                                issue_one(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)], L0 + op - BT);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            };
+            phase(std::integral_constant<int, 0>{});
+            phase(std::integral_constant<int, 1>{});
+            if constexpr (NP >= 4) {
+                phase(std::integral_constant<int, 2>{});
+                phase(std::integral_constant<int, 3>{});
+            }
+            if constexpr (NP >= 8) {
+                phase(std::integral_constant<int, 4>{});
+                phase(std::integral_constant<int, 5>{});
+                phase(std::integral_constant<int, 6>{});
+                phase(std::integral_constant<int, 7>{});
+            }
+            static_assert(NP == 2 || NP == 4 || NP == 8, "one, two or four token parts");
+        }
+    }
+    pin_acc();
+    // The loads of the steps beyond the last are still in flight and nothing reads what they bring:
+    // every register of the ring passes through the final wait.
+    static_assert(DD_D == 2, "the final wait lists three weight sets");
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(ws[0].a[0][0]), "+v"(ws[0].a[0][1]), "+v"(ws[0].a[1][0]), "+v"(ws[0].a[1][1]),
+                   "+v"(ws[0].a[2][0]), "+v"(ws[0].a[2][1]), "+v"(ws[0].a[3][0]), "+v"(ws[0].a[3][1]),
+                   "+v"(ws[1].a[0][0]), "+v"(ws[1].a[0][1]), "+v"(ws[1].a[1][0]), "+v"(ws[1].a[1][1]),
+                   "+v"(ws[1].a[2][0]), "+v"(ws[1].a[2][1]), "+v"(ws[1].a[3][0]), "+v"(ws[1].a[3][1]),
+                   "+v"(ws[2].a[0][0]), "+v"(ws[2].a[0][1]), "+v"(ws[2].a[1][0]), "+v"(ws[2].a[1][1]),
+                   "+v"(ws[2].a[2][0]), "+v"(ws[2].a[2][1]), "+v"(ws[2].a[3][0]), "+v"(ws[2].a[3][1])
+                 :
+                 : "memory");
+    asm volatile("s_barrier" ::: "memory");
+    const TileOut out{P.y, P.bias, P.O, P.T, P.ldy};
+    store_tile16<T, AB, TB>(acc, smem + wave * (TT * (AB * 32 + 16)), lane, f0 + wave * 64, t0, out);
+}
+
+template <typename T, int TB, int NH> static int launch_dense16(DfParams &P, hipStream_t s)
+{
+    constexpr int TT = TB * 16;
+    P.tiles_m = (int)((P.O + 255) / 256);
+    P.tiles_n = (int)((P.T + TT - 1) / TT);
+    dim3 grid((unsigned)(P.tiles_m * P.tiles_n));
+    constexpr size_t ring = (size_t)DD_NS * TT * 128, stg = (size_t)4 * TT * (4 * 32 + 16);
+    constexpr size_t lds = ring > stg ? ring : stg;
+    static_assert(lds <= 160 * 1024, "LDS");
+    auto k = dense16_direct_kernel<T, TB, NH>;
+    NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(k, grid, dim3(256), lds, s, P);
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
 template <typename T> static int launch_dense(DfParams &P, int variant, hipStream_t s)
 {
-    // 256 x 256 tiles (variant 1) move fewer bytes per flop through the vector caches and are 5-6 %
-    // faster per flop in steady state (8192^2 x 4096 tokens: 414 against 439 us); one workgroup per
-    // CU either way, so what decides is how full the last round of tiles is.  (A sixteen-phase form
-    // of the 256 x 256 tile once gave wrong values now and then; that form is gone, the eight-phase
-    // form here passes the static check of its hand-tracked loads and the repeated full-chip test.)
+    // 256 x 256 tiles move fewer bytes per flop through the vector caches and are 5-6 % faster per
+    // flop in steady state; one workgroup per CU either way, so what decides is how full the last
+    // round of tiles is.  Variants 0 / 1: 256 x 128 / 256 x 256 with the 32 x 32 x 16 instruction,
+    // 5 / 2: the same tiles with the 16 x 16 x 32 instruction, 9-15 % faster (8192^2 4:8 x 4096
+    // tokens: 346 against 405 us; 16384x4096 grad_input: 364 against 400; 4096^2 x 2048: 50 against
+    // 56), which is what the automatic choice takes.  (A sixteen-phase form of the 256 x 256 tile
+    // once gave wrong values now and then; that form is gone, the forms here pass the static check
+    // of their hand-tracked loads and the repeated full-chip test.)
     if (variant < 0) {
         const int64_t tm = (P.O + 255) / 256, t256 = tm * ((P.T + 255) / 256), t128 = tm * ((P.T + 127) / 128);
         const double fill256 = (double)t256 / (double)((t256 + 255) / 256 * 256);
         const double fill128 = (double)t128 / (double)((t128 + 255) / 256 * 256);
-        variant = (P.ksplit <= 1 && t256 >= 256 && fill256 * 1.055 >= fill128) ? 1 : 0;
+        variant = (P.ksplit <= 1 && t256 >= 256 && fill256 * 1.055 >= fill128) ? 2 : 5;
     }
     if (variant == 1) return launch_dense_direct<T, 2, 8, 4, 1, 2>(P, s);
+    if (variant == 2) return launch_dense16<T, 16, 2>(P, s);
+    if (variant == 3) return launch_dense16<T, 16, 4>(P, s);
+    if (variant == 4) return launch_dense16<T, 8, 1>(P, s);
+    if (variant == 5) return launch_dense16<T, 8, 2>(P, s);
     return launch_dense_direct<T, 2, 4, 4, 1, 1>(P, s);
 }
 
@@ -628,7 +903,7 @@ extern "C" int nmg_spmm_densefrag(const void *d_df, int64_t O, int64_t K, const 
 {
     NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED, "densefrag takes f16/bf16");
     NMG_REQUIRE(O >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
-    NMG_REQUIRE(variant >= -1 && variant <= 1, NMG_ERR_ARG, "unknown tile variant %d", variant);
+    NMG_REQUIRE(variant >= -1 && variant <= 5, NMG_ERR_ARG, "unknown tile variant %d", variant);
     NMG_REQUIRE(ldx >= K && ldy >= O, NMG_ERR_ARG, "leading dimension smaller than row length");
     NMG_REQUIRE(K % 64 == 0 && K > 0 && ldx % 8 == 0 && ((uintptr_t)d_x % 16) == 0, NMG_ERR_UNSUPPORTED,
                 "needs K %% 64 == 0 and 16-byte aligned activation rows");

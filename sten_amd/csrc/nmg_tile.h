@@ -6,6 +6,7 @@
 namespace nmg {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
 typedef const __attribute__((address_space(1))) void *glb_ptr_t;
@@ -29,30 +30,15 @@ struct TileOut {
 // staged through its own LDS region `stg` as [token][feature] so the global stores are 16 B per
 // lane and FB*64 B contiguous per token row.  fw / tw = first feature / token of the wavefront.
 // The caller guarantees that no load into LDS is pending.
-template <typename T, int FB, int TB>
-__device__ __forceinline__ void smf_store_tile(const f32x16 (&acc)[FB][TB], unsigned char *stg, int lane,
-                                               int64_t fw, int64_t tw, const TileOut &P)
+// Second half of the staged epilogues: NROWS token rows of FB*64 B (+16 B pad) lie in `stg`; every
+// lane moves 16 B per pass, FB*64 B contiguous per token row, adding the bias on the way.
+template <typename T, int FB, int NROWS>
+__device__ __forceinline__ void store_staged_rows(const unsigned char *stg, int lane, int64_t fw, int64_t tw,
+                                                  const TileOut &P)
 {
     constexpr int ROW = FB * 64 + 16;       // bytes per staged token row (16 B pad: conflict-free)
     constexpr int CPR = FB * 4;             // 16-byte chunks per row
     constexpr int RPP = 64 / CPR;           // token rows per pass of the wavefront
-    const int j = lane & 31, h = lane >> 5;
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-    for (int tb = 0; tb < TB; tb++)
-#pragma unroll
-        for (int fb = 0; fb < FB; fb++)
-#pragma unroll
-            for (int rq = 0; rq < 4; rq++) {
-                uint16_t hh[4];
-#pragma unroll
-                for (int i = 0; i < 4; i++) hh[i] = f32_to_bits16(acc[fb][tb][rq * 4 + i], (T *)nullptr);
-                uint2 pk;
-                pk.x = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
-                pk.y = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
-                *(uint2 *)(stg + (tb * 32 + j) * ROW + (fb * 32 + rq * 8 + h * 4) * 2) = pk;
-            }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     uint16_t *Y = (uint16_t *)P.y;
     const T *bias = (const T *)P.bias;
     const bool vec_ok = (P.ldy & 7) == 0 && ((uintptr_t)P.y & 15) == 0;
@@ -62,7 +48,7 @@ __device__ __forceinline__ void smf_store_tile(const f32x16 (&acc)[FB][TB], unsi
 #pragma unroll
     for (int i = 0; i < 8; i++) bv[i] = (bias && f + i < P.M) ? to_f32(bias[f + i]) : 0.f;
 #pragma unroll 4
-    for (int it = 0; it < TB * 32 / RPP; it++) {
+    for (int it = 0; it < NROWS / RPP; it++) {
         const int tl = it * RPP + lane / CPR;
         const int64_t tok = tw + tl;
         u32x4 v = *(const u32x4 *)(stg + tl * ROW + fc * 16);
@@ -89,6 +75,57 @@ __device__ __forceinline__ void smf_store_tile(const f32x16 (&acc)[FB][TB], unsi
                 if (f + i < P.M) dst[i] = (uint16_t)(w[i >> 1] >> ((i & 1) * 16));
         }
     }
+}
+
+template <typename T, int FB, int TB>
+__device__ __forceinline__ void smf_store_tile(const f32x16 (&acc)[FB][TB], unsigned char *stg, int lane,
+                                               int64_t fw, int64_t tw, const TileOut &P)
+{
+    constexpr int ROW = FB * 64 + 16;
+    const int j = lane & 31, h = lane >> 5;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int tb = 0; tb < TB; tb++)
+#pragma unroll
+        for (int fb = 0; fb < FB; fb++)
+#pragma unroll
+            for (int rq = 0; rq < 4; rq++) {
+                uint16_t hh[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) hh[i] = f32_to_bits16(acc[fb][tb][rq * 4 + i], (T *)nullptr);
+                uint2 pk;
+                pk.x = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
+                pk.y = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
+                *(uint2 *)(stg + (tb * 32 + j) * ROW + (fb * 32 + rq * 8 + h * 4) * 2) = pk;
+            }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    store_staged_rows<T, FB, TB * 32>(stg, lane, fw, tw, P);
+}
+
+// The 16 x 16 form of the instruction: a lane holds token l%16 and outputs 4*(l/16) + 0..3 of every
+// 16 x 16 block.  AB blocks of 16 outputs (a multiple of 2) x TB blocks of 16 tokens per wavefront.
+template <typename T, int AB, int TB>
+__device__ __forceinline__ void store_tile16(const f32x4 (&acc)[AB][TB], unsigned char *stg, int lane,
+                                             int64_t fw, int64_t tw, const TileOut &P)
+{
+    static_assert(AB % 2 == 0, "whole 32-output rows of the staging area");
+    constexpr int ROW = AB * 32 + 16;
+    const int j = lane & 15, q = lane >> 4;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int tb = 0; tb < TB; tb++)
+#pragma unroll
+        for (int ab = 0; ab < AB; ab++) {
+            uint16_t hh[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) hh[i] = f32_to_bits16(acc[ab][tb][i], (T *)nullptr);
+            uint2 pk;
+            pk.x = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
+            pk.y = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
+            *(uint2 *)(stg + (tb * 16 + j) * ROW + (ab * 16 + q * 4) * 2) = pk;
+        }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    store_staged_rows<T, AB / 2, TB * 16>(stg, lane, fw, tw, P);
 }
 
 // The same epilogue for a transposed output, Y[M, T] row-major (tokens contiguous): the
