@@ -583,6 +583,9 @@ __global__ __launch_bounds__(256, 1) void dense16_direct_kernel(DfParams P)
     // workgroup -> tile as in dense_direct_kernel
     int id = blockIdx.x;
     const int ntiles = P.tiles_m * P.tiles_n;
+    // slices of the reduction: the slices of a tile are workgroups ntiles apart
+    const int slice = P.ksplit > 1 ? id / ntiles : 0;
+    id -= slice * ntiles;
     if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
     constexpr int GH = 4;
     const int band = id / (GH * P.tiles_n);
@@ -590,15 +593,20 @@ __global__ __launch_bounds__(256, 1) void dense16_direct_kernel(DfParams P)
     const int in_band = id - band * GH * P.tiles_n;
     const int tile_m = band * GH + in_band % band_h, tile_n = in_band / band_h;
     const int64_t f0 = (int64_t)tile_m * TF, t0 = (int64_t)tile_n * TT;
-    const int KP = P.KP;
+    // K steps kp_lo .. kp_lo + KP - 1 of the operand's KPT (the host leaves no slice empty)
+    const int KPT = P.KP;
+    const int kp_per = P.ksplit > 1 ? (KPT + P.ksplit - 1) / P.ksplit : KPT;
+    const int kp_lo = slice * kp_per;
+    const int KP = min(KPT, kp_lo + kp_per) - kp_lo;
     const int ob0 = (int)(f0 / 32) + wave * 2;
 
     const unsigned char *av_base[2];
 #pragma unroll
-    for (int o = 0; o < 2; o++) av_base[o] = (const unsigned char *)P.df + ((int64_t)(ob0 + o) * KP * 4) * 1024;
+    for (int o = 0; o < 2; o++)
+        av_base[o] = (const unsigned char *)P.df + (((int64_t)(ob0 + o) * KPT + kp_lo) * 4) * 1024;
     const int r16 = lane & 15, kq = lane >> 4;
     const uint32_t lane_a = (uint32_t)((kq >> 1) * 1024 + ((kq & 1) * 32 + r16) * 16);
-    const unsigned char *x_base = (const unsigned char *)P.x;
+    const unsigned char *x_base = (const unsigned char *)P.x + (int64_t)kp_lo * 128;
     uint32_t x_off[XL];
 #pragma unroll
     for (int i = 0; i < XL; i++) {
@@ -782,6 +790,11 @@ __global__ __launch_bounds__(256, 1) void dense16_direct_kernel(DfParams P)
                  :
                  : "memory");
     asm volatile("s_barrier" ::: "memory");
+    if (P.ksplit > 1) {
+        store_partial_tile16<AB, TB>(acc, P.part + (int64_t)slice * P.T * P.part_ld, P.part_ld, lane,
+                                     f0 + wave * 64, t0, P.T);
+        return;
+    }
     const TileOut out{P.y, P.bias, P.O, P.T, P.ldy};
     store_tile16<T, AB, TB>(acc, smem + wave * (TT * (AB * 32 + 16)), lane, f0 + wave * 64, t0, out);
 }
@@ -791,7 +804,8 @@ template <typename T, int TB, int NH> static int launch_dense16(DfParams &P, hip
     constexpr int TT = TB * 16;
     P.tiles_m = (int)((P.O + 255) / 256);
     P.tiles_n = (int)((P.T + TT - 1) / TT);
-    dim3 grid((unsigned)(P.tiles_m * P.tiles_n));
+    const int slices = P.ksplit > 1 ? P.ksplit : 1;
+    dim3 grid((unsigned)(P.tiles_m * P.tiles_n * slices));
     constexpr size_t ring = (size_t)DD_NS * TT * 128, stg = (size_t)4 * TT * (4 * 32 + 16);
     constexpr size_t lds = ring > stg ? ring : stg;
     static_assert(lds <= 160 * 1024, "LDS");
@@ -799,6 +813,10 @@ template <typename T, int TB, int NH> static int launch_dense16(DfParams &P, hip
     NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(k, grid, dim3(256), lds, s, P);
     NMG_HIP_TRY(hipGetLastError());
+    if (slices > 1) {
+        const SplitSum Q{P.part, P.y, P.bias, P.O, P.T, P.ldy, P.part_ld, slices};
+        return launch_splitk_sum<T>(Q, s);
+    }
     return NMG_OK;
 }
 
@@ -816,7 +834,7 @@ template <typename T> static int launch_dense(DfParams &P, int variant, hipStrea
         const int64_t tm = (P.O + 255) / 256, t256 = tm * ((P.T + 255) / 256), t128 = tm * ((P.T + 127) / 128);
         const double fill256 = (double)t256 / (double)((t256 + 255) / 256 * 256);
         const double fill128 = (double)t128 / (double)((t128 + 255) / 256 * 256);
-        variant = (P.ksplit <= 1 && t256 >= 256 && fill256 * 1.055 >= fill128) ? 2 : 5;
+        variant = (P.ksplit <= 1 && t256 >= 256 && fill256 * 1.055 >= fill128) ? 3 : 5;
     }
     if (variant == 1) return launch_dense_direct<T, 2, 8, 4, 1, 2>(P, s);
     if (variant == 2) return launch_dense16<T, 16, 2>(P, s);
@@ -960,6 +978,5 @@ extern "C" int nmg_spmm_densefrag_splitk(const void *d_df, int64_t O, int64_t K,
     P.part = (float *)d_workspace;
     P.part_ld = tiles_m * 256;
     hipStream_t s = (hipStream_t)stream;
-    return dtype == NMG_F16 ? launch_dense_direct<__half, 2, 4, 4, 1, 1>(P, s)
-                            : launch_dense_direct<__hip_bfloat16, 2, 4, 4, 1, 1>(P, s);
+    return dtype == NMG_F16 ? launch_dense16<__half, 8, 2>(P, s) : launch_dense16<__hip_bfloat16, 8, 2>(P, s);
 }

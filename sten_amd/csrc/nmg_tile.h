@@ -224,6 +224,28 @@ __device__ __forceinline__ void store_partial_tile(const f32x16 (&acc)[FB][TB], 
     }
 }
 
+// The same for the 16 x 16 form: a lane holds token l%16 and outputs 4*(l/16) + 0..3 of every block.
+template <int AB, int TB>
+__device__ __forceinline__ void store_partial_tile16(const f32x4 (&acc)[AB][TB], float *part, int64_t part_ld,
+                                                     int lane, int64_t fw, int64_t tw, int64_t T)
+{
+    const int j = lane & 15, q = lane >> 4;
+#pragma unroll
+    for (int tb = 0; tb < TB; tb++) {
+        const int64_t tok = tw + tb * 16 + j;
+        if (tok >= T) continue;
+#pragma unroll
+        for (int ab = 0; ab < AB; ab++) {
+            float4 v;
+            v.x = acc[ab][tb][0];
+            v.y = acc[ab][tb][1];
+            v.z = acc[ab][tb][2];
+            v.w = acc[ab][tb][3];
+            *(float4 *)(part + tok * part_ld + fw + ab * 16 + q * 4) = v;
+        }
+    }
+}
+
 template <typename T> __global__ __launch_bounds__(256) void splitk_sum_kernel(SplitSum P)
 {
     const int64_t quads = (P.M + 3) / 4;
