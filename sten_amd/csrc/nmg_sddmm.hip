@@ -17,6 +17,9 @@
 // Workgroup: 4 wavefronts, tile 256 positions x 256 lines, each wavefront 128 x 128 (4 x 4
 // accumulator blocks of 32 x 32, 256 accumulator registers).  A K step is 32 tokens; its two
 // operand tiles (2 x 16 KiB) are one stage of a 4-stage LDS ring filled 3 steps ahead.
+// Patterns with m == 4 take sddmm16_kernel below: the same tile and ring around
+// V_MFMA_F32_16X16X32 (8 x 8 accumulator blocks of 16 x 16), whose 4 registers per block are
+// exactly one block of the pattern.
 //
 // Epilogue: the tile is staged in LDS as [line][position] in the output type; thread = line walks
 // the blocks of m positions, looks up the slot of (line, block) in the slot map (the inverse of
@@ -116,11 +119,11 @@ static_assert(SD_LDS <= 160 * 1024, "LDS of a CU");
 static_assert(SD_D < SD_NS, "a stage is refilled only after the barrier that ends its last read");
 static_assert(SD_D * SD_LPW < 64, "vmcnt is a 6-bit counter");
 
-// MODE 8 + n (n = 1, 2, 4): m == 8, the same after an exchange between the two lanes that hold a block.
-// MODE 1 .. 4: m == 4 and n == MODE.  The 4 consecutive positions a lane holds of its line are one
-// block, so the kept values are picked in registers (one byte permute with a per-pattern selector)
-// and stored by the lane itself; the slots of the lane's 64 (line, block) pairs are fetched when the
-// kernel starts and wait in registers through the product.  MODE 0: any n:m, through the staged tile.
+// MODE 8 + n (n = 1, 2, 4): m == 8.  After an exchange between the two lanes that hold a block the
+// 8 consecutive positions of a block lie in one lane, so the kept values are picked in registers
+// (byte permutes with per-pattern selectors) and stored by the lane itself; the slots of the lane's
+// (line, block) pairs are fetched when the kernel starts and wait in registers through the product.
+// MODE 0: any n:m, through the staged tile.  (m == 4 is sddmm16_kernel's.)
 // NT = true: the operands are given with the reduction (tokens) as their fast dim, L^T [G, T] and
 // P^T [S, T] (the weight gradient of torch.mm(W, B): grad_out [R, N] and B [C, N] as they lie in
 // memory).  An operand tile of a K step is then 256 feature rows of 64 bytes; a fragment -- the
@@ -130,6 +133,7 @@ template <typename T, int MODE, bool NT = false>
 __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
 {
     using Mm = SdMma<T>;
+    static_assert(MODE == 0 || MODE == 9 || MODE == 10 || MODE == 12, "the staged tile, or m == 8 in registers");
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -149,35 +153,7 @@ __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
     const int wm = wave >> 1, wn = wave & 1;   // position half / line half of the wavefront
     const int KP = P.KP;
 
-    // ---- MODE 1: the lane's slots.  Accumulator block (x, y), register quad rq: line
-    // l0 + wn*128 + y*32 + l%32, block (p0 + wm*128 + x*32 + rq*8 + (l/32)*4) / 4.
-    uint32_t my_slot[MODE >= 1 ? (MODE <= 4 ? 32 : 16) : 1];   // two slots per register
-    if constexpr (MODE >= 1 && MODE <= 4) {
-        // byte selectors of V_PERM_B32 per pattern: kept halves 0, 1 (and 2, 3) out of the 8 bytes
-        // {positions 0, 1 | positions 2, 3} of a block, from the packed order table
-        uint32_t *s_sel = (uint32_t *)(smem + 256 * SD_PITCH);
-        if (tid < 16) {
-            const uint32_t o = (uint32_t)(P.ord4 >> (8 * (tid & 7)));
-            const int jj = (tid >> 3) * 2;
-            const uint32_t a = (o >> (2 * jj)) & 3, b = (o >> (2 * jj + 2)) & 3;
-            s_sel[tid] = (2 * a) | ((2 * a + 1) << 8) | ((2 * b) << 16) | ((2 * b + 1) << 24);
-        }
-        const int j = lane & 31, h = lane >> 5;
-#pragma unroll
-        for (int y = 0; y < 4; y++) {
-            const int64_t line = min(l0 + wn * 128 + y * 32 + j, P.Gpad - 1);
-#pragma unroll
-            for (int x = 0; x < 4; x++)
-#pragma unroll
-                for (int rp = 0; rp < 2; rp++) {
-                    const int blk0 = min((int)(p0 / 4) + wm * 32 + x * 8 + rp * 4 + h, (int)P.nb - 1);
-                    const int blk1 = min((int)(p0 / 4) + wm * 32 + x * 8 + rp * 4 + 2 + h, (int)P.nb - 1);
-                    my_slot[(y * 4 + x) * 2 + rp] = (uint32_t)(uint16_t)P.slot[blk0 * P.Gpad + line] |
-                                                    ((uint32_t)(uint16_t)P.slot[blk1 * P.Gpad + line] << 16);
-                }
-        }
-    }
-
+    uint32_t my_slot[MODE > 8 ? 16 : 1];   // two slots per register
     if constexpr (MODE > 8) {
         // ---- MODE 8 + n: m == 8.  A block of a line lies in two lanes (positions 0..3 in lane
         // l%32, 4..7 in lane l%32 + 32); after the exchange in the epilogue lane l owns the blocks
@@ -509,74 +485,6 @@ __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
             epilogue(std::false_type{});
         return;
     }
-    if constexpr (MODE >= 1 && MODE <= 4) {
-        // ---- epilogue in registers (D rows = positions 8*(r/4) + 4*(l/32) + r%4 of the block,
-        // column = line l%32: registers rq*4 .. +3 of a lane are one block of its line).  Offsets
-        // into val are 32-bit (the host checks that val is smaller than 4 GiB).
-        constexpr int N = MODE;
-        const uint32_t *s_sel = (const uint32_t *)(smem + 256 * SD_PITCH);
-        const int j = lane & 31, h = lane >> 5;
-        int blk_base = (int)(p0 / 4) + wm * 32 + h;
-        asm volatile("" : "+v"(blk_base));   // computed afresh: nothing is kept in registers through the product for it
-        const uint32_t cg = (uint32_t)P.cg, nb = (uint32_t)P.nb;
-        const uint32_t g1_mask = P.g > 1 ? 0u : ~0u;   // inv_g is 0 for g == 1
-        unsigned char *vbase = (unsigned char *)P.val;
-        auto epilogue = [&](auto interior_tag) {
-            constexpr bool INTERIOR = decltype(interior_tag)::value;   // every line and block of the tile exists
-#pragma unroll
-            for (int y = 0; y < 4; y++) {
-                const uint32_t line = (uint32_t)l0 + wn * 128 + y * 32 + j;
-                const bool line_in = INTERIOR || line < (uint32_t)P.Gpad, line_ok = INTERIOR || line < (uint32_t)P.G;
-                const uint32_t rowbase = ((line / cg) * nb + (uint32_t)blk_base) * cg;
-#pragma unroll
-                for (int x = 0; x < 4; x++) {
-                    // the slots and selectors of the block's four quads first (LDS reads in flight together)
-                    uint32_t sl[4], sel[4], sel2[4];
-#pragma unroll
-                    for (int rq = 0; rq < 4; rq++) {
-                        sl[rq] = min((my_slot[(y * 4 + x) * 2 + (rq >> 1)] >> (16 * (rq & 1))) & 0x7fffu, cg - 1);
-                        const uint32_t pat = __umulhi(sl[rq], P.inv_g) + (sl[rq] & g1_mask);   // slot / g without a branch
-                        if constexpr (N < 4) sel[rq] = s_sel[pat & 7];
-                        if constexpr (N == 3) sel2[rq] = s_sel[8 + (pat & 7)];
-                    }
-#pragma unroll
-                    for (int rq = 0; rq < 4; rq++) {
-                        uint16_t hh[4];
-#pragma unroll
-                        for (int e = 0; e < 4; e++) hh[e] = sd_bits16<T>(sd_from_acc(acc[x][y][rq * 4 + e]));
-                        uint32_t lo = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
-                        uint32_t hi = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
-                        if (!INTERIOR && !line_ok) lo = hi = 0;
-                        if (!INTERIOR && (!line_in || blk_base + x * 8 + rq * 2 >= (int)nb)) continue;
-                        unsigned char *dst =
-                            vbase + (size_t)((rowbase + (uint32_t)(x * 8 + rq * 2) * cg + sl[rq]) * (uint32_t)(2 * N));
-                        if constexpr (N == 4) {
-                            *(uint2 *)dst = uint2{lo, hi};
-                        } else {
-                            const uint32_t out = __builtin_amdgcn_perm(hi, lo, sel[rq]);
-                            if constexpr (N == 1) {
-                                *(uint16_t *)dst = (uint16_t)out;
-                            } else if constexpr (N == 2) {
-                                *(uint32_t *)dst = out;
-                            } else {   // 6-byte entries are 2-byte aligned only
-                                const uint32_t out2 = __builtin_amdgcn_perm(hi, lo, sel2[rq]);
-                                ((uint16_t *)dst)[0] = (uint16_t)out;
-                                ((uint16_t *)dst)[1] = (uint16_t)(out >> 16);
-                                ((uint16_t *)dst)[2] = (uint16_t)out2;
-                            }
-                        }
-                    }
-                    // an accumulator block at a time: its registers are read when it is stored
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
-        };
-        if (l0 + 256 <= P.G && p0 + 256 <= P.nb * 4)
-            epilogue(std::true_type{});
-        else
-            epilogue(std::false_type{});
-        return;
-    }
     asm volatile("s_barrier" ::: "memory");
 
     // ---- epilogue through LDS: stage [line][position] in the output type (D rows = positions
@@ -640,6 +548,340 @@ __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
                 }
             }
         }
+    }
+}
+
+// ------------------------------------------- the same product with V_MFMA_F32_16X16X32
+// The 16 x 16 x 32 form of the instruction sustains 10-17 % more flops under the power limit than
+// the 32 x 32 x 16 form, and a K step of 32 tokens is exactly one of its reduction steps.  Same
+// tile, same ring, same DMA loads and counted waits as sddmm_kernel; what differs:
+//   fragments: lane (kq = l/16, i = l%16) holds feature i of a 16-feature block at tokens
+//     8 kq .. 8 kq + 7 -- two transposing reads (token-major operands) or one 16-byte read
+//     (reduction-contiguous operands).  For the transposing reads the 64-byte granules of a token
+//     row are XOR-swizzled with (t % 4) + 4 * ((t / 8) % 2): the 32 lanes served together cover
+//     tokens t .. t+3 and t+8 .. t+11, which must not share banks.
+//   accumulators: 8 x 8 blocks of 16 positions x 16 lines, 4 registers each; lane (j = l%16,
+//     q = l/16) holds line j and the positions 4q .. 4q+3 of the block -- one block of m = 4.
+//   a K step is two phases (position blocks 0..3, 4..7) of 32 MFMAs, column by column; the line
+//     fragments live in one register set: column y of the second phase frees fragment y, which is
+//     then read for the next step.
+// MODE 1 .. 4: m == 4, n == MODE; the epilogue stays in registers: the kept values of a block are
+// picked with one byte permute (per-pattern selector) and stored by the lane itself; the slots of
+// the lane's 64 (line, block) pairs are fetched when the kernel starts and wait in registers.
+template <typename T> struct SdMma16;
+template <> struct SdMma16<__half> {
+    using F = sd_f16x8;
+    __device__ static f32x4 run(F a, F b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+};
+template <> struct SdMma16<__hip_bfloat16> {
+    using F = sd_bf16x8;
+    __device__ static f32x4 run(F a, F b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+};
+
+template <typename T, int MODE, bool NT = false>
+__global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
+{
+    using Mm = SdMma16<T>;
+    static_assert(MODE >= 1 && MODE <= 4, "m == 4, n == MODE");
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    // workgroup -> tile as in sddmm_kernel
+    int id = blockIdx.x;
+    const int ntiles = P.tiles_p * P.tiles_l;
+    if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
+    constexpr int GH = 4;
+    const int band = id / (GH * P.tiles_l);
+    const int band_h = min(P.tiles_p - band * GH, GH);
+    const int in_band = id - band * GH * P.tiles_l;
+    const int tile_p = band * GH + in_band % band_h, tile_l = in_band / band_h;
+    const int64_t p0 = (int64_t)tile_p * 256, l0 = (int64_t)tile_l * 256;
+    const int wm = wave >> 1, wn = wave & 1;   // position half / line half of the wavefront
+    const int KP = P.KP;
+    const int j16 = lane & 15, kq = lane >> 4;
+
+    // ---- MODE 1..4: the lane's slots.  Accumulator block (x, y): line l0 + wn*128 + 16 y + l%16,
+    // block p0/4 + wm*32 + 4 x + l/16.  Two slots per register (x even in the low half).
+    uint32_t my_slot[32];
+    {
+        uint32_t *s_sel = (uint32_t *)(smem + 256 * SD_PITCH);
+        if (tid < 16) {
+            const uint32_t o = (uint32_t)(P.ord4 >> (8 * (tid & 7)));
+            const int jj = (tid >> 3) * 2;
+            const uint32_t a = (o >> (2 * jj)) & 3, b = (o >> (2 * jj + 2)) & 3;
+            s_sel[tid] = (2 * a) | ((2 * a + 1) << 8) | ((2 * b) << 16) | ((2 * b + 1) << 24);
+        }
+#pragma unroll
+        for (int y = 0; y < 8; y++) {
+            const int64_t line = min(l0 + wn * 128 + y * 16 + j16, P.Gpad - 1);
+#pragma unroll
+            for (int xp = 0; xp < 4; xp++) {
+                const int blk0 = min((int)(p0 / 4) + wm * 32 + (2 * xp) * 4 + kq, (int)P.nb - 1);
+                const int blk1 = min((int)(p0 / 4) + wm * 32 + (2 * xp + 1) * 4 + kq, (int)P.nb - 1);
+                my_slot[y * 4 + xp] = (uint32_t)(uint16_t)P.slot[blk0 * P.Gpad + line] |
+                                      ((uint32_t)(uint16_t)P.slot[blk1 * P.Gpad + line] << 16);
+            }
+        }
+    }
+
+    // ---- DMA sources: as in sddmm_kernel, except for the swizzle of the token-major tiles
+    const bool is_l = wave >= 2;
+    const unsigned char *gsrc = (const unsigned char *)(is_l ? P.lop : P.pop);
+    const int64_t ld = is_l ? P.ldl : P.ldp, ext = is_l ? P.G : P.S, f0 = is_l ? l0 : p0;
+    uint32_t g_off[SD_LPW];
+#pragma unroll
+    for (int i = 0; i < SD_LPW; i++) {
+        if constexpr (NT) {
+            const int row = (wave & 1) * 128 + 16 * i + (lane >> 2);
+            const int piece = (lane & 3) ^ ((row >> 2) & 3);
+            int64_t feat = f0 + row;
+            if (feat > ext - 1) feat = ext - 1;
+            g_off[i] = (uint32_t)(((feat - min(f0, ext - 1)) * ld + piece * 8) * 2);
+        } else {
+            const int tok = (((wave & 1) * 8 + i) << 1) + (lane >> 5);
+            const int chunk = (lane & 31) ^ (((tok & 3) | ((tok >> 1) & 4)) << 2);
+            int64_t feat = f0 + chunk * 8;
+            if (feat > ext - 8) feat = ext - 8;   // columns beyond the extent feed outputs that are never stored
+            g_off[i] = (uint32_t)((tok * ld + feat) * 2);
+        }
+    }
+    const int tok_hi = lane >> 5;
+    const int nt_tok = ((lane & 3) ^ ((lane >> 4) & 3)) * 8;
+    const unsigned char *zero = (const unsigned char *)P.zero;
+    struct Step {
+        const unsigned char *b;
+        uint32_t dst;
+        int rem;
+    };
+    auto step_of = [&](int kp) {
+        const int kc = kp < KP ? kp : KP - 1;
+        Step st;
+        st.b = NT ? gsrc + (min(f0, ext - 1) * ld + (int64_t)kc * SD_KS) * 2 : gsrc + (int64_t)kc * SD_KS * ld * 2;
+        st.dst = (uint32_t)(uintptr_t)(lds_ptr_t)(smem + (kp & (SD_NS - 1)) * SD_STAGE + (is_l ? SD_OP : 0) +
+                                                  (wave & 1) * 8 * 1024);
+        st.rem = (int)min((int64_t)SD_KS, P.T - (int64_t)kc * SD_KS);
+        return st;
+    };
+    auto issue_one = [&](const Step &st, int i, auto tail_tag) {
+        if constexpr (decltype(tail_tag)::value) {
+            const int tok = NT ? nt_tok : (((wave & 1) * 8 + i) << 1) + tok_hi;
+            const unsigned char *src = tok < st.rem ? st.b + g_off[i] : zero;
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                         :: "v"(src), "s"(st.dst + i * 1024) : "memory");
+        } else {
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :: "v"(g_off[i]), "s"(st.b), "s"(st.dst + i * 1024) : "memory");
+        }
+    };
+
+    // ---- fragment addresses.  Token-major: lane (kq, i) of a transposing read supplies the 8 bytes
+    // at token 8 kq + 4 r + i/4, features 4 (i%4) .. +3 of the block, and receives feature i at
+    // tokens 8 kq + 4 r + 0..3.  Feature block f of an operand tile lies in granule f/2 (^ the
+    // swizzle of the token), half f%2.
+    const int tsw = (j16 >> 2) | ((kq & 1) << 2);
+    const int tn_base = (8 * kq + (j16 >> 2)) * 512 + (j16 & 3) * 8;
+    int fa_off[4], fb_off[4];   // per pair of feature blocks of the wavefront
+#pragma unroll
+    for (int f = 0; f < 4; f++) {
+        if constexpr (NT) {
+            // lane (kq, i) reads the 16 bytes of feature row 16 f' + i, piece kq ^ (row/4)%4
+            fa_off[f] = (wm * 128 + f * 32 + j16) * 64 + ((kq ^ ((j16 >> 2) & 3)) << 4);
+            fb_off[f] = (wn * 128 + f * 32 + j16) * 64 + ((kq ^ ((j16 >> 2) & 3)) << 4) + SD_OP;
+        } else {
+            fa_off[f] = tn_base + (((wm * 4 + f) ^ tsw) << 6);
+            fb_off[f] = tn_base + (((wn * 4 + f) ^ tsw) << 6) + SD_OP;
+        }
+    }
+    struct Frag {
+        sd_i16x4 h[2];
+    };
+    Frag fa[2][4], fb[8];
+    // half 0 / 1 of fragment f (0..7) of the position side (is_a) or the line side
+    auto read_half = [&](Frag &d, const unsigned char *stage, bool is_a, int f, int r) {
+        const int off = (is_a ? fa_off[f >> 1] : fb_off[f >> 1]);
+        if constexpr (NT) {
+            if (r == 0) {
+                union {
+                    u32x4 u;
+                    sd_i16x4 h[2];
+                } c;
+                c.u = *(const u32x4 *)(stage + off + (f & 1) * 16 * 64);
+                d.h[0] = c.h[0];
+                d.h[1] = c.h[1];
+            }
+        } else {
+            d.h[r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((sd_lds_i16x4)(stage + off + (f & 1) * 32 + r * 4 * 512));
+        }
+    };
+    constexpr int RPF = NT ? 1 : 2;   // LDS reads per fragment
+
+    f32x4 acc[8][8];   // [position block][line block]
+#pragma unroll
+    for (int x = 0; x < 8; x++)
+#pragma unroll
+        for (int y = 0; y < 8; y++) acc[x][y] = f32x4{0.f, 0.f, 0.f, 0.f};
+    auto pin_acc = [&]() {
+#pragma unroll
+        for (int x = 0; x < 8; x++)
+#pragma unroll
+            for (int y = 0; y < 8; y++) asm volatile("" : "+a"(acc[x][y]));
+    };
+    pin_acc();
+    auto mma = [&](const Frag &a, const Frag &b, int x, int y) {
+        union {
+            sd_i16x4 h[2];
+            typename Mm::F v;
+        } ca, cb;
+        ca.h[0] = a.h[0];
+        ca.h[1] = a.h[1];
+        cb.h[0] = b.h[0];
+        cb.h[1] = b.h[1];
+        acc[x][y] = Mm::run(ca.v, cb.v, acc[x][y]);
+    };
+
+    // The ring: as in sddmm_kernel (SD_LPW loads per wavefront and K step, SD_D steps ahead; the
+    // counted wait of step kp means "my share of step kp+1 has landed", the barrier "everybody's";
+    // stage kp % SD_NS is read for the last time before that barrier and refilled during step kp+1).
+#pragma unroll
+    for (int s0 = 0; s0 < SD_D; s0++) {
+        const Step st = step_of(s0);
+#pragma unroll
+        for (int i = 0; i < SD_LPW; i++) issue_one(st, i, std::true_type{});
+    }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SD_D - 1) * SD_LPW) : "memory");
+    asm volatile("s_barrier" ::: "memory");
+#pragma unroll
+    for (int f = 0; f < 4; f++)
+#pragma unroll
+        for (int r = 0; r < RPF; r++) read_half(fa[0][f], smem, true, f, r);
+#pragma unroll
+    for (int f = 0; f < 8; f++)
+#pragma unroll
+        for (int r = 0; r < RPF; r++) read_half(fb[f], smem, false, f, r);
+
+    auto k_step = [&](int kp, auto tail_tag) {
+        const unsigned char *cur = smem + (kp & (SD_NS - 1)) * SD_STAGE;
+        const unsigned char *nxt = smem + ((kp + 1) & (SD_NS - 1)) * SD_STAGE;
+        const Step st = step_of(kp + SD_D);
+        // phase 0: position blocks 0..3, column by column; behind the MFMAs the position
+        // fragments 4..7 of this step and the DMA loads of step kp + SD_D, alternating
+        constexpr int NA = 4 * RPF;   // reads of four position fragments
+#pragma unroll
+        for (int i = 0; i < 32; i++) {
+            mma(fa[0][i & 3], fb[i >> 2], i & 3, i >> 2);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i % 2 == 0) {
+                const int k = i / 2;   // 0..15: read, load, read, load ...
+                if (k % 2 == 0 && k / 2 < NA)
+                    read_half(fa[1][(k / 2) / RPF], cur, true, 4 + (k / 2) / RPF, (k / 2) % RPF);
+                else if (k % 2 == 1 && k / 2 < SD_LPW)
+                    issue_one(st, k / 2, tail_tag);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // wait for step kp+1 and meet the other wavefronts (the reads of stage kp are complete)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SD_D - 1) * SD_LPW) : "memory");
+        asm volatile("s_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        // phase 1: position blocks 4..7; behind the MFMAs first the position fragments 0..3 of the
+        // next step, then its line fragments, fragment y once column y is done
+#pragma unroll
+        for (int i = 0; i < 32; i++) {
+            mma(fa[1][i & 3], fb[i >> 2], 4 + (i & 3), i >> 2);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i < NA) {
+                read_half(fa[0][i / RPF], nxt, true, i / RPF, i % RPF);
+            } else {
+                // line fragment read number k = i - NA, not before column k / RPF is done
+#pragma unroll
+                for (int k = 0; k < 8 * RPF; k++) {
+                    const int at = NA + k > 4 * (k / RPF) + 3 ? NA + k : 4 * (k / RPF) + 3;
+                    if (at == i) read_half(fb[k / RPF], nxt, false, k / RPF, k % RPF);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // reads whose slot lies beyond the last MFMA
+#pragma unroll
+        for (int k = 0; k < 8 * RPF; k++) {
+            const int at = NA + k > 4 * (k / RPF) + 3 ? NA + k : 4 * (k / RPF) + 3;
+            if (at >= 32) read_half(fb[k / RPF], nxt, false, k / RPF, k % RPF);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    const int kp_tail = max(0, KP - 1 - SD_D);
+    for (int kp = 0; kp < kp_tail; kp++) k_step(kp, std::false_type{});
+    for (int kp = kp_tail; kp < KP; kp++) k_step(kp, std::true_type{});
+    pin_acc();
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+
+    {
+        // ---- epilogue in registers: the 4 registers of an accumulator block are one block of the
+        // lane's line.  Offsets into val are 32-bit (the host checks that val is smaller than 4 GiB).
+        constexpr int N = MODE;
+        const uint32_t *s_sel = (const uint32_t *)(smem + 256 * SD_PITCH);
+        int blk_base = (int)(p0 / 4) + wm * 32 + kq;
+        asm volatile("" : "+v"(blk_base));
+        const uint32_t cg = (uint32_t)P.cg, nb = (uint32_t)P.nb;
+        const uint32_t g1_mask = P.g > 1 ? 0u : ~0u;   // inv_g is 0 for g == 1
+        unsigned char *vbase = (unsigned char *)P.val;
+        asm volatile("s_barrier" ::: "memory");   // the selector table was written by other wavefronts
+        auto epilogue = [&](auto interior_tag) {
+            constexpr bool INTERIOR = decltype(interior_tag)::value;
+#pragma unroll
+            for (int y = 0; y < 8; y++) {
+                const uint32_t line = (uint32_t)l0 + wn * 128 + y * 16 + j16;
+                const bool line_in = INTERIOR || line < (uint32_t)P.Gpad, line_ok = INTERIOR || line < (uint32_t)P.G;
+                const uint32_t rowbase = ((line / cg) * nb + (uint32_t)blk_base) * cg;
+#pragma unroll
+                for (int xq = 0; xq < 2; xq++) {
+                    uint32_t sl[4], sel[4], sel2[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int x = xq * 4 + e;
+                        sl[e] = min((my_slot[y * 4 + (x >> 1)] >> (16 * (x & 1))) & 0x7fffu, cg - 1);
+                        const uint32_t pat = __umulhi(sl[e], P.inv_g) + (sl[e] & g1_mask);   // slot / g without a branch
+                        if constexpr (N < 4) sel[e] = s_sel[pat & 7];
+                        if constexpr (N == 3) sel2[e] = s_sel[8 + (pat & 7)];
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int x = xq * 4 + e;
+                        uint16_t hh[4];
+#pragma unroll
+                        for (int r = 0; r < 4; r++) hh[r] = sd_bits16<T>(sd_from_acc(acc[x][y][r]));
+                        uint32_t lo = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
+                        uint32_t hi = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
+                        if (!INTERIOR && !line_ok) lo = hi = 0;
+                        if (!INTERIOR && (!line_in || blk_base + x * 4 >= (int)nb)) continue;
+                        unsigned char *dst =
+                            vbase + (size_t)((rowbase + (uint32_t)(x * 4) * cg + sl[e]) * (uint32_t)(2 * N));
+                        if constexpr (N == 4) {
+                            *(uint2 *)dst = uint2{lo, hi};
+                        } else {
+                            const uint32_t out = __builtin_amdgcn_perm(hi, lo, sel[e]);
+                            if constexpr (N == 1) {
+                                *(uint16_t *)dst = (uint16_t)out;
+                            } else if constexpr (N == 2) {
+                                *(uint32_t *)dst = out;
+                            } else {   // 6-byte entries are 2-byte aligned only
+                                const uint32_t out2 = __builtin_amdgcn_perm(hi, lo, sel2[e]);
+                                ((uint16_t *)dst)[0] = (uint16_t)out;
+                                ((uint16_t *)dst)[1] = (uint16_t)(out >> 16);
+                                ((uint16_t *)dst)[2] = (uint16_t)out2;
+                            }
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        };
+        if (l0 + 256 <= P.G && p0 + 256 <= P.nb * 4)
+            epilogue(std::true_type{});
+        else
+            epilogue(std::false_type{});
     }
 }
 
@@ -735,7 +977,7 @@ static int sddmm_impl(bool nt, const void *d_lines, int64_t ld_lines, const void
     auto launch_t = [&](auto tag) -> int {
         using T = decltype(tag);
         if (nt) {   // reduction-contiguous operands: 2:4 in registers, every other pattern through the staged tile
-            if (in_regs && n == 2 && S % 4 == 0) return launch(sddmm_kernel<T, 2, true>);   // (no padded positions)
+            if (in_regs && n == 2 && S % 4 == 0) return launch(sddmm16_kernel<T, 2, true>);   // (no padded positions)
             return launch(sddmm_kernel<T, 0, true>);
         }
         if (in_regs8) {
@@ -745,10 +987,10 @@ static int sddmm_impl(bool nt, const void *d_lines, int64_t ld_lines, const void
         }
         if (!in_regs) return launch(sddmm_kernel<T, 0>);
         switch (n) {
-        case 1: return launch(sddmm_kernel<T, 1>);
-        case 2: return launch(sddmm_kernel<T, 2>);
-        case 3: return launch(sddmm_kernel<T, 3>);
-        default: return launch(sddmm_kernel<T, 4>);
+        case 1: return launch(sddmm16_kernel<T, 1>);
+        case 2: return launch(sddmm16_kernel<T, 2>);
+        case 3: return launch(sddmm16_kernel<T, 3>);
+        default: return launch(sddmm16_kernel<T, 4>);
         }
     };
     const int rc = dtype == NMG_F16 ? launch_t(__half{}) : launch_t(__hip_bfloat16{});
