@@ -17,9 +17,9 @@
 // Workgroup: 4 wavefronts, tile 256 positions x 256 lines, each wavefront 128 x 128 (4 x 4
 // accumulator blocks of 32 x 32, 256 accumulator registers).  A K step is 32 tokens; its two
 // operand tiles (2 x 16 KiB) are one stage of a 4-stage LDS ring filled 3 steps ahead.
-// Patterns with m == 4 take sddmm16_kernel below: the same tile and ring around
-// V_MFMA_F32_16X16X32 (8 x 8 accumulator blocks of 16 x 16), whose 4 registers per block are
-// exactly one block of the pattern.
+// Patterns with m == 4 (and m == 8 with n = 1, 2, 4) take sddmm16_kernel below: the same tile and
+// ring around V_MFMA_F32_16X16X32 (8 x 8 accumulator blocks of 16 x 16), whose 4 registers per
+// block are exactly one block of m = 4, or one half of a block of m = 8.
 //
 // Epilogue: the tile is staged in LDS as [line][position] in the output type; thread = line walks
 // the blocks of m positions, looks up the slot of (line, block) in the slot map (the inverse of
@@ -119,11 +119,8 @@ static_assert(SD_LDS <= 160 * 1024, "LDS of a CU");
 static_assert(SD_D < SD_NS, "a stage is refilled only after the barrier that ends its last read");
 static_assert(SD_D * SD_LPW < 64, "vmcnt is a 6-bit counter");
 
-// MODE 8 + n (n = 1, 2, 4): m == 8.  After an exchange between the two lanes that hold a block the
-// 8 consecutive positions of a block lie in one lane, so the kept values are picked in registers
-// (byte permutes with per-pattern selectors) and stored by the lane itself; the slots of the lane's
-// (line, block) pairs are fetched when the kernel starts and wait in registers through the product.
-// MODE 0: any n:m, through the staged tile.  (m == 4 is sddmm16_kernel's.)
+// MODE 0: any n:m, through the staged tile.  (m == 4 and m == 8 with n = 1, 2, 4 take
+// sddmm16_kernel, whose epilogue stays in registers.)
 // NT = true: the operands are given with the reduction (tokens) as their fast dim, L^T [G, T] and
 // P^T [S, T] (the weight gradient of torch.mm(W, B): grad_out [R, N] and B [C, N] as they lie in
 // memory).  An operand tile of a K step is then 256 feature rows of 64 bytes; a fragment -- the
@@ -133,7 +130,7 @@ template <typename T, int MODE, bool NT = false>
 __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
 {
     using Mm = SdMma<T>;
-    static_assert(MODE == 0 || MODE == 9 || MODE == 10 || MODE == 12, "the staged tile, or m == 8 in registers");
+    static_assert(MODE == 0, "the staged tile (the epilogues in registers are sddmm16_kernel's)");
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -152,44 +149,6 @@ __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
     const int64_t p0 = (int64_t)tile_p * 256, l0 = (int64_t)tile_l * 256;
     const int wm = wave >> 1, wn = wave & 1;   // position half / line half of the wavefront
     const int KP = P.KP;
-
-    uint32_t my_slot[MODE > 8 ? 16 : 1];   // two slots per register
-    if constexpr (MODE > 8) {
-        // ---- MODE 8 + n: m == 8.  A block of a line lies in two lanes (positions 0..3 in lane
-        // l%32, 4..7 in lane l%32 + 32); after the exchange in the epilogue lane l owns the blocks
-        // (p0 + wm*128 + x*32) / 8 + 2k + l/32, k = 0, 1, of its line: their slots, k = 1 in the
-        // high half.  Selector table: per pattern and output word two V_PERM_B32 selectors, one for
-        // the positions 0..3, one for 4..7 (bytes that come from the other half select zero).
-        constexpr int N = MODE - 8, ND = (N + 1) / 2;
-        uint32_t *s_sel = (uint32_t *)(smem + 256 * SD_PITCH);
-        for (int e = tid; e < P.order_bytes / N * ND; e += 256) {
-            const int pat = e / ND, w = e - pat * ND;
-            uint32_t sa = 0x0c0c0c0cu, sb = 0x0c0c0c0cu;
-#pragma unroll
-            for (int jj = 0; jj < 2; jj++) {
-                const int j = 2 * w + jj;
-                if (j >= N) break;
-                const uint32_t q = (uint32_t)P.order[pat * N + j] & 7u;
-                const uint32_t two = (2 * (q & 3)) | ((2 * (q & 3) + 1) << 8);
-                if (q < 4) sa = (sa & ~(0xffffu << (16 * jj))) | (two << (16 * jj));
-                else sb = (sb & ~(0xffffu << (16 * jj))) | (two << (16 * jj));
-            }
-            s_sel[2 * e] = sa;
-            s_sel[2 * e + 1] = sb;
-        }
-        const int j = lane & 31, h = lane >> 5;
-#pragma unroll
-        for (int y = 0; y < 4; y++) {
-            const int64_t line = min(l0 + wn * 128 + y * 32 + j, P.Gpad - 1);
-#pragma unroll
-            for (int x = 0; x < 4; x++) {
-                const int blk0 = min((int)(p0 / 8) + wm * 16 + x * 4 + h, (int)P.nb - 1);
-                const int blk1 = min((int)(p0 / 8) + wm * 16 + x * 4 + 2 + h, (int)P.nb - 1);
-                my_slot[y * 4 + x] = (uint32_t)(uint16_t)P.slot[blk0 * P.Gpad + line] |
-                                     ((uint32_t)(uint16_t)P.slot[blk1 * P.Gpad + line] << 16);
-            }
-        }
-    }
 
     // ---- DMA sources.  Wavefronts 0, 1 fetch the position tile, 2, 3 the line tile; load i of a
     // wavefront fills token rows 2r, 2r+1 (r = (wave & 1) * 8 + i) of its operand tile: 1 KiB of
@@ -405,86 +364,6 @@ __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
     uint16_t *val = (uint16_t *)P.val;
     const int n = P.n, m = P.m;
 
-    if constexpr (MODE > 8) {
-        // ---- epilogue in registers, m == 8 (D rows = positions 8*(r/4) + 4*(l/32) + r%4 of the
-        // 32-position block: register quad rq of lanes l%32 and l%32 + 32 is block rq, low and
-        // high half).  The quads 2k and 2k+1 are rounded, packed and exchanged between the two
-        // lanes (V_PERMLANE32_SWAP), after which the low lane holds block 2k and the high lane
-        // block 2k+1 as four words; the kept values are picked with two byte permutes per word.
-        constexpr int N = MODE - 8, ND = (N + 1) / 2;
-        const uint32_t *s_sel = (const uint32_t *)(smem + 256 * SD_PITCH);
-        asm volatile("s_barrier" ::: "memory");   // the selector table was written by other wavefronts
-        const int j = lane & 31, h = lane >> 5;
-        int blk_base = (int)(p0 / 8) + wm * 16 + h;
-        asm volatile("" : "+v"(blk_base));
-        const uint32_t cg = (uint32_t)P.cg, nb = (uint32_t)P.nb;
-        const uint32_t g1_mask = P.g > 1 ? 0u : ~0u;
-        unsigned char *vbase = (unsigned char *)P.val;
-        auto epilogue = [&](auto interior_tag) {
-            constexpr bool INTERIOR = decltype(interior_tag)::value;
-#pragma unroll
-            for (int y = 0; y < 4; y++) {
-                const uint32_t line = (uint32_t)l0 + wn * 128 + y * 32 + j;
-                const bool line_in = INTERIOR || line < (uint32_t)P.Gpad, line_ok = INTERIOR || line < (uint32_t)P.G;
-                const uint32_t rowbase = ((line / cg) * nb + (uint32_t)blk_base) * cg;
-#pragma unroll
-                for (int x = 0; x < 4; x++) {
-#pragma unroll
-                    for (int k = 0; k < 2; k++) {
-                        const uint32_t sl = min((my_slot[y * 4 + x] >> (16 * k)) & 0x7fffu, cg - 1);
-                        const uint32_t pat = __umulhi(sl, P.inv_g) + (sl & g1_mask);
-                        uint32_t sel[ND][2];
-#pragma unroll
-                        for (int w = 0; w < ND; w++) {
-                            sel[w][0] = s_sel[(pat * ND + w) * 2];
-                            sel[w][1] = s_sel[(pat * ND + w) * 2 + 1];
-                        }
-                        uint32_t d[4];   // before the exchange: quad 2k words 0, 1, quad 2k+1 words 0, 1
-#pragma unroll
-                        for (int qd = 0; qd < 2; qd++)
-#pragma unroll
-                            for (int w = 0; w < 2; w++) {
-                                const uint16_t lo16 = sd_bits16<T>(sd_from_acc(acc[x][y][(2 * k + qd) * 4 + 2 * w]));
-                                const uint16_t hi16 = sd_bits16<T>(sd_from_acc(acc[x][y][(2 * k + qd) * 4 + 2 * w + 1]));
-                                d[qd * 2 + w] = (uint32_t)lo16 | ((uint32_t)hi16 << 16);
-                            }
-                        // words of (quad 2k, quad 2k+1): low lanes keep quad 2k and receive its
-                        // high half from the lane 32 up, which receives the low half of quad 2k+1
-                        uint32_t blkw[4];   // positions 0,1 | 2,3 | 4,5 | 6,7 of the lane's block
-#pragma unroll
-                        for (int w = 0; w < 2; w++) {
-                            const auto sw = __builtin_amdgcn_permlane32_swap(d[w], d[2 + w], false, false);
-                            blkw[w] = sw[0];
-                            blkw[2 + w] = sw[1];
-                        }
-                        if (!INTERIOR && !line_ok) blkw[0] = blkw[1] = blkw[2] = blkw[3] = 0;
-                        if (!INTERIOR && (!line_in || blk_base + x * 4 + 2 * k >= (int)nb)) continue;
-                        unsigned char *dst =
-                            vbase + (size_t)((rowbase + (uint32_t)(x * 4 + 2 * k) * cg + sl) * (uint32_t)(2 * N));
-                        uint32_t out[ND];
-#pragma unroll
-                        for (int w = 0; w < ND; w++)
-                            out[w] = __builtin_amdgcn_perm(blkw[1], blkw[0], sel[w][0]) |
-                                     __builtin_amdgcn_perm(blkw[3], blkw[2], sel[w][1]);
-                        if constexpr (N == 1) {
-                            *(uint16_t *)dst = (uint16_t)out[0];
-                        } else if constexpr (N == 2) {
-                            *(uint32_t *)dst = out[0];
-                        } else {
-                            static_assert(N == 4, "m == 8 is built for n = 1, 2, 4");
-                            *(uint2 *)dst = uint2{out[0], out[1]};
-                        }
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
-        };
-        if (l0 + 256 <= P.G && p0 + 256 <= P.nb * 8)
-            epilogue(std::true_type{});
-        else
-            epilogue(std::false_type{});
-        return;
-    }
     asm volatile("s_barrier" ::: "memory");
 
     // ---- epilogue through LDS: stage [line][position] in the output type (D rows = positions
@@ -571,6 +450,8 @@ __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
 // MODE 1 .. 4: m == 4, n == MODE; the epilogue stays in registers: the kept values of a block are
 // picked with one byte permute (per-pattern selector) and stored by the lane itself; the slots of
 // the lane's 64 (line, block) pairs are fetched when the kernel starts and wait in registers.
+// MODE 8 + n (n = 1, 2, 4): m == 8; the two lanes that hold the halves of a block exchange them
+// first (V_PERMLANE16_SWAP), then two byte permutes per output word.
 template <typename T> struct SdMma16;
 template <> struct SdMma16<__half> {
     using F = sd_f16x8;
@@ -585,7 +466,7 @@ template <typename T, int MODE, bool NT = false>
 __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
 {
     using Mm = SdMma16<T>;
-    static_assert(MODE >= 1 && MODE <= 4, "m == 4, n == MODE");
+    static_assert((MODE >= 1 && MODE <= 4) || MODE == 9 || MODE == 10 || MODE == 12, "m == 4, n == MODE; m == 8, n == MODE - 8");
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -604,10 +485,13 @@ __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
     const int KP = P.KP;
     const int j16 = lane & 15, kq = lane >> 4;
 
-    // ---- MODE 1..4: the lane's slots.  Accumulator block (x, y): line l0 + wn*128 + 16 y + l%16,
-    // block p0/4 + wm*32 + 4 x + l/16.  Two slots per register (x even in the low half).
-    uint32_t my_slot[32];
-    {
+    // ---- the lane's slots, two per register.  MODE 1..4: accumulator block (x, y) is line
+    // l0 + wn*128 + 16 y + l%16, block p0/4 + wm*32 + 4 x + l/16 (x even in the low half).
+    // MODE 8 + n: a block of 8 positions lies in the lanes q = l/16 even (positions 0..3) and odd
+    // (4..7) of one accumulator block; after the exchange in the epilogue a lane owns, per pair of
+    // position blocks xp, block p0/8 + wm*16 + 4 xp + 2 (q%2) + q/2 of its line (xp even in the low half).
+    uint32_t my_slot[MODE <= 4 ? 32 : 16];
+    if constexpr (MODE <= 4) {
         uint32_t *s_sel = (uint32_t *)(smem + 256 * SD_PITCH);
         if (tid < 16) {
             const uint32_t o = (uint32_t)(P.ord4 >> (8 * (tid & 7)));
@@ -623,6 +507,38 @@ __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
                 const int blk0 = min((int)(p0 / 4) + wm * 32 + (2 * xp) * 4 + kq, (int)P.nb - 1);
                 const int blk1 = min((int)(p0 / 4) + wm * 32 + (2 * xp + 1) * 4 + kq, (int)P.nb - 1);
                 my_slot[y * 4 + xp] = (uint32_t)(uint16_t)P.slot[blk0 * P.Gpad + line] |
+                                      ((uint32_t)(uint16_t)P.slot[blk1 * P.Gpad + line] << 16);
+            }
+        }
+    } else {
+        // selector table: per pattern and output word two V_PERM_B32 selectors, one for the
+        // positions 0..3, one for 4..7 (bytes that come from the other half select zero)
+        constexpr int N = MODE - 8, ND = (N + 1) / 2;
+        uint32_t *s_sel = (uint32_t *)(smem + 256 * SD_PITCH);
+        for (int e = tid; e < P.order_bytes / N * ND; e += 256) {
+            const int pat = e / ND, w = e - pat * ND;
+            uint32_t sa = 0x0c0c0c0cu, sb = 0x0c0c0c0cu;
+#pragma unroll
+            for (int jj = 0; jj < 2; jj++) {
+                const int j = 2 * w + jj;
+                if (j >= N) break;
+                const uint32_t q = (uint32_t)P.order[pat * N + j] & 7u;
+                const uint32_t two = (2 * (q & 3)) | ((2 * (q & 3) + 1) << 8);
+                if (q < 4) sa = (sa & ~(0xffffu << (16 * jj))) | (two << (16 * jj));
+                else sb = (sb & ~(0xffffu << (16 * jj))) | (two << (16 * jj));
+            }
+            s_sel[2 * e] = sa;
+            s_sel[2 * e + 1] = sb;
+        }
+        const int own = 2 * (kq & 1) + (kq >> 1);
+#pragma unroll
+        for (int y = 0; y < 8; y++) {
+            const int64_t line = min(l0 + wn * 128 + y * 16 + j16, P.Gpad - 1);
+#pragma unroll
+            for (int xq = 0; xq < 2; xq++) {
+                const int blk0 = min((int)(p0 / 8) + wm * 16 + 4 * (2 * xq) + own, (int)P.nb - 1);
+                const int blk1 = min((int)(p0 / 8) + wm * 16 + 4 * (2 * xq + 1) + own, (int)P.nb - 1);
+                my_slot[y * 2 + xq] = (uint32_t)(uint16_t)P.slot[blk0 * P.Gpad + line] |
                                       ((uint32_t)(uint16_t)P.slot[blk1 * P.Gpad + line] << 16);
             }
         }
@@ -820,7 +736,79 @@ __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
     pin_acc();
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 
-    {
+    if constexpr (MODE > 8) {
+        // ---- epilogue in registers, m == 8.  The lanes q even / odd round and pack their halves of
+        // the blocks in the accumulator blocks 2 xp and 2 xp + 1 and exchange them
+        // (V_PERMLANE16_SWAP: odd rows of 16 lanes of the first operand <-> even rows of the second),
+        // after which each owns one whole block as four words; the kept values are picked with two
+        // byte permutes per output word.
+        constexpr int N = MODE - 8, ND = (N + 1) / 2;
+        const uint32_t *s_sel = (const uint32_t *)(smem + 256 * SD_PITCH);
+        asm volatile("s_barrier" ::: "memory");   // the selector table was written by other wavefronts
+        int blk_base = (int)(p0 / 8) + wm * 16 + 2 * (kq & 1) + (kq >> 1);
+        asm volatile("" : "+v"(blk_base));
+        const uint32_t cg = (uint32_t)P.cg, nb = (uint32_t)P.nb;
+        const uint32_t g1_mask = P.g > 1 ? 0u : ~0u;
+        unsigned char *vbase = (unsigned char *)P.val;
+        auto epilogue = [&](auto interior_tag) {
+            constexpr bool INTERIOR = decltype(interior_tag)::value;
+#pragma unroll
+            for (int y = 0; y < 8; y++) {
+                const uint32_t line = (uint32_t)l0 + wn * 128 + y * 16 + j16;
+                const bool line_in = INTERIOR || line < (uint32_t)P.Gpad, line_ok = INTERIOR || line < (uint32_t)P.G;
+                const uint32_t rowbase = ((line / cg) * nb + (uint32_t)blk_base) * cg;
+#pragma unroll
+                for (int xp = 0; xp < 4; xp++) {
+                    const uint32_t sl = min((my_slot[y * 2 + (xp >> 1)] >> (16 * (xp & 1))) & 0x7fffu, cg - 1);
+                    const uint32_t pat = __umulhi(sl, P.inv_g) + (sl & g1_mask);
+                    uint32_t sel[ND][2];
+#pragma unroll
+                    for (int w = 0; w < ND; w++) {
+                        sel[w][0] = s_sel[(pat * ND + w) * 2];
+                        sel[w][1] = s_sel[(pat * ND + w) * 2 + 1];
+                    }
+                    uint32_t d[4];   // before the exchange: block 2 xp words 0, 1, block 2 xp + 1 words 0, 1
+#pragma unroll
+                    for (int qd = 0; qd < 2; qd++)
+#pragma unroll
+                        for (int w = 0; w < 2; w++) {
+                            const uint16_t lo16 = sd_bits16<T>(sd_from_acc(acc[2 * xp + qd][y][2 * w]));
+                            const uint16_t hi16 = sd_bits16<T>(sd_from_acc(acc[2 * xp + qd][y][2 * w + 1]));
+                            d[qd * 2 + w] = (uint32_t)lo16 | ((uint32_t)hi16 << 16);
+                        }
+                    uint32_t blkw[4];   // positions 0,1 | 2,3 | 4,5 | 6,7 of the lane's block
+#pragma unroll
+                    for (int w = 0; w < 2; w++) {
+                        const auto sw = __builtin_amdgcn_permlane16_swap(d[w], d[2 + w], false, false);
+                        blkw[w] = sw[0];
+                        blkw[2 + w] = sw[1];
+                    }
+                    if (!INTERIOR && !line_ok) blkw[0] = blkw[1] = blkw[2] = blkw[3] = 0;
+                    if (!INTERIOR && (!line_in || blk_base + xp * 4 >= (int)nb)) continue;
+                    unsigned char *dst =
+                        vbase + (size_t)((rowbase + (uint32_t)(xp * 4) * cg + sl) * (uint32_t)(2 * N));
+                    uint32_t out[ND];
+#pragma unroll
+                    for (int w = 0; w < ND; w++)
+                        out[w] = __builtin_amdgcn_perm(blkw[1], blkw[0], sel[w][0]) |
+                                 __builtin_amdgcn_perm(blkw[3], blkw[2], sel[w][1]);
+                    if constexpr (N == 1) {
+                        *(uint16_t *)dst = (uint16_t)out[0];
+                    } else if constexpr (N == 2) {
+                        *(uint32_t *)dst = out[0];
+                    } else {
+                        static_assert(N == 4, "m == 8 is built for n = 1, 2, 4");
+                        *(uint2 *)dst = uint2{out[0], out[1]};
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        };
+        if (l0 + 256 <= P.G && p0 + 256 <= P.nb * 8)
+            epilogue(std::true_type{});
+        else
+            epilogue(std::false_type{});
+    } else {
         // ---- epilogue in registers: the 4 registers of an accumulator block are one block of the
         // lane's line.  Offsets into val are 32-bit (the host checks that val is smaller than 4 GiB).
         constexpr int N = MODE;
@@ -984,9 +972,9 @@ static int sddmm_impl(bool nt, const void *d_lines, int64_t ld_lines, const void
             return launch(sddmm_kernel<T, 0, true>);
         }
         if (in_regs8) {
-            if (n == 1) return launch(sddmm_kernel<T, 9>);
-            if (n == 2) return launch(sddmm_kernel<T, 10>);
-            return launch(sddmm_kernel<T, 12>);
+            if (n == 1) return launch(sddmm16_kernel<T, 9>);
+            if (n == 2) return launch(sddmm16_kernel<T, 10>);
+            return launch(sddmm16_kernel<T, 12>);
         }
         if (!in_regs) return launch(sddmm_kernel<T, 0>);
         switch (n) {
