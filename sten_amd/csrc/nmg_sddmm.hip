@@ -10,21 +10,22 @@
 // Both operands have the reduction (tokens) as their slow dim, the opposite of what the matrix
 // cores want (a lane holds 8 consecutive reduction positions of one row).  The transposition is
 // done by the LDS transpose read of gfx950, DS_READ_B64_TR_B16: token-major tiles go global ->
-// LDS by DMA (global_load_lds, 16 bytes per lane), and a fragment of V_MFMA_F32_32X32X16 is two
+// LDS by DMA (global_load_lds, 16 bytes per lane), and a fragment of V_MFMA_F32_16X16X32 is two
 // such reads.  Measured lane layout of the instruction: in every group of 16 lanes, lane i
 // receives as element j the 16-bit element (i % 4) of the 8 bytes addressed by lane 4j + i/4.
 //
-// Workgroup: 4 wavefronts, tile 256 positions x 256 lines, each wavefront 128 x 128 (4 x 4
-// accumulator blocks of 32 x 32, 256 accumulator registers).  A K step is 32 tokens; its two
-// operand tiles (2 x 16 KiB) are one stage of a 4-stage LDS ring filled 3 steps ahead.
-// Patterns with m == 4 (and m == 8 with n = 1, 2, 4) take sddmm16_kernel below: the same tile and
-// ring around V_MFMA_F32_16X16X32 (8 x 8 accumulator blocks of 16 x 16), whose 4 registers per
-// block are exactly one block of m = 4, or one half of a block of m = 8.
+// Workgroup: 4 wavefronts, tile 256 positions x 256 lines, each wavefront 128 x 128 (8 x 8
+// accumulator blocks of 16 x 16, 256 accumulator registers).  A K step is 32 tokens -- one
+// reduction step of the instruction; its two operand tiles (2 x 16 KiB) are one stage of a
+// 4-stage LDS ring filled 3 steps ahead.
 //
-// Epilogue: the tile is staged in LDS as [line][position] in the output type; thread = line walks
-// the blocks of m positions, looks up the slot of (line, block) in the slot map (the inverse of
-// `idx`, built once per pattern by nmg_slotmap), derives the pattern from the slot and writes the
-// n kept values of the block to their place in `val`.
+// Epilogue: the four registers a lane holds of an accumulator block are four consecutive
+// positions of one line -- one block of m = 4, half a block of m = 8 -- so for those patterns
+// the kept values are picked in registers and stored by the lane itself.  Every other pattern
+// stages the tile in LDS as [line][position] in the output type; thread = line walks the blocks
+// of m positions, looks up the slot of (line, block) in the slot map (the inverse of `idx`,
+// built once per pattern by nmg_slotmap), derives the pattern from the slot and writes the n
+// kept values of the block to their place in `val`.
 #include "nmg_common.h"
 #include "nmg_tile.h"
 
@@ -36,16 +37,6 @@ typedef _Float16 sd_f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 sd_bf16x8 __attribute__((ext_vector_type(8)));
 typedef short sd_i16x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) sd_i16x4 *sd_lds_i16x4;
-
-template <typename T> struct SdMma;
-template <> struct SdMma<__half> {
-    using F = sd_f16x8;
-    __device__ static f32x16 run(F a, F b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
-};
-template <> struct SdMma<__hip_bfloat16> {
-    using F = sd_bf16x8;
-    __device__ static f32x16 run(F a, F b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
-};
 
 // fp32 -> stored 16 bits, round to nearest even (bf16 by the conversion instruction of gfx950)
 template <typename T> __device__ __forceinline__ uint16_t sd_bits16(float x);
@@ -119,279 +110,16 @@ static_assert(SD_LDS <= 160 * 1024, "LDS of a CU");
 static_assert(SD_D < SD_NS, "a stage is refilled only after the barrier that ends its last read");
 static_assert(SD_D * SD_LPW < 64, "vmcnt is a 6-bit counter");
 
-// MODE 0: any n:m, through the staged tile.  (m == 4 and m == 8 with n = 1, 2, 4 take
-// sddmm16_kernel, whose epilogue stays in registers.)
-// NT = true: the operands are given with the reduction (tokens) as their fast dim, L^T [G, T] and
-// P^T [S, T] (the weight gradient of torch.mm(W, B): grad_out [R, N] and B [C, N] as they lie in
-// memory).  An operand tile of a K step is then 256 feature rows of 64 bytes; a fragment -- the
-// lane's 8 consecutive tokens of its feature -- is one 16-byte LDS read, and the 16-byte pieces of
-// a row are XOR-swizzled with (row/4)%4 on the global side so that the reads hit every bank once.
-template <typename T, int MODE, bool NT = false>
-__global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
+// Second half of the staged epilogue: the tile lies in LDS as [line][position] in the output type
+// (SD_PITCH bytes per line), the order table behind it; thread = line walks the blocks of m
+// positions that meet the tile, looks up the slot of (line, block) in the slot map, derives the
+// pattern from the slot and writes the n kept values of the block to their place in val.
+__device__ __forceinline__ void sd_staged_walk(const SddmmParams &P, const unsigned char *smem, int tid, int64_t l0,
+                                               int64_t p0)
 {
-    using Mm = SdMma<T>;
-    static_assert(MODE == 0, "the staged tile (the epilogues in registers are sddmm16_kernel's)");
-    extern __shared__ __align__(16) unsigned char smem[];
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-
-    // Workgroup -> tile.  Consecutive ids are dealt round-robin to the 8 XCDs: give each XCD a
-    // contiguous run of ids, and walk the grid in bands of 4 position tiles, so that a run covers
-    // a compact block of tiles whose operands stay in that XCD's L2.
-    int id = blockIdx.x;
-    const int ntiles = P.tiles_p * P.tiles_l;
-    if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
-    constexpr int GH = 4;
-    const int band = id / (GH * P.tiles_l);
-    const int band_h = min(P.tiles_p - band * GH, GH);
-    const int in_band = id - band * GH * P.tiles_l;
-    const int tile_p = band * GH + in_band % band_h, tile_l = in_band / band_h;
-    const int64_t p0 = (int64_t)tile_p * 256, l0 = (int64_t)tile_l * 256;
-    const int wm = wave >> 1, wn = wave & 1;   // position half / line half of the wavefront
-    const int KP = P.KP;
-
-    // ---- DMA sources.  Wavefronts 0, 1 fetch the position tile, 2, 3 the line tile; load i of a
-    // wavefront fills token rows 2r, 2r+1 (r = (wave & 1) * 8 + i) of its operand tile: 1 KiB of
-    // LDS, lane l -> row 2r + l/32, 16-byte piece l%32.  Piece x of token row t holds the logical
-    // chunk x ^ 4*(t%4) (8 features): the transposing reads below then hit every bank once.
-    const bool is_l = wave >= 2;
-    const unsigned char *gsrc = (const unsigned char *)(is_l ? P.lop : P.pop);
-    const int64_t ld = is_l ? P.ldl : P.ldp, ext = is_l ? P.G : P.S, f0 = is_l ? l0 : p0;
-    uint32_t g_off[SD_LPW];
-#pragma unroll
-    for (int i = 0; i < SD_LPW; i++) {
-        if constexpr (NT) {
-            // load i fills feature rows (wave & 1) * 128 + 16 i + l/4, slot l%4 <- logical piece
-            // (l%4) ^ (row/4)%4 (8 tokens); rows beyond the extent repeat the last one (never stored)
-            const int row = (wave & 1) * 128 + 16 * i + (lane >> 2);
-            const int piece = (lane & 3) ^ ((row >> 2) & 3);
-            int64_t feat = f0 + row;
-            if (feat > ext - 1) feat = ext - 1;
-            g_off[i] = (uint32_t)(((feat - min(f0, ext - 1)) * ld + piece * 8) * 2);
-        } else {
-            const int tok = (((wave & 1) * 8 + i) << 1) + (lane >> 5);
-            const int chunk = (lane & 31) ^ ((tok & 3) << 2);
-            int64_t feat = f0 + chunk * 8;
-            if (feat > ext - 8) feat = ext - 8;   // columns beyond the extent feed outputs that are never stored
-            g_off[i] = (uint32_t)((tok * ld + feat) * 2);
-        }
-    }
-    const int tok_hi = lane >> 5;
-    const int nt_tok = ((lane & 3) ^ ((lane >> 4) & 3)) * 8;   // NT: first token of the lane's piece (the same in every load)
-    const unsigned char *zero = (const unsigned char *)P.zero;
-    // The DMA loads are written as instructions: they have no destination registers, so nothing
-    // the compiler does with registers can race with them, and the compiler -- which would make
-    // every LDS read wait for all DMA loads in flight -- does not see them.  Their completion is
-    // tracked by the counted waits below.  (Every load that writes registers is the compiler's.)
-    // K step kp goes to stage kp % SD_NS.  Steps beyond the last are fetched like the last one
-    // (the count of outstanding operations stays uniform; the data is never used).
-    struct Step {
-        const unsigned char *b;   // first token row of the step in the wavefront's operand
-        uint32_t dst;             // LDS address of the wavefront's first load
-        int rem;                  // valid token rows of the step (>= SD_KS except at the end)
-    };
-    auto step_of = [&](int kp) {
-        const int kq = kp < KP ? kp : KP - 1;
-        Step st;
-        st.b = NT ? gsrc + (min(f0, ext - 1) * ld + (int64_t)kq * SD_KS) * 2 : gsrc + (int64_t)kq * SD_KS * ld * 2;
-        st.dst = (uint32_t)(uintptr_t)(lds_ptr_t)(smem + (kp & (SD_NS - 1)) * SD_STAGE + (is_l ? SD_OP : 0) +
-                                                  (wave & 1) * 8 * 1024);
-        st.rem = (int)min((int64_t)SD_KS, P.T - (int64_t)kq * SD_KS);
-        return st;
-    };
-    // tail_tag: the step may hold the end of the operands -- token rows beyond it come from a page
-    // of zeros, at the price of a 64-bit address per lane; the steps before the last take the
-    // scalar base + 32-bit lane offset form.
-    auto issue_one = [&](const Step &st, int i, auto tail_tag) {
-        if constexpr (decltype(tail_tag)::value) {
-            const int tok = NT ? nt_tok : (((wave & 1) * 8 + i) << 1) + tok_hi;
-            const unsigned char *src = tok < st.rem ? st.b + g_off[i] : zero;
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                         :: "v"(src), "s"(st.dst + i * 1024) : "memory");
-        } else {
-            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                         :: "v"(g_off[i]), "s"(st.b), "s"(st.dst + i * 1024) : "memory");
-        }
-    };
-
-    // ---- fragment addresses.  Lane (q = l/16, i = l%16) of a transposing read supplies the 8
-    // bytes at token 8*(q/2) + i/4 (+ 16*kk + 4*r), features 16*(q%2) + 4*(i%4) .. +3 of the
-    // 32-feature block, and receives feature 16*(q%2) + i = l%32 at tokens 8*(l/32) + 4r + 0..3:
-    // reads r = 0, 1 give the lane its 8 reduction positions of k-step kk, the operand order of
-    // the instruction with reduction slot 8h + 4r + j <-> token 16kk + 8h + 4r + j on both sides.
-    const int q = lane >> 4, i16 = lane & 15, a = i16 >> 2;
-    const int lane_base = (8 * (q >> 1) + a) * 512 + (2 * (q & 1) + ((i16 & 3) >> 1)) * 16 + (i16 & 1) * 8;
-    int fa_off[4], fb_off[4];   // per 32-feature block of the wavefront: position side, line side
-#pragma unroll
-    for (int f = 0; f < 4; f++) {
-        fa_off[f] = lane_base + ((wm * 4 + (f ^ a)) << 6);
-        fb_off[f] = lane_base + ((wn * 4 + (f ^ a)) << 6) + SD_OP;
-    }
-
-    struct Frags {
-        sd_i16x4 a[4][2], b[4][2];
-    };
-    Frags fr[2];
-    // fragment number w in the order the MFMAs first need them: a0, b0, b1, b2, b3, a1, a2, a3
-    // NT: lane (i = l%32, h = l/32) reads the 16 bytes of feature row 32*blk + i, piece 2*kk + h
-    // (stored at slot piece ^ (row/4)%4): its 8 tokens of k-step kk.
-    const int nt_row = (lane & 31) * 64, nt_sw = (lane >> 2) & 3, nt_h = lane >> 5;
-    auto read_one = [&](Frags &f, const unsigned char *stage, int kk, int w) {
-        const bool is_a = w == 0 || w >= 5;
-        const int x = w == 0 ? 0 : (w >= 5 ? w - 4 : w - 1);
-        if constexpr (NT) {
-            const int at = ((is_a ? wm : wn) * 4 + x) * 32 * 64 + nt_row + (((2 * kk + nt_h) ^ nt_sw) << 4) + (is_a ? 0 : SD_OP);
-            union {
-                u32x4 u;
-                sd_i16x4 h[2];
-            } c;
-            c.u = *(const u32x4 *)(stage + at);
-            if (is_a) {
-                f.a[x][0] = c.h[0];
-                f.a[x][1] = c.h[1];
-            } else {
-                f.b[x][0] = c.h[0];
-                f.b[x][1] = c.h[1];
-            }
-            return;
-        }
-#pragma unroll
-        for (int r = 0; r < 2; r++) {
-            if (is_a)
-                f.a[x][r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (sd_lds_i16x4)(stage + fa_off[x] + (16 * kk + 4 * r) * 512));
-            else
-                f.b[x][r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (sd_lds_i16x4)(stage + fb_off[x] + (16 * kk + 4 * r) * 512));
-        }
-    };
-    auto read_frags = [&](Frags &f, const unsigned char *stage, int kk) {
-#pragma unroll
-        for (int w = 0; w < 8; w++) read_one(f, stage, kk, w);
-    };
-
-    f32x16 acc[4][4];   // [position block][line block]
-#pragma unroll
-    for (int x = 0; x < 4; x++)
-#pragma unroll
-        for (int y = 0; y < 4; y++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[x][y][r] = 0.f;
-
-    auto mma = [&](const Frags &f, int lo, int hi) {
-#pragma unroll
-        for (int x = 0; x < 4; x++) {
-            union {
-                sd_i16x4 h[2];
-                typename Mm::F v;
-            } ca;
-            ca.h[0] = f.a[x][0];
-            ca.h[1] = f.a[x][1];
-#pragma unroll
-            for (int y = 0; y < 4; y++) {
-                if (x * 4 + y < lo || x * 4 + y >= hi) continue;
-                union {
-                    sd_i16x4 h[2];
-                    typename Mm::F v;
-                } cb;
-                cb.h[0] = f.b[y][0];
-                cb.h[1] = f.b[y][1];
-                acc[x][y] = Mm::run(ca.v, cb.v, acc[x][y]);
-            }
-        }
-    };
-
-    // Invariants of the ring.  (1) Outstanding memory operations of a wavefront complete in issue
-    // order, SD_LPW per K step; at the counted wait of step kp the steps kp+1 .. kp+SD_D are
-    // outstanding, so vmcnt((SD_D-1) * SD_LPW) means "my share of step kp+1 has landed", and the
-    // barrier after it "everybody's".  (2) Stage (kp+SD_D) % SD_NS is refilled during step kp; its
-    // last readers were the fragment reads of step kp+SD_D-SD_NS <= kp-1, all of which completed
-    // (lgkmcnt(0)) before the barrier that ended that step.
-#pragma unroll
-    for (int s0 = 0; s0 < SD_D; s0++) {
-        const Step st = step_of(s0);
-#pragma unroll
-        for (int i = 0; i < SD_LPW; i++) issue_one(st, i, std::true_type{});
-    }
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SD_D - 1) * SD_LPW) : "memory");
-    asm volatile("s_barrier" ::: "memory");
-    read_frags(fr[0], smem, 0);
-
-    // The statements between scheduling fences are issued in this order: one MFMA (32 clocks of
-    // the matrix pipe), then the LDS reads or the DMA load that run in its shadow.
-    auto k_step = [&](int kp, auto tail_tag) {
-        const unsigned char *cur = smem + (kp & (SD_NS - 1)) * SD_STAGE;
-        const unsigned char *nxt = smem + ((kp + 1) & (SD_NS - 1)) * SD_STAGE;
-        const Step st = step_of(kp + SD_D);
-        // k-step 0: under its MFMAs, the fragments of k-step 1, then the loads of step kp+SD_D
-#pragma unroll
-        for (int w = 0; w < 8; w++) {
-            mma(fr[0], w, w + 1);
-            __builtin_amdgcn_sched_barrier(0);
-            read_one(fr[1], cur, 1, w);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-#pragma unroll
-        for (int w = 0; w < 8; w++) {
-            mma(fr[0], 8 + w, 9 + w);
-            __builtin_amdgcn_sched_barrier(0);
-            issue_one(st, w, tail_tag);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        // k-step 1: after its first MFMAs, wait for step kp+1 and meet the other wavefronts (the
-        // LDS reads of step kp are complete); then the first fragments of step kp+1
-        mma(fr[1], 0, 4);
-        __builtin_amdgcn_sched_barrier(0);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SD_D - 1) * SD_LPW) : "memory");
-        asm volatile("s_barrier" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int w = 0; w < 8; w++) {
-            mma(fr[1], 4 + w, 5 + w);
-            __builtin_amdgcn_sched_barrier(0);
-            read_one(fr[0], nxt, 0, w);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        mma(fr[1], 12, 16);
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    // steps whose prefetch (step kp + SD_D) lies before the last step take the short address form
-    const int kp_tail = max(0, KP - 1 - SD_D);
-    for (int kp = 0; kp < kp_tail; kp++) k_step(kp, std::false_type{});
-    for (int kp = kp_tail; kp < KP; kp++) k_step(kp, std::true_type{});
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    const int8_t *s_ord = (const int8_t *)(smem + 256 * SD_PITCH);
     uint16_t *val = (uint16_t *)P.val;
     const int n = P.n, m = P.m;
-
-    asm volatile("s_barrier" ::: "memory");
-
-    // ---- epilogue through LDS: stage [line][position] in the output type (D rows = positions
-    // 8*(r/4) + 4*(l/32) + r%4 of the block, column = line l%32: a lane stores 4 consecutive
-    // positions of its line)
-    int8_t *s_ord = (int8_t *)(smem + 256 * SD_PITCH);
-    for (int i = tid; i < P.order_bytes; i += 256) s_ord[i] = P.order[i];
-    {
-        const int j = lane & 31, h = lane >> 5;
-#pragma unroll
-        for (int y = 0; y < 4; y++)
-#pragma unroll
-            for (int x = 0; x < 4; x++)
-#pragma unroll
-                for (int rq = 0; rq < 4; rq++) {
-                    uint16_t hh[4];
-#pragma unroll
-                    for (int e = 0; e < 4; e++) hh[e] = f32_to_bits16(acc[x][y][rq * 4 + e], (T *)nullptr);
-                    uint2 pk;
-                    pk.x = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
-                    pk.y = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
-                    const int line = wn * 128 + y * 32 + j, pos = wm * 128 + x * 32 + rq * 8 + h * 4;
-                    *(uint2 *)(smem + line * SD_PITCH + pos * 2) = pk;
-                }
-    }
-    __syncthreads();
-
-    // ---- thread = line: walk the blocks of m positions that meet the tile
     const int64_t line = l0 + tid;
     if (line >= P.Gpad) return;
     const bool line_ok = line < P.G;
@@ -430,10 +158,9 @@ __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
     }
 }
 
-// ------------------------------------------- the same product with V_MFMA_F32_16X16X32
-// The 16 x 16 x 32 form of the instruction sustains 10-17 % more flops under the power limit than
-// the 32 x 32 x 16 form, and a K step of 32 tokens is exactly one of its reduction steps.  Same
-// tile, same ring, same DMA loads and counted waits as sddmm_kernel; what differs:
+// ------------------------------------------------------------------------------ the product
+// V_MFMA_F32_16X16X32: of the two dense forms of the instruction the one that sustains more flops
+// under the power limit (10-17 % more than 32 x 32 x 16), and its reduction step is the K step.
 //   fragments: lane (kq = l/16, i = l%16) holds feature i of a 16-feature block at tokens
 //     8 kq .. 8 kq + 7 -- two transposing reads (token-major operands) or one 16-byte read
 //     (reduction-contiguous operands).  For the transposing reads the 64-byte granules of a token
@@ -443,7 +170,7 @@ __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
 //     placement that separates them, 16-byte pieces XOR 4 * (t % 4) + 2 * ((t / 8) % 2), measured
 //     conflict-free and 2.4 % slower: the LDS reads are not what the loop waits for.)
 //   accumulators: 8 x 8 blocks of 16 positions x 16 lines, 4 registers each; lane (j = l%16,
-//     q = l/16) holds line j and the positions 4q .. 4q+3 of the block -- one block of m = 4.
+//     q = l/16) holds line j and the positions 4q .. 4q+3 of the block.
 //   a K step is two phases (position blocks 0..3, 4..7) of 32 MFMAs, column by column; the line
 //     fragments live in one register set: column y of the second phase frees fragment y, which is
 //     then read for the next step.
@@ -452,6 +179,12 @@ __global__ __launch_bounds__(256, 1) void sddmm_kernel(SddmmParams P)
 // the lane's 64 (line, block) pairs are fetched when the kernel starts and wait in registers.
 // MODE 8 + n (n = 1, 2, 4): m == 8; the two lanes that hold the halves of a block exchange them
 // first (V_PERMLANE16_SWAP), then two byte permutes per output word.
+// MODE 0: any n:m, through the staged tile.
+// NT = true: the operands are given with the reduction (tokens) as their fast dim, L^T [G, T] and
+// P^T [S, T] (the weight gradient of torch.mm(W, B): grad_out [R, N] and B [C, N] as they lie in
+// memory).  An operand tile of a K step is then 256 feature rows of 64 bytes; a fragment -- the
+// lane's 8 consecutive tokens of its feature -- is one 16-byte LDS read, and the 16-byte pieces of
+// a row are XOR-swizzled with (row/4)%4 on the global side.
 template <typename T> struct SdMma16;
 template <> struct SdMma16<__half> {
     using F = sd_f16x8;
@@ -466,12 +199,14 @@ template <typename T, int MODE, bool NT = false>
 __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
 {
     using Mm = SdMma16<T>;
-    static_assert((MODE >= 1 && MODE <= 4) || MODE == 9 || MODE == 10 || MODE == 12, "m == 4, n == MODE; m == 8, n == MODE - 8");
+    static_assert((MODE >= 0 && MODE <= 4) || MODE == 9 || MODE == 10 || MODE == 12, "the staged tile; m == 4, n == MODE; m == 8, n == MODE - 8");
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    // workgroup -> tile as in sddmm_kernel
+    // Workgroup -> tile.  Consecutive ids are dealt round-robin to the 8 XCDs: give each XCD a
+    // contiguous run of ids, and walk the grid in bands of 4 position tiles, so that a run covers
+    // a compact block of tiles whose operands stay in that XCD's L2.
     int id = blockIdx.x;
     const int ntiles = P.tiles_p * P.tiles_l;
     if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
@@ -490,8 +225,8 @@ __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
     // MODE 8 + n: a block of 8 positions lies in the lanes q = l/16 even (positions 0..3) and odd
     // (4..7) of one accumulator block; after the exchange in the epilogue a lane owns, per pair of
     // position blocks xp, block p0/8 + wm*16 + 4 xp + 2 (q%2) + q/2 of its line (xp even in the low half).
-    uint32_t my_slot[MODE <= 4 ? 32 : 16];
-    if constexpr (MODE <= 4) {
+    uint32_t my_slot[MODE == 0 ? 1 : (MODE <= 4 ? 32 : 16)];
+    if constexpr (MODE >= 1 && MODE <= 4) {
         uint32_t *s_sel = (uint32_t *)(smem + 256 * SD_PITCH);
         if (tid < 16) {
             const uint32_t o = (uint32_t)(P.ord4 >> (8 * (tid & 7)));
@@ -510,7 +245,7 @@ __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
                                       ((uint32_t)(uint16_t)P.slot[blk1 * P.Gpad + line] << 16);
             }
         }
-    } else {
+    } else if constexpr (MODE > 8) {
         // selector table: per pattern and output word two V_PERM_B32 selectors, one for the
         // positions 0..3, one for 4..7 (bytes that come from the other half select zero)
         constexpr int N = MODE - 8, ND = (N + 1) / 2;
@@ -544,7 +279,12 @@ __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
         }
     }
 
-    // ---- DMA sources: as in sddmm_kernel, except for the swizzle of the token-major tiles
+    // ---- DMA sources.  Wavefronts 0, 1 fetch the position tile, 2, 3 the line tile; load i of a
+    // wavefront fills token rows 2r, 2r+1 (r = (wave & 1) * 8 + i) of its operand tile: 1 KiB of
+    // LDS, lane l -> row 2r + l/32, 16-byte piece l%32, which holds the logical chunk (8 features)
+    // (l%32) ^ 4 * ((t % 4) + 4 * ((t / 8) % 2)) of token row t.  NT: load i fills feature rows
+    // (wave & 1) * 128 + 16 i + l/4, slot l%4 <- logical piece (l%4) ^ (row/4)%4 (8 tokens); rows
+    // beyond the extent repeat the last one (never stored).
     const bool is_l = wave >= 2;
     const unsigned char *gsrc = (const unsigned char *)(is_l ? P.lop : P.pop);
     const int64_t ld = is_l ? P.ldl : P.ldp, ext = is_l ? P.G : P.S, f0 = is_l ? l0 : p0;
@@ -568,10 +308,16 @@ __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
     const int tok_hi = lane >> 5;
     const int nt_tok = ((lane & 3) ^ ((lane >> 4) & 3)) * 8;
     const unsigned char *zero = (const unsigned char *)P.zero;
+    // The DMA loads are written as instructions: they have no destination registers, so nothing
+    // the compiler does with registers can race with them, and the compiler -- which would make
+    // every LDS read wait for all DMA loads in flight -- does not see them.  Their completion is
+    // tracked by the counted waits below.  (Every load that writes registers is the compiler's.)
+    // K step kp goes to stage kp % SD_NS.  Steps beyond the last are fetched like the last one
+    // (the count of outstanding operations stays uniform; the data is never used).
     struct Step {
-        const unsigned char *b;
-        uint32_t dst;
-        int rem;
+        const unsigned char *b;   // first token row of the step in the wavefront's operand
+        uint32_t dst;             // LDS address of the wavefront's first load
+        int rem;                  // valid token rows of the step (>= SD_KS except at the end)
     };
     auto step_of = [&](int kp) {
         const int kc = kp < KP ? kp : KP - 1;
@@ -582,6 +328,9 @@ __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
         st.rem = (int)min((int64_t)SD_KS, P.T - (int64_t)kc * SD_KS);
         return st;
     };
+    // tail_tag: the step may hold the end of the operands -- token rows beyond it come from a page
+    // of zeros, at the price of a 64-bit address per lane; the steps before the last take the
+    // scalar base + 32-bit lane offset form.
     auto issue_one = [&](const Step &st, int i, auto tail_tag) {
         if constexpr (decltype(tail_tag)::value) {
             const int tok = NT ? nt_tok : (((wave & 1) * 8 + i) << 1) + tok_hi;
@@ -659,9 +408,14 @@ __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
         acc[x][y] = Mm::run(ca.v, cb.v, acc[x][y]);
     };
 
-    // The ring: as in sddmm_kernel (SD_LPW loads per wavefront and K step, SD_D steps ahead; the
-    // counted wait of step kp means "my share of step kp+1 has landed", the barrier "everybody's";
-    // stage kp % SD_NS is read for the last time before that barrier and refilled during step kp+1).
+    // Invariants of the ring.  (1) Outstanding memory operations of a wavefront complete in issue
+    // order, SD_LPW per K step; at the counted wait of step kp the steps kp+1 .. kp+SD_D are
+    // outstanding, so vmcnt((SD_D-1) * SD_LPW) means "my share of step kp+1 has landed", and the
+    // barrier after it "everybody's".  (2) Stage (kp+SD_D) % SD_NS = (kp-1) % SD_NS is refilled
+    // during the first phase of step kp; its last readers were the first-phase reads of step kp-1
+    // (from their own stage) and the second-phase reads of step kp-2 (which fetch ahead); both
+    // completed (lgkmcnt(0)) before the barrier of step kp-1, which every wavefront has passed
+    // before it issues the loads of step kp.
 #pragma unroll
     for (int s0 = 0; s0 < SD_D; s0++) {
         const Step st = step_of(s0);
@@ -730,13 +484,34 @@ __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
         }
         __builtin_amdgcn_sched_barrier(0);
     };
+    // steps whose prefetch (step kp + SD_D) lies before the last step take the short address form
     const int kp_tail = max(0, KP - 1 - SD_D);
     for (int kp = 0; kp < kp_tail; kp++) k_step(kp, std::false_type{});
     for (int kp = kp_tail; kp < KP; kp++) k_step(kp, std::true_type{});
     pin_acc();
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 
-    if constexpr (MODE > 8) {
+    if constexpr (MODE == 0) {
+        // ---- epilogue through LDS: stage [line][position] in the output type, then thread = line
+        asm volatile("s_barrier" ::: "memory");   // every wavefront is done with the ring
+        int8_t *s_ord = (int8_t *)(smem + 256 * SD_PITCH);
+        for (int i = tid; i < P.order_bytes; i += 256) s_ord[i] = P.order[i];
+#pragma unroll
+        for (int y = 0; y < 8; y++)
+#pragma unroll
+            for (int x = 0; x < 8; x++) {
+                uint16_t hh[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) hh[r] = sd_bits16<T>(sd_from_acc(acc[x][y][r]));
+                uint2 pk;
+                pk.x = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
+                pk.y = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
+                const int line = wn * 128 + y * 16 + j16, pos = wm * 128 + x * 16 + kq * 4;
+                *(uint2 *)(smem + line * SD_PITCH + pos * 2) = pk;
+            }
+        __syncthreads();
+        sd_staged_walk(P, smem, tid, l0, p0);
+    } else if constexpr (MODE > 8) {
         // ---- epilogue in registers, m == 8.  The lanes q even / odd round and pack their halves of
         // the blocks in the accumulator blocks 2 xp and 2 xp + 1 and exchange them
         // (V_PERMLANE16_SWAP: odd rows of 16 lanes of the first operand <-> even rows of the second),
@@ -969,14 +744,14 @@ static int sddmm_impl(bool nt, const void *d_lines, int64_t ld_lines, const void
         using T = decltype(tag);
         if (nt) {   // reduction-contiguous operands: 2:4 in registers, every other pattern through the staged tile
             if (in_regs && n == 2 && S % 4 == 0) return launch(sddmm16_kernel<T, 2, true>);   // (no padded positions)
-            return launch(sddmm_kernel<T, 0, true>);
+            return launch(sddmm16_kernel<T, 0, true>);
         }
         if (in_regs8) {
             if (n == 1) return launch(sddmm16_kernel<T, 9>);
             if (n == 2) return launch(sddmm16_kernel<T, 10>);
             return launch(sddmm16_kernel<T, 12>);
         }
-        if (!in_regs) return launch(sddmm_kernel<T, 0>);
+        if (!in_regs) return launch(sddmm16_kernel<T, 0>);
         switch (n) {
         case 1: return launch(sddmm16_kernel<T, 1>);
         case 2: return launch(sddmm16_kernel<T, 2>);
