@@ -1,5 +1,5 @@
-// nmg x dense matmul on the dense matrix cores (V_MFMA_F32_32X32X16_{F16,BF16}) with the weight
-// expanded beforehand into the register order of the instruction ("densefrag" operand).
+// nmg x dense matmul on the dense matrix cores (V_MFMA_F32_16X16X32_{F16,BF16}) with the weight
+// expanded beforehand into the register order of the matrix instructions ("densefrag" operand).
 //
 // Serves what the sparse matrix cores cannot: patterns that do not fit 2-of-4 groups (4:8,
 // 3:4, ...) and the reduction along the *group* dim, i.e. the gradient with respect to the
@@ -9,16 +9,18 @@
 //   transpose = 1:  Y[tok, s] = sum_q X[tok, q] * W2[q, s]
 //
 // Two kernels:
-//   densefrag_kernel   rowpack -> densefrag, through an LDS tile (reads and writes contiguous);
-//   dense_direct_kernel  the multiplication, same skeleton as the direct-weights kernel of the
-//                        sparse matrix cores: 4 wavefronts stacked on the output dim, weight
-//                        fragments global -> registers DD_D K steps ahead, activation tile
-//                        global -> LDS by DMA, one barrier per K step of 64.
+//   densefrag_kernel       rowpack -> densefrag, through an LDS tile (reads and writes contiguous);
+//   dense16_direct_kernel  the multiplication, same skeleton as the direct-weights kernel of the
+//                          sparse matrix cores: 4 wavefronts stacked on the output dim, weight
+//                          fragments global -> registers DD_D K steps ahead, activation tile
+//                          global -> LDS by DMA, one barrier per K step of 64.
 //
 // densefrag [OB][K16][64 lanes][8]: for output block ob (32 outputs) and k-step k16 (16 reduction
 // positions), lane l holds the 8 weights of output ob*32 + l%32 at reduction positions
-// k16*16 + 8*(l/32) + 0..7 -- the A operand of the instruction.  OB is padded to a multiple of 8
-// (256 outputs), the reduction extent must be a multiple of 64; padding is zero.
+// k16*16 + 8*(l/32) + 0..7 -- the A operand of V_MFMA_F32_32X32X16, which the first form of the
+// multiplication used; the 16 x 16 x 32 instruction finds its fragments in it with another lane
+// offset (below).  OB is padded to a multiple of 8 (256 outputs), the reduction extent must be a
+// multiple of 64; padding is zero.
 #include "nmg_common.h"
 #include "nmg_tile.h"
 
@@ -28,16 +30,6 @@ namespace nmg {
 
 typedef _Float16 df_f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 df_bf16x8 __attribute__((ext_vector_type(8)));
-
-template <typename T> struct DfMma;
-template <> struct DfMma<__half> {
-    using F = df_f16x8;
-    __device__ static f32x16 run(F a, F b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
-};
-template <> struct DfMma<__hip_bfloat16> {
-    using F = df_bf16x8;
-    __device__ static f32x16 run(F a, F b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
-};
 
 // ------------------------------------------------------------------ rowpack -> densefrag
 constexpr int DFX_L = 64, DFX_P = 128;   // LDS tile: lines x positions
@@ -177,368 +169,10 @@ struct DfParams {
 constexpr int DD_D = 2;    // K steps in flight (a dense K step takes twice the MFMA time of a sparse one)
 constexpr int DD_NS = 4;   // activation stages in LDS (>= DD_D + 1)
 
-// FB x TB accumulator blocks (32 outputs x 32 tokens) per wavefront, WM x WN wavefronts, NH token
-// parts per k-step.  A K step (64) is 4 k-steps of 16; a phase is one (k-step, token part) pair:
-// its MFMAs run while the activation fragments of the next phase are read from LDS, and the
-// loads of K step kp+DD_D are dealt out over the phases.
-template <typename T, int FB, int TB, int WM, int WN, int NH>
-__global__ __launch_bounds__(256, 1) void dense_direct_kernel(DfParams P)
-{
-    using Mm = DfMma<T>;
-    static_assert(WM * WN == 4, "four wavefronts");
-    static_assert(TB % NH == 0, "token blocks split evenly into phases");
-    constexpr int TF = WM * FB * 32, TT = WN * TB * 32;   // workgroup tile: outputs x tokens
-    constexpr int STAGE = TT * 128;                       // activation bytes per K step
-    constexpr int XL = TT / 32;                           // DMA loads per wavefront per K step
-    constexpr int OPS = XL + 4 * FB;                      // memory operations per wavefront per K step
-    constexpr int BT = TB / NH;                           // token blocks per phase
-    constexpr int NP = 4 * NH;                            // phases per K step
-    constexpr int NM = FB * BT;                           // MFMAs per phase
-    static_assert(OPS * DD_D < 64, "vmcnt is a 6-bit counter");
-    static_assert(NM >= 4, "phase too short to hide the loads behind");
-    extern __shared__ __align__(16) unsigned char smem[];
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-
-    // Workgroup -> tile: consecutive ids are dealt round-robin to the 8 XCDs; give each XCD a
-    // contiguous run of ids and walk the grid in bands of 4 output tiles, so that a run covers
-    // a compact block of tiles whose weights and activations stay in that XCD's L2.
-    int id = blockIdx.x;
-    const int ntiles = P.tiles_m * P.tiles_n;
-    // slices of the reduction: the slices of a tile are workgroups ntiles apart
-    const int slice = P.ksplit > 1 ? id / ntiles : 0;
-    id -= slice * ntiles;
-    if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
-    constexpr int GH = 4;
-    const int band = id / (GH * P.tiles_n);
-    const int band_h = min(P.tiles_m - band * GH, GH);
-    const int in_band = id - band * GH * P.tiles_n;
-    const int tile_m = band * GH + in_band % band_h, tile_n = in_band / band_h;
-    const int64_t f0 = (int64_t)tile_m * TF, t0 = (int64_t)tile_n * TT;
-    // K steps kp_lo .. kp_lo + KP - 1 of the operand's KPT (the host leaves no slice empty)
-    const int KPT = P.KP;
-    const int kp_per = P.ksplit > 1 ? (KPT + P.ksplit - 1) / P.ksplit : KPT;
-    const int kp_lo = slice * kp_per;
-    const int KP = min(KPT, kp_lo + kp_per) - kp_lo;
-    const int wm = wave / WN, wn = wave % WN;
-    const int ob0 = (int)(f0 / 32) + wm * FB;
-
-    // ---- global sources (wavefront-uniform bases in scalar registers, the lane's share as a
-    //      32-bit offset) ----
-    const unsigned char *av_base[FB];
-#pragma unroll
-    for (int fb = 0; fb < FB; fb++)
-        av_base[fb] = (const unsigned char *)P.df + (((int64_t)(ob0 + fb) * KPT + kp_lo) * 4) * 1024;
-    const uint32_t lane16 = lane * 16;
-    const unsigned char *x_base = (const unsigned char *)P.x + (int64_t)kp_lo * 128;
-    uint32_t x_off[XL];
-#pragma unroll
-    for (int i = 0; i < XL; i++) {
-        const int row = (wave * XL + i) * 8 + (lane >> 3);
-        const int piece = lane & 7;
-        const int q = piece ^ ((row >> 1) & 7);   // logical 16-byte chunk stored at this piece
-        int64_t tok = t0 + row;
-        if (tok >= P.T) tok = P.T - 1;            // clamped rows are computed, never stored
-        x_off[i] = (uint32_t)((tok * P.ldx + q * 8) * 2);
-    }
-
-    struct WSet {
-        u32x4 a[FB][4];
-    };
-    WSet ws[DD_D + 1];
-    // Steps beyond the last repeat it: the operation count stays uniform, the data is unused.
-    auto issue_x = [&](int kp) {
-        if (kp >= KP) kp = KP - 1;
-        unsigned char *base = smem + (kp & (DD_NS - 1)) * STAGE;
-        const unsigned char *xb = x_base + (int64_t)kp * 128;
-#pragma unroll
-        for (int i = 0; i < XL; i++)
-            __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[i]),
-                                             (lds_ptr_t)(base + (wave * XL + i) * 1024), 16, 0, 0);
-    };
-    // load number i (0 .. OPS-1) of K step kp: first the XL activation DMA loads, then the
-    // 4 * FB weight fragments
-    auto issue_one = [&](int kp, WSet &w, int i) {
-        if (kp >= KP) kp = KP - 1;
-        if (i < XL) {
-            unsigned char *base = smem + (kp & (DD_NS - 1)) * STAGE;
-            const unsigned char *xb = x_base + (int64_t)kp * 128;
-#pragma unroll
-            for (int q = 0; q < XL; q++)
-                if (q == i)
-                    __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[q]),
-                                                     (lds_ptr_t)(base + (wave * XL + q) * 1024), 16, 0, 0);
-        } else {
-#pragma unroll
-            for (int fb = 0; fb < FB; fb++)
-#pragma unroll
-                for (int k16 = 0; k16 < 4; k16++)
-                    if (XL + fb * 4 + k16 == i) {
-                        const unsigned char *av = av_base[fb] + (int64_t)kp * 4096 + k16 * 1024;
-                        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(w.a[fb][k16]) : "v"(lane16), "s"(av) : "memory");
-                    }
-        }
-    };
-    auto issue_a = [&](int kp, WSet &w) {
-        if (kp >= KP) kp = KP - 1;
-#pragma unroll
-        for (int fb = 0; fb < FB; fb++) {
-            // Written as instructions so that their completion is tracked by the explicit vmcnt
-            // waits below and by nothing else, and with accumulation registers as targets: a
-            // compiler-made copy of a register whose load is still in flight would copy stale
-            // data, and the ring does not fit in the architectural registers.
-            const unsigned char *av = av_base[fb] + (int64_t)kp * 4096;
-            asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(w.a[fb][0]) : "v"(lane16), "s"(av) : "memory");
-            asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(w.a[fb][1]) : "v"(lane16), "s"(av) : "memory");
-            asm volatile("global_load_dwordx4 %0, %1, %2 offset:2048" : "=v"(w.a[fb][2]) : "v"(lane16), "s"(av) : "memory");
-            asm volatile("global_load_dwordx4 %0, %1, %2 offset:3072" : "=v"(w.a[fb][3]) : "v"(lane16), "s"(av) : "memory");
-        }
-    };
-
-    f32x16 acc[FB][TB];
-#pragma unroll
-    for (int i = 0; i < FB; i++)
-#pragma unroll
-        for (int j = 0; j < TB; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
-    // 256 accumulators would fill the architectural registers exactly; pin half of them to
-    // the accumulation registers (the MFMA takes its C/D operand from either file).
-    auto pin_acc = [&]() {
-        if constexpr (FB * TB * 16 > 128) {
-#pragma unroll
-            for (int tb = 0; tb < TB; tb++) asm volatile("" : "+a"(acc[FB - 1][tb]));
-        }
-    };
-    pin_acc();
-
-    // Activation fragment of k-step k16 (B operand): lane (token j = l%32, h = l/32) holds the 8
-    // reduction positions 16*k16 + 8h + 0..7 = 16-byte chunk 2*k16 + h of its token row; chunks
-    // are stored XOR-swizzled with (row/2)%8, so that 16 consecutive rows hit all banks.
-    const int j = lane & 31, h = lane >> 5, sw = (j >> 1) & 7;
-    int b_off[4];
-#pragma unroll
-    for (int k16 = 0; k16 < 4; k16++) b_off[k16] = (wn * TB * 32 + j) * 128 + (((k16 * 2 + h) ^ sw) << 4);
-
-    struct BFrags {
-        u32x4 b[BT];
-    };
-    BFrags fr[2];
-    // part 0 / 1: the first / second half of the phase's reads (part < 0: all of them)
-    auto read_b = [&](BFrags &f, const unsigned char *base, int ph, int part = -1) {
-        const int k16 = ph / NH, hh = ph % NH;
-#pragma unroll
-        for (int t = 0; t < BT; t++) {
-            if (part >= 0 && t / ((BT + 1) / 2) != part) continue;
-            f.b[t] = *(const u32x4 *)(base + b_off[k16] + (hh * BT + t) * 32 * 128);
-        }
-    };
-    // MFMAs lo..hi-1 of phase PH, numbered fb * BT + t
-    auto mma = [&](const WSet &w, const BFrags &f, auto ph_tag, int lo, int hi) {
-        constexpr int PH = decltype(ph_tag)::value, K16 = PH / NH, HH = PH % NH;
-#pragma unroll
-        for (int fb = 0; fb < FB; fb++) {
-            union {
-                u32x4 u;
-                typename Mm::F v;
-            } ca;
-            ca.u = w.a[fb][K16];
-#pragma unroll
-            for (int t = 0; t < BT; t++) {
-                if (fb * BT + t < lo || fb * BT + t >= hi) continue;
-                union {
-                    u32x4 u;
-                    typename Mm::F v;
-                } cb;
-                cb.u = f.b[t];
-                acc[fb][HH * BT + t] = Mm::run(ca.v, cb.v, acc[fb][HH * BT + t]);
-            }
-        }
-    };
-
-    // The counted wait.  Invariants it rests on:
-    //  (1) a wavefront's vector memory operations complete in issue order, and it issues exactly
-    //      OPS of them per K step (XL DMA loads, then 4 * FB weight fragments), all of step
-    //      kp+DD_D before the wait at the end of step kp; so at that wait the newest (DD_D-1) * OPS
-    //      operations are the steps kp+2 .. kp+DD_D and everything older -- step kp+1 -- has landed
-    //      once the counter is down to (DD_D-1) * OPS.  The barrier after it makes that true for
-    //      the DMA loads of the other wavefronts too.
-    //  (2) the weight set of step kp+1 is passed through the wait as in/out operands: whatever
-    //      uses those registers afterwards is ordered after the wait by the compiler as well.
-    //      (What it does with them *before* the wait is checked on the compiled code: no
-    //      instruction may touch a register with a load in flight, `python -m sten_amd.isa_check`.)
-    //  (3) LDS stage (kp+DD_D) % DD_NS is refilled during step kp; its last readers were the
-    //      fragment reads of step kp+DD_D-DD_NS <= kp-2, complete (lgkmcnt(0), same wait) before
-    //      the barrier that ended that step.  The two fragment sets alternate by phase; NP is
-    //      even, so the set read after the barrier (for phase 0 of the next step) is set 0.
-    static_assert(DD_NS > DD_D, "a stage must not be refilled while the step that reads it is in flight");
-    static_assert(NP % 2 == 0, "fragment sets alternate by phase across K steps");
-    static_assert(FB == 2, "the wait lists the registers of two fragment rows");
-    auto landed = [&](WSet &w) {
-        asm volatile("s_waitcnt vmcnt(%8) lgkmcnt(0)"
-                     : "+v"(w.a[0][0]), "+v"(w.a[0][1]), "+v"(w.a[0][2]), "+v"(w.a[0][3]),
-                       "+v"(w.a[1][0]), "+v"(w.a[1][1]), "+v"(w.a[1][2]), "+v"(w.a[1][3])
-                     : "n"((DD_D - 1) * OPS)
-                     : "memory");
-    };
-
-    // prologue: steps 0 .. DD_D-1 in flight, then wait for step 0
-#pragma unroll
-    for (int st = 0; st < DD_D; st++) {
-        issue_x(st);
-        issue_a(st, ws[st]);
-    }
-    landed(ws[0]);
-    asm volatile("s_barrier" ::: "memory");
-    read_b(fr[0], smem, 0);
-
-    for (int kp0 = 0; kp0 < KP; kp0 += DD_D + 1) {
-#pragma unroll
-        for (int u = 0; u <= DD_D; u++) {
-            const int kp = kp0 + u;
-            if (kp >= KP) break;
-            const unsigned char *base = smem + (kp & (DD_NS - 1)) * STAGE;
-            const unsigned char *next = smem + ((kp + 1) & (DD_NS - 1)) * STAGE;
-            // One phase: two MFMAs; the LDS reads of the next phase into the other fragment set;
-            // in the first two phases the loads of step kp+DD_D; the rest of the MFMAs.  Before
-            // the reads of the last phase, which fetch from the next stage, the barrier.  The
-            // instruction statements fence the scheduler, so this is also the issue order.
-            auto phase = [&](auto ph_tag) {
-                constexpr int PH = decltype(ph_tag)::value;
-                constexpr int L0 = PH * OPS / NP, L1 = (PH + 1) * OPS / NP;   // this phase's loads
-                // One memory instruction (or two LDS reads) goes into the shadow of one MFMA: a load
-                // holds the wavefront's issue for about 20 clocks, an LDS read for 7, an MFMA runs 32.
-                constexpr bool SPLIT = BT >= 2 && NM >= 6;
-                if (PH == NP - 1) {
-                    mma(ws[u], fr[PH % 2], ph_tag, 0, 2);
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int i = L0; i < OPS; i++) issue_one(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)], i);
-                    __builtin_amdgcn_sched_barrier(0);
-                    // fragments of step kp are in registers, my share of step kp+1 has landed ...
-                    landed(ws[(u + 1) % (DD_D + 1)]);
-                    asm volatile("s_barrier" ::: "memory");              // ... and everybody else's
-                    __builtin_amdgcn_sched_barrier(0);
-                    if constexpr (SPLIT) {
-                        mma(ws[u], fr[PH % 2], ph_tag, 2, 3);
-                        __builtin_amdgcn_sched_barrier(0);
-                        read_b(fr[(PH + 1) % 2], next, 0, 0);
-                        __builtin_amdgcn_sched_barrier(0);
-                        mma(ws[u], fr[PH % 2], ph_tag, 3, 4);
-                        __builtin_amdgcn_sched_barrier(0);
-                        read_b(fr[(PH + 1) % 2], next, 0, 1);
-                        __builtin_amdgcn_sched_barrier(0);
-                        mma(ws[u], fr[PH % 2], ph_tag, 4, NM);
-                    } else {
-                        read_b(fr[(PH + 1) % 2], next, 0);
-                        mma(ws[u], fr[PH % 2], ph_tag, 2, NM);
-                    }
-                } else {
-                    if constexpr (SPLIT) {
-                        mma(ws[u], fr[PH % 2], ph_tag, 0, 1);
-                        __builtin_amdgcn_sched_barrier(0);
-                        read_b(fr[(PH + 1) % 2], base, PH + 1, 0);
-                        __builtin_amdgcn_sched_barrier(0);
-                        mma(ws[u], fr[PH % 2], ph_tag, 1, 2);
-                        __builtin_amdgcn_sched_barrier(0);
-                        read_b(fr[(PH + 1) % 2], base, PH + 1, 1);
-                    } else {
-                        mma(ws[u], fr[PH % 2], ph_tag, 0, 2);
-                        __builtin_amdgcn_sched_barrier(0);
-                        read_b(fr[(PH + 1) % 2], base, PH + 1);
-                    }
-                    // The step's OPS loads are dealt out evenly over its phases, one at a time behind
-                    // an MFMA: a burst would find the CU's vector memory path busy and stall with
-                    // its MFMAs unissued.  (In the last phase the loads come before the counted
-                    // wait, which assumes them.)
-#pragma unroll
-                    for (int i = L0; i < L1; i++) {
-                        __builtin_amdgcn_sched_barrier(0);
-                        if (2 + i - L0 < NM) mma(ws[u], fr[PH % 2], ph_tag, 2 + i - L0, 3 + i - L0);
-                        __builtin_amdgcn_sched_barrier(0);
-                        issue_one(kp + DD_D, ws[(u + DD_D) % (DD_D + 1)], i);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (2 + L1 - L0 < NM) mma(ws[u], fr[PH % 2], ph_tag, 2 + L1 - L0, NM);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            };
-            phase(std::integral_constant<int, 0>{});
-            phase(std::integral_constant<int, 1>{});
-            phase(std::integral_constant<int, 2>{});
-            phase(std::integral_constant<int, 3>{});
-            if constexpr (NP >= 8) {
-                phase(std::integral_constant<int, 4>{});
-                phase(std::integral_constant<int, 5>{});
-                phase(std::integral_constant<int, 6>{});
-                phase(std::integral_constant<int, 7>{});
-            }
-            if constexpr (NP == 16) {
-                phase(std::integral_constant<int, 8>{});
-                phase(std::integral_constant<int, 9>{});
-                phase(std::integral_constant<int, 10>{});
-                phase(std::integral_constant<int, 11>{});
-                phase(std::integral_constant<int, 12>{});
-                phase(std::integral_constant<int, 13>{});
-                phase(std::integral_constant<int, 14>{});
-                phase(std::integral_constant<int, 15>{});
-            }
-            static_assert(NP == 4 || NP == 8 || NP == 16, "one, two or four token parts");
-        }
-    }
-    pin_acc();
-    // The loads of the steps beyond the last are still in flight and nothing reads what they bring:
-    // every register of the ring passes through the final wait, so that none of them is given to
-    // the epilogue while a load may still land in it.
-    static_assert(DD_D == 2 && FB == 2, "the final wait lists three weight sets of two fragment rows");
-    asm volatile("s_waitcnt vmcnt(0)"
-                 : "+v"(ws[0].a[0][0]), "+v"(ws[0].a[0][1]), "+v"(ws[0].a[0][2]), "+v"(ws[0].a[0][3]),
-                   "+v"(ws[0].a[1][0]), "+v"(ws[0].a[1][1]), "+v"(ws[0].a[1][2]), "+v"(ws[0].a[1][3]),
-                   "+v"(ws[1].a[0][0]), "+v"(ws[1].a[0][1]), "+v"(ws[1].a[0][2]), "+v"(ws[1].a[0][3]),
-                   "+v"(ws[1].a[1][0]), "+v"(ws[1].a[1][1]), "+v"(ws[1].a[1][2]), "+v"(ws[1].a[1][3]),
-                   "+v"(ws[2].a[0][0]), "+v"(ws[2].a[0][1]), "+v"(ws[2].a[0][2]), "+v"(ws[2].a[0][3]),
-                   "+v"(ws[2].a[1][0]), "+v"(ws[2].a[1][1]), "+v"(ws[2].a[1][2]), "+v"(ws[2].a[1][3])
-                 :
-                 : "memory");
-    asm volatile("s_barrier" ::: "memory");
-    if (P.ksplit > 1) {
-        store_partial_tile<FB, TB>(acc, P.part + (int64_t)slice * P.T * P.part_ld, P.part_ld, lane,
-                                   f0 + wm * FB * 32, t0 + wn * TB * 32, P.T);
-        return;
-    }
-    const TileOut out{P.y, P.bias, P.O, P.T, P.ldy};
-    smf_store_tile<T, FB, TB>(acc, smem + wave * (TB * 32 * (FB * 64 + 16)), lane, f0 + wm * FB * 32,
-                              t0 + wn * TB * 32, out);
-}
-
-template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_dense_direct(DfParams &P, hipStream_t s)
-{
-    constexpr int TF = WM * FB * 32, TT = WN * TB * 32;
-    static_assert(TF == 256, "the operand is padded to 256 outputs");
-    P.tiles_m = (int)((P.O + TF - 1) / TF);
-    P.tiles_n = (int)((P.T + TT - 1) / TT);
-    const int slices = P.ksplit > 1 ? P.ksplit : 1;
-    dim3 grid((unsigned)(P.tiles_m * P.tiles_n * slices));
-    constexpr size_t ring = (size_t)DD_NS * TT * 128, stg = (size_t)4 * TB * 32 * (FB * 64 + 16);
-    constexpr size_t lds = ring > stg ? ring : stg;
-    static_assert(lds <= 160 * 1024, "LDS");
-    auto k = dense_direct_kernel<T, FB, TB, WM, WN, NH>;
-    NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(k, grid, dim3(256), lds, s, P);
-    NMG_HIP_TRY(hipGetLastError());
-    if (slices > 1) {
-        const SplitSum Q{P.part, P.y, P.bias, P.O, P.T, P.ldy, P.part_ld, slices};
-        return launch_splitk_sum<T>(Q, s);
-    }
-    return NMG_OK;
-}
-
-// ------------------------------------------------- the same product with V_MFMA_F32_16X16X32
-// The 16 x 16 x 32 form of the instruction draws less power per flop than the 32 x 32 x 16 form
-// (from registers, random operands: 1.76-1.97 against 1.61-1.71 PFLOP/s), and with this skeleton
-// around it the difference stays.  Same operand, same ring, same counted waits as
-// dense_direct_kernel; what changes is who holds what:
+// V_MFMA_F32_16X16X32: of the two dense forms of the instruction the one that draws less power
+// per flop (from registers, random operands: 1.76-1.97 against 1.61-1.71 PFLOP/s for 32 x 32 x 16),
+// and with this skeleton around it the difference stays: the first form of this kernel, on
+// 32 x 32 x 16, reached matrix-pipe utilisation 0.90 and was 9-15 % slower.
 //   A fragment (16 outputs x 32 k): lane (r = l%16, kq = l/16) wants the 8 weights of output
 //     16*ab + r at k = 32*k32 + 8*kq + 0..7, which the densefrag operand stores in fragment
 //     (ob = ab/2, k16 = 2*k32 + kq/2) at lane 32*(kq%2) + 16*(ab%2) + r: a load still covers four
@@ -549,7 +183,8 @@ template <typename T, int FB, int TB, int WM, int WN, int NH> static int launch_
 //   D: lane holds token l%16, outputs 4*(l/16) + 0..3 of the 16 x 16 block.
 // A wavefront owns 64 outputs x TB*16 tokens: 4 x TB accumulator blocks of 4 registers, all of
 // them in the accumulation registers.  A K step of 64 is two k-steps of 32; a phase is one
-// (k-step, token part) pair of 4 * TB / NH MFMAs.
+// (k-step, token part) pair of 4 * TB / NH MFMAs: they run while the activation fragments of the
+// next phase are read from LDS, and the loads of K step kp+DD_D are dealt out over the phases.
 template <typename T> struct DfMma16;
 template <> struct DfMma16<__half> {
     using F = df_f16x8;
@@ -580,7 +215,9 @@ __global__ __launch_bounds__(256, 1) void dense16_direct_kernel(DfParams P)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    // workgroup -> tile as in dense_direct_kernel
+    // Workgroup -> tile: consecutive ids are dealt round-robin to the 8 XCDs; give each XCD a
+    // contiguous run of ids and walk the grid in bands of 4 output tiles, so that a run covers
+    // a compact block of tiles whose weights and activations stay in that XCD's L2.
     int id = blockIdx.x;
     const int ntiles = P.tiles_m * P.tiles_n;
     // slices of the reduction: the slices of a tile are workgroups ntiles apart
@@ -691,9 +328,21 @@ __global__ __launch_bounds__(256, 1) void dense16_direct_kernel(DfParams P)
         acc[ab][HH * BT + t] = Mm::run(ca.v, cb.v, acc[ab][HH * BT + t]);
     };
 
-    // The counted wait: as in dense_direct_kernel -- OPS memory operations per K step, issued in
-    // order, all of step kp+DD_D before the wait of step kp; the set of step kp+1 passes through
-    // the wait as in/out operands.
+    // The counted wait.  Invariants it rests on:
+    //  (1) a wavefront's vector memory operations complete in issue order, and it issues exactly
+    //      OPS of them per K step (XL DMA loads, then 2 * AB weight fragments), all of step
+    //      kp+DD_D before the wait in the last phase of step kp; so at that wait the newest
+    //      (DD_D-1) * OPS operations are the steps kp+2 .. kp+DD_D and everything older -- step
+    //      kp+1 -- has landed once the counter is down to (DD_D-1) * OPS.  The barrier after it
+    //      makes that true for the DMA loads of the other wavefronts too.
+    //  (2) the weight set of step kp+1 is passed through the wait as in/out operands: whatever
+    //      uses those registers afterwards is ordered after the wait by the compiler as well.
+    //      (What it does with them *before* the wait is checked on the compiled code: no
+    //      instruction may touch a register with a load in flight, `python -m sten_amd.isa_check`.)
+    //  (3) LDS stage (kp+DD_D) % DD_NS is refilled during step kp; its last readers were the
+    //      fragment reads of step kp+DD_D-DD_NS <= kp-2, complete (lgkmcnt(0), same wait) before
+    //      the barrier that ended that step.  The two fragment sets alternate by phase; NP is
+    //      even, so the set read after the barrier (for phase 0 of the next step) is set 0.
     static_assert(DD_NS > DD_D, "a stage must not be refilled while the step that reads it is in flight");
     auto landed = [&](WSet &w) {
         asm volatile("s_waitcnt vmcnt(%8) lgkmcnt(0)"
@@ -822,26 +471,20 @@ template <typename T, int TB, int NH> static int launch_dense16(DfParams &P, hip
 
 template <typename T> static int launch_dense(DfParams &P, int variant, hipStream_t s)
 {
-    // 256 x 256 tiles move fewer bytes per flop through the vector caches and are 5-6 % faster per
-    // flop in steady state; one workgroup per CU either way, so what decides is how full the last
-    // round of tiles is.  Variants 0 / 1: 256 x 128 / 256 x 256 with the 32 x 32 x 16 instruction,
-    // 5 / 2: the same tiles with the 16 x 16 x 32 instruction, 9-15 % faster (8192^2 4:8 x 4096
-    // tokens: 346 against 405 us; 16384x4096 grad_input: 364 against 400; 4096^2 x 2048: 50 against
-    // 56), which is what the automatic choice takes.  (A sixteen-phase form of the 256 x 256 tile
-    // once gave wrong values now and then; that form is gone, the forms here pass the static check
-    // of their hand-tracked loads and the repeated full-chip test.)
+    // Variant 0: 256 outputs x 128 tokens per workgroup, 1: 256 x 256.  The larger tile moves fewer
+    // bytes per flop through the vector caches and is 5-6 % faster per flop in steady state; one
+    // workgroup per CU either way, so what decides is how full the last round of tiles is.
+    // (A sixteen-phase form of the 256 x 256 tile on the 32 x 32 x 16 instruction once gave wrong
+    // values now and then; the forms here pass the static check of their hand-tracked loads and
+    // the repeated full-chip test.)
     if (variant < 0) {
         const int64_t tm = (P.O + 255) / 256, t256 = tm * ((P.T + 255) / 256), t128 = tm * ((P.T + 127) / 128);
         const double fill256 = (double)t256 / (double)((t256 + 255) / 256 * 256);
         const double fill128 = (double)t128 / (double)((t128 + 255) / 256 * 256);
-        variant = (P.ksplit <= 1 && t256 >= 256 && fill256 * 1.055 >= fill128) ? 3 : 5;
+        variant = (P.ksplit <= 1 && t256 >= 256 && fill256 * 1.055 >= fill128) ? 1 : 0;
     }
-    if (variant == 1) return launch_dense_direct<T, 2, 8, 4, 1, 2>(P, s);
-    if (variant == 2) return launch_dense16<T, 16, 2>(P, s);
-    if (variant == 3) return launch_dense16<T, 16, 4>(P, s);
-    if (variant == 4) return launch_dense16<T, 8, 1>(P, s);
-    if (variant == 5) return launch_dense16<T, 8, 2>(P, s);
-    return launch_dense_direct<T, 2, 4, 4, 1, 1>(P, s);
+    if (variant == 1) return launch_dense16<T, 16, 4>(P, s);
+    return launch_dense16<T, 8, 2>(P, s);
 }
 
 }  // namespace nmg
@@ -921,7 +564,7 @@ extern "C" int nmg_spmm_densefrag(const void *d_df, int64_t O, int64_t K, const 
 {
     NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED, "densefrag takes f16/bf16");
     NMG_REQUIRE(O >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
-    NMG_REQUIRE(variant >= -1 && variant <= 5, NMG_ERR_ARG, "unknown tile variant %d", variant);
+    NMG_REQUIRE(variant >= -1 && variant <= 1, NMG_ERR_ARG, "unknown tile variant %d", variant);
     NMG_REQUIRE(ldx >= K && ldy >= O, NMG_ERR_ARG, "leading dimension smaller than row length");
     NMG_REQUIRE(K % 64 == 0 && K > 0 && ldx % 8 == 0 && ((uintptr_t)d_x % 16) == 0, NMG_ERR_UNSUPPORTED,
                 "needs K %% 64 == 0 and 16-byte aligned activation rows");

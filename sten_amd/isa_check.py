@@ -31,7 +31,7 @@ CSRC = os.path.join(HERE, "csrc")
 # sources whose kernels issue loads as instruction statements, and the kernels (substring of the
 # mangled name) that do
 CHECKED = {
-    "nmg_densefrag.hip": ["dense_direct_kernel", "dense16_direct_kernel"],
+    "nmg_densefrag.hip": ["dense16_direct_kernel"],
     "nmg_smfmac.hip": ["spmm_smfmac_direct_kernel", "decode_staged_kernel"],
     "nmg_w4.hip": ["w4_linear_staged_kernel"],
     "nmg_sddmm.hip": ["sddmm16_kernel"],

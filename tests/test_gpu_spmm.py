@@ -504,7 +504,7 @@ def test_dense_nt_gemm_entry_point(dtype, O_, K, T):
     assert rel_l2(to_np(Y), ref) <= TOL[dtype]
 
 
-@pytest.mark.parametrize("dense_variant", [-1, 0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("dense_variant", [-1, 0, 1])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M,K,T,n,m,g", [
     (256, 64, 128, 2, 4, 16),     # one tile, one K step
@@ -727,7 +727,7 @@ def test_direct_kernels_on_a_full_chip_with_a_long_reduction():
             assert torch.equal(sten.spmm(w, x, reduce_dim=1, kernel="smfmac"), ref), f"variant {variant}"
     g = seeded((T, M), torch.float16, seed=79).to(DEV)
     want = (g @ w.to_dense()).float()
-    for dense_variant in (0, 1, 2, 3, 5):
+    for dense_variant in (0, 1):
         w.spmm_opt["dense_variant"] = dense_variant
         for _ in range(4):
             got = sten.spmm(w, g, reduce_dim=0, kernel="densefrag").float()
