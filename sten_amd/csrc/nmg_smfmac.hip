@@ -61,6 +61,7 @@ struct SmfParams {
     int64_t M, K, T, ldx, ldy;
     int MB, KP;          // feature blocks of 32, k pairs of 64
     int tiles_m, tiles_n;
+    int band;            // direct kernel: line tiles per band of the tile walk (4 or 8)
     // direct kernel with the reduction cut into slices (0 / 1: whole): slice s of a tile writes
     // its sums in single precision to part[s][token][feature], part_ld features per token
     int ksplit;
@@ -321,7 +322,7 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
     const int slice = P.ksplit > 1 ? id / ntiles : 0;
     id -= slice * ntiles;
     if ((ntiles & 7) == 0) id = (id & 7) * (ntiles >> 3) + (id >> 3);
-    constexpr int GH = 4;
+    const int GH = P.band;
     const int band = id / (GH * P.tiles_n);
     const int band_h = min(P.tiles_m - band * GH, GH);
     const int in_band = id - band * GH * P.tiles_n;
@@ -552,7 +553,7 @@ __global__ __launch_bounds__(256, 1) void spmm_smfmac_direct_kernel(SmfParams P)
                 // One memory instruction (or two LDS reads) goes into the shadow of one MFMA: a load
                 // holds the wavefront's issue for about 20 clocks, an LDS read for 7, an MFMA runs 32.
                 // (XT: the transposing reads of a block stay together.)
-                constexpr bool SPLIT = !XT && TB == 8;   // measured: -3..6 % on the 256 x 256 tile, +5 % where two 256 x 128 workgroups share a CU
+                constexpr bool SPLIT = !XT && BT >= 2 && NM >= 4;   // measured in steady state: -3..6 % on the 256 x 256 tile, -1 % on 256 x 128
                 if (PH == NP - 1) {
                     mma(ws[u], fr[PH % 2], ph_tag, 0, 2);
                     __builtin_amdgcn_sched_barrier(0);
@@ -658,6 +659,10 @@ static int launch_smfmac_direct(SmfParams &P, hipStream_t s)
     static_assert(TF == 256, "the operand is padded to 256 lines");
     P.tiles_m = (int)((P.M + TF - 1) / TF);
     P.tiles_n = (int)((P.T + TT - 1) / TT);
+    // An XCD works on 32 consecutive tiles of the walk at a time, a block of `band` line tiles x
+    // 32 / band token tiles, and fetches that block's weights and activations into its L2: the
+    // block is taller where a token tile's activations outweigh a line tile's weights.
+    P.band = (int64_t)TT * 2 * 8 > (int64_t)TF * 9 ? 8 : 4;   // bytes per reduction position: TT * 2 against TF * 9 / 8
     const int slices = P.ksplit > 1 ? P.ksplit : 1;
     dim3 grid((unsigned)(P.tiles_m * P.tiles_n * slices));
     constexpr size_t ring = (size_t)DR_NS * TT * 128;
@@ -1183,7 +1188,7 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
     case 8:                                                     // 256 x 256
         if (P.K % 64 != 0 || P.T * P.ldx * 2 >= (int64_t)1 << 31)
             return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
-        if (variant == 8) return launch_smfmac_direct<T, 2, 8, 4, 1, 2>(P, s);
+        if (variant == 8) return launch_smfmac_direct<T, 2, 8, 4, 1, 4>(P, s);
         return launch_smfmac_direct<T, 2, 4, 4, 1, 2>(P, s);
     }
     return NMG_ERR_ARG;
