@@ -185,6 +185,56 @@ def matrix_ceiling(iters=4000):
     return res
 
 
+MIX_KINDS = [
+    "dense 256x256, V_MFMA_F32_32X32X16: MFMAs alone", "dense 256x256, 32X32X16: + LDS reads",
+    "dense 256x256, 32X32X16: + LDS reads, weight loads, DMA loads",
+    "dense 256x256, V_MFMA_F32_16X16X32: MFMAs alone", "dense 256x256, 16X16X32: + LDS reads",
+    "dense 256x256, 16X16X32: + LDS reads, weight loads, DMA loads",
+    "dense 256x256, 32X32X16, eight wavefronts: everything", "dense 256x256, 16X16X32, eight wavefronts: everything",
+    "sparse 256x256, V_SMFMAC_F32_32X32X32: everything", "sparse 256x256, V_SMFMAC_F32_16X16X64: everything",
+    "sparse 256x128, 32X32X32: MFMAs alone", "sparse 256x128, 32X32X32: + LDS reads",
+    "sparse 256x128, 32X32X32: + LDS reads, weight loads, DMA loads", "sparse 256x128, 32X32X32: without the DMA loads",
+    "sparse 256x128, 32X32X32: without the weight loads", "sparse 256x128, 32X32X32: without the index loads",
+    "sparse 256x128, 32X32X32: wavefronts 2 x 2", "sparse 256x128, 16X16X64: MFMAs alone",
+    "sparse 256x128, 16X16X64: + LDS reads, weight loads, DMA loads",
+    "sparse 256x256, 32X32X32: MFMAs alone", "sparse 256x256, 16X16X64: MFMAs alone",
+]
+
+
+def instruction_mix(steps=2048):
+    """What a K step of the large-batch kernels costs beyond its matrix instructions
+    (nmg_probe_instruction_mix: the step's instruction mix on L2-resident N(0,1) data, parts of it
+    left out, the instruction exchanged).  TFLOP/s over the chip, dense-equivalent."""
+    import torch
+    from sten_amd import native
+
+    lib = native.load()
+    dev = "cuda:0"
+    torch.manual_seed(0)
+    data = torch.randn(8 * 1024 * 1024, device=dev).half()
+    out = torch.empty(256 * 512, dtype=torch.float32, device=dev)
+    stream = native.stream_ptr(out.device)
+    res = {}
+    for kind, name in enumerate(MIX_KINDS):
+        flops = lib.nmg_probe_instruction_mix_flops(kind, steps)
+
+        def launch():
+            native.check(lib.nmg_probe_instruction_mix(kind, native.ptr(data), data.numel() * 2, native.ptr(out),
+                                                       out.numel(), steps, stream))
+        settle_end = time.perf_counter() + SETTLE_S
+        while time.perf_counter() < settle_end:
+            launch()
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(5):
+            launch()
+        e1.record()
+        torch.cuda.synchronize()
+        res[name] = round(flops / (e0.elapsed_time(e1) / 5 * 1e-3) / 1e12, 1)
+    return res
+
+
 def calibrate_copy():
     import torch
     n = 64 * 1024 * 1024
@@ -377,6 +427,8 @@ def main():
     ap.add_argument("--matrix-ceiling", action="store_true",
                     help="only measure what the matrix cores sustain from registers, per instruction")
     ap.add_argument("--no-ceiling", action="store_true", help="skip that measurement in the default run")
+    ap.add_argument("--instruction-mix", action="store_true",
+                    help="only measure what a K step of the large-batch kernels costs beyond its MFMAs")
     ap.add_argument("--copies", type=int, default=0,
                     help="decode shapes: separate copies of the weight that the steps take in turn "
                          "(0: as many as exceed 512 MiB, so that no step finds its weight in a cache)")
@@ -389,6 +441,9 @@ def main():
         return
     if args.matrix_ceiling:
         print(json.dumps({"matrix_ceiling_tflops": matrix_ceiling()}))
+        return
+    if args.instruction_mix:
+        print(json.dumps({"instruction_mix_tflops": instruction_mix()}, indent=1))
         return
 
     row = measure(args.workload, args.steps, args.warmup, args.kernel, args.variant, args.eager, args.graph,

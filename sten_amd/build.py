@@ -7,7 +7,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libnmg_hip.so")
 SOURCES = ["nmg_runtime.hip", "nmg_sparsify.hip", "nmg_spmm.hip", "nmg_smfmac.hip", "nmg_dense.hip",
-           "nmg_densefrag.hip", "nmg_w4.hip", "nmg_pack.hip", "nmg_sddmm.hip", "nmg_perfect.hip", "nmg_probe.hip"]
+           "nmg_densefrag.hip", "nmg_w4.hip", "nmg_pack.hip", "nmg_sddmm.hip", "nmg_perfect.hip", "nmg_probe.hip",
+           "nmg_probe_mix.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

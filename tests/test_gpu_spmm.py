@@ -747,3 +747,23 @@ def test_matrix_rate_probe_runs_every_instruction():
     assert bool(torch.isfinite(out).all())
     assert lib.nmg_probe_matrix_rate(7, native.ptr(src), native.ptr(out), 10, None) == 1
     assert lib.nmg_probe_matrix_rate_flops(7, 10) == -1
+
+
+def test_instruction_mix_probe_runs_every_kind():
+    # measurement aid of bench.py: launches and finishes for every kind, refuses bad arguments
+    lib = native.load()
+    data = torch.randn(8 * 1024 * 1024, device=DEV).half()
+    out = torch.empty(256 * 512, dtype=torch.float32, device=DEV)
+    for kind in range(21):
+        print(f"case instruction mix {kind}", flush=True)
+        tok = 128 if 10 <= kind <= 18 else 256
+        assert lib.nmg_probe_instruction_mix_flops(kind, 4) == 2 * 256 * tok * 64 * 4 * 256
+        native.check(lib.nmg_probe_instruction_mix(kind, native.ptr(data), data.numel() * 2, native.ptr(out),
+                                                   out.numel(), 4, None))
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())
+    args = (native.ptr(data), data.numel() * 2, native.ptr(out), out.numel())
+    assert lib.nmg_probe_instruction_mix(21, *args, 4, None) == 1          # unknown kind
+    assert lib.nmg_probe_instruction_mix(0, *args, 3, None) == 1           # odd step count
+    assert lib.nmg_probe_instruction_mix(0, native.ptr(data), 1 << 20, native.ptr(out), out.numel(), 4, None) == 1
+    assert lib.nmg_probe_instruction_mix_flops(21, 4) == -1
