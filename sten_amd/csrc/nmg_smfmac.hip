@@ -811,15 +811,16 @@ template <typename T, int NW, int UN> static int launch_smfmac_skinny(SmfParams 
 // A weight of few blocks (4096 lines: 128) would leave half of the CUs without a workgroup:
 // SPLIT workgroups share a block, each fetches the runs of its 32 / SPLIT lines of every
 // fragment and multiplies zeros in the other lanes -- no sum across workgroups is needed.
-template <typename T, int SK_NW, int ND, int SPLIT>
+template <typename T, int SK_NW, int ND, int SPLIT, int TK = 16>
 __global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_decode_staged_kernel(SmfParams P)
 {
     using S = Smf<T>;
     constexpr int OPS = ND + 6;
     constexpr int LPB = 32 / SPLIT;                     // lines of the block that this workgroup owns
-    constexpr int BUF = 16 * 256;                       // one chunk: 16 token rows x 256 bytes
+    constexpr int BUF = TK * 256;                       // one chunk: TK (16 or 32) token rows x 256 bytes
+    static_assert((TK == 16 || TK == 32) && ND * 4 <= TK, "four token rows per DMA load");
     extern __shared__ __align__(16) unsigned char smem[];
-    static_assert(SK_NW * 2 * BUF >= SK_NW * 32 * 17 * 4, "the reduction buffer reuses the staging area");
+    static_assert(SK_NW * 2 * BUF >= SK_NW * 32 * (TK + 1) * 4, "the reduction buffer reuses the staging area");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int mb = blockIdx.x / SPLIT, part = blockIdx.x % SPLIT;
@@ -859,7 +860,7 @@ __global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_decode_staged_kernel(S
         for (int ks = 0; ks < 2; ks++)
 #pragma unroll
             for (int c = 0; c < 2; c++)
-                b_off[kl][ks][c] = (j & 15) * 256 + (((kl * 8 + ks * 4 + 2 * h + c) ^ (j & 15)) << 4);
+                b_off[kl][ks][c] = (j & (TK - 1)) * 256 + (((kl * 8 + ks * 4 + 2 * h + c) ^ (j & 15)) << 4);
 
     struct ASet {
         u32x4 a[2][2];
@@ -946,14 +947,14 @@ __global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_decode_staged_kernel(S
                  :
                  : "memory");
     __syncthreads();   // every wavefront is done with its staging area: reuse it for the reduction
-    float(*red)[32][17] = (float(*)[32][17])smem;
+    float(*red)[32][TK + 1] = (float(*)[32][TK + 1])smem;
     // D[row = line][col = token]: lane holds token j, lines 8*(r/4) + 4*h + r%4
-    if (j < 16) {
+    if (j < TK) {
 #pragma unroll
         for (int r = 0; r < 16; r++) red[wave][(r >> 2) * 8 + h * 4 + (r & 3)][j] = acc[r];
     }
     __syncthreads();
-    for (int e = tid; e < LPB * 16; e += 64 * SK_NW) {
+    for (int e = tid; e < LPB * TK; e += 64 * SK_NW) {
         const int line = part * LPB + (e & (LPB - 1)), tok = e / LPB;
         const int64_t f = (int64_t)mb * 32 + line;
         if (tok >= P.T || f >= P.M) continue;
@@ -965,12 +966,13 @@ __global__ __launch_bounds__(64 * SK_NW) void spmm_smfmac_decode_staged_kernel(S
     }
 }
 
-template <typename T, int NW, int ND, int SPLIT>
+template <typename T, int NW, int ND, int SPLIT, int TK = 16>
 static int launch_smfmac_decode_staged(SmfParams &P, hipStream_t s)
 {
     dim3 grid((unsigned)((P.M + 31) / 32 * SPLIT));
-    const size_t lds = (size_t)NW * 2 * 16 * 256;
-    auto k = spmm_smfmac_decode_staged_kernel<T, NW, ND, SPLIT>;
+    constexpr size_t lds = (size_t)NW * 2 * TK * 256;
+    if (lds > 160 * 1024) return NMG_ERR_UNSUPPORTED;   // (16 wavefronts x 32 token rows: not dispatched)
+    auto k = spmm_smfmac_decode_staged_kernel<T, NW, ND, SPLIT, TK>;
     if (lds > 64 * 1024)
         NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(k, grid, dim3(64 * NW), lds, s, P);
@@ -985,7 +987,12 @@ static int launch_smfmac_decode_staged_nd(SmfParams &P, hipStream_t s)
     case 1: return launch_smfmac_decode_staged<T, NW, 1, SPLIT>(P, s);
     case 2: return launch_smfmac_decode_staged<T, NW, 2, SPLIT>(P, s);
     case 3: return launch_smfmac_decode_staged<T, NW, 3, SPLIT>(P, s);
-    default: return launch_smfmac_decode_staged<T, NW, 4, SPLIT>(P, s);
+    case 4: return launch_smfmac_decode_staged<T, NW, 4, SPLIT>(P, s);
+    // 17 .. 32 tokens: the second half of the instruction's 32 token columns is used too
+    case 5: return launch_smfmac_decode_staged<T, NW, 5, SPLIT, 32>(P, s);
+    case 6: return launch_smfmac_decode_staged<T, NW, 6, SPLIT, 32>(P, s);
+    case 7: return launch_smfmac_decode_staged<T, NW, 7, SPLIT, 32>(P, s);
+    default: return launch_smfmac_decode_staged<T, NW, 8, SPLIT, 32>(P, s);
     }
 }
 
@@ -1167,8 +1174,9 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
     }
     switch (variant) {
     case 0: return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);  // register-prefetch kernel, 256 lines x 128 tokens: any K
-    case 5:                                                     // decode shapes, T <= 16
-        if (P.T > 16) return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
+    case 5:                                                     // decode shapes, T <= 16 (staged form: <= 32)
+        if (P.T > 32 || (P.T > 16 && !(P.K % 128 == 0 && P.T * P.ldx * 2 < ((int64_t)1 << 31))))
+            return launch_smfmac_cfg<T, 2, 2, 4, 2, 1>(P, s);
         // few line blocks: many wavefronts per workgroup keep enough loads in flight per CU;
         // many line blocks: small workgroups pack several per CU and balance better
         // reduction extents that are a multiple of 128: activations staged through LDS
@@ -1179,7 +1187,7 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
             // (344 blocks): one of 4 wavefronts 11.6 / 14.0, two of 4 12.1 / 16.2.
             const int64_t blocks = (P.M + 31) / 32;
             if (blocks >= 256) return launch_smfmac_decode_staged_nd<T, 4, 1>(P, s);
-            if (blocks >= 64) return launch_smfmac_decode_staged_nd<T, 8, 2>(P, s);
+            if (blocks >= 64 || P.T > 16) return launch_smfmac_decode_staged_nd<T, 8, 2>(P, s);   // (32 token rows: 16 wavefronts would not fit LDS)
             return launch_smfmac_decode_staged_nd<T, 16, 2>(P, s);
         }
         if ((P.M + 31) / 32 >= 256) return launch_smfmac_skinny<T, 4, 4>(P, s);

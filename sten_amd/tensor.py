@@ -428,6 +428,12 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
     if packed is not None:
         if T <= 16 and kname in ("auto", "skinny"):
             variant = 5                 # decode shapes: streaming kernel on the same operand
+        elif (T <= 24 and kname == "auto" and variant == -1 and K % 128 == 0
+              and T * x.stride(0) * 2 < 2 ** 31 and "slices" not in weight.spmm_opt):
+            # 17 .. 24 tokens: the streaming kernel with the second half of its 32 token columns in
+            # use is still ahead of the sliced reduction (4096 x 11008: 15.8 / 17.9 against 18.2 /
+            # 18.7 us at 17 / 24 tokens; at 32 tokens 20.1 against 19.3)
+            variant = 5
         lib = native.load()
         if T > 16 and variant == -1 and K % 64 == 0 and T * x.stride(0) * 2 < 2 ** 31:
             # few tiles for the chip: the reduction is cut into slices, summed by a second kernel

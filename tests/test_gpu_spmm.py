@@ -314,6 +314,34 @@ def test_split_reduction_on_the_target_weight_at_intermediate_batches():
         assert rel_l2(to_np(y), to_np(x.double() @ Wd.t())) <= TOL[torch.float16]
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,K,n,m,g", [
+    (4096, 1024, 2, 4, 16),     # 128 blocks of 32 lines: two workgroups per block
+    (300, 640, 1, 4, 4),        # ragged lines, few blocks
+    (11008, 512, 2, 4, 16),     # 344 blocks: one workgroup per block
+])
+def test_streaming_kernel_with_17_to_32_tokens(dtype, M, K, n, m, g):
+    # the decode kernel with the second half of its 32 token columns in use; every count from 17 to
+    # 32 (4 token rows per DMA load: 5 .. 8 loads per chunk), with a bias, against the fp64 product
+    print(f"case wide decode {dtype} M={M} K={K} {n}:{m}:{g}", flush=True)
+    W = seeded((M, K), dtype, seed=M + K, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, 1)
+    w = make(W, n, m, g, 1)
+    b = seeded((M,), dtype, seed=5)
+    for T in range(17, 33):
+        x = seeded((T, K), dtype, seed=T)
+        ref = to_np(x).astype(np.float64) @ Wd.T + to_np(b).astype(np.float64)
+        w.spmm_opt["variant"] = 5
+        y = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)
+        assert y.shape == (T, M)
+        assert rel_l2(to_np(y), ref) <= TOL[dtype], T
+        w.spmm_opt.pop("variant")
+        y2 = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)      # automatic choice (<= 24: the same kernel)
+        assert rel_l2(to_np(y2), ref) <= TOL[dtype], T
+        if T <= 24:
+            assert torch.equal(y, y2), T
+
+
 def test_target_weight_against_the_oracle_at_decode_and_large_batches():
     # the north-star weight 4096 x 11008 2:4:16 compressed by the CPU oracle (val / idx compared
     # bit for bit), then the product at 1 and 16 tokens (decode kernel) and 2048 tokens (direct
