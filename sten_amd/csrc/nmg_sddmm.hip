@@ -742,8 +742,20 @@ static int sddmm_impl(bool nt, const void *d_lines, int64_t ld_lines, const void
     };
     auto launch_t = [&](auto tag) -> int {
         using T = decltype(tag);
-        if (nt) {   // reduction-contiguous operands: 2:4 in registers, every other pattern through the staged tile
-            if (in_regs && n == 2 && S % 4 == 0) return launch(sddmm16_kernel<T, 2, true>);   // (no padded positions)
+        if (nt) {   // reduction-contiguous operands; the epilogues in registers need every block of m positions whole
+            if (in_regs && S % 4 == 0) {
+                switch (n) {
+                case 1: return launch(sddmm16_kernel<T, 1, true>);
+                case 2: return launch(sddmm16_kernel<T, 2, true>);
+                case 3: return launch(sddmm16_kernel<T, 3, true>);
+                default: return launch(sddmm16_kernel<T, 4, true>);
+                }
+            }
+            if (in_regs8 && S % 8 == 0) {
+                if (n == 1) return launch(sddmm16_kernel<T, 9, true>);
+                if (n == 2) return launch(sddmm16_kernel<T, 10, true>);
+                return launch(sddmm16_kernel<T, 12, true>);
+            }
             return launch(sddmm16_kernel<T, 0, true>);
         }
         if (in_regs8) {

@@ -176,6 +176,12 @@ def test_training_step_uses_the_fused_kernel():
     (264, 776, 136, 4, 8, 2, 0),
     (96, 528, 200, 3, 6, 2, 1),
     (768, 1024, 160, 2, 4, 1, 1),
+    (256, 512, 72, 1, 4, 8, 1),          # the other epilogues in registers: m = 4 with n = 1, 3, 4 ...
+    (512, 264, 96, 3, 4, 2, 0),
+    (264, 256, 40, 4, 4, 4, 1),
+    (512, 512, 136, 1, 8, 32, 1),        # ... and m = 8 with n = 1, 2, 4
+    (896, 264, 64, 2, 8, 32, 0),
+    (280, 512, 48, 4, 8, 4, 1),
 ])
 def test_masked_product_reduction_contiguous_operands(dtype, R, C, T, n, m, g, sd):
     # operands given as [R, T] and [C, T] (the weight gradient of torch.mm(W, B)): same values as
