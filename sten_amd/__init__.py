@@ -16,7 +16,7 @@ from .layout import NMGLayout
 from .native import NmgError
 from . import perfect
 from .perfect import PerfectNMSparsifier, PerfectNMTensor, is_correct_nm
-from .tensor import GroupedNMTensor, spmm, spmm_tt
+from .tensor import GroupedNMTensor, spmm, spmm_tt, spmm_tt_dense
 from . import w4
 from .w4 import SparseMarlinSparsifier, SparseMarlinTensor
 

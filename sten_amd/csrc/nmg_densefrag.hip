@@ -185,6 +185,11 @@ constexpr int DD_NS = 4;   // activation stages in LDS (>= DD_D + 1)
 // them in the accumulation registers.  A K step of 64 is two k-steps of 32; a phase is one
 // (k-step, token part) pair of 4 * TB / NH MFMAs: they run while the activation fragments of the
 // next phase are read from LDS, and the loads of K step kp+DD_D are dealt out over the phases.
+// XT = true is the product with both dense operands transposed, C[O, T] = A * B for B [K, T] (the
+// gradient with respect to B of torch.mm(W, B): W^T * grad_out as they lie in memory): the
+// activation tile of a K step is then 64 reduction rows x TT tokens, fetched as it lies, an
+// activation fragment is two LDS transpose reads (DS_READ_B64_TR_B16), and the epilogue stages
+// [output][token] and stores token-contiguous rows.
 template <typename T> struct DfMma16;
 template <> struct DfMma16<__half> {
     using F = df_f16x8;
@@ -195,7 +200,7 @@ template <> struct DfMma16<__hip_bfloat16> {
     __device__ static f32x4 run(F a, F b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
 };
 
-template <typename T, int TB, int NH>
+template <typename T, int TB, int NH, bool XT = false>
 __global__ __launch_bounds__(256, 1) void dense16_direct_kernel(DfParams P)
 {
     using Mm = DfMma16<T>;
@@ -243,16 +248,31 @@ __global__ __launch_bounds__(256, 1) void dense16_direct_kernel(DfParams P)
         av_base[o] = (const unsigned char *)P.df + (((int64_t)(ob0 + o) * KPT + kp_lo) * 4) * 1024;
     const int r16 = lane & 15, kq = lane >> 4;
     const uint32_t lane_a = (uint32_t)((kq >> 1) * 1024 + ((kq & 1) * 32 + r16) * 16);
-    const unsigned char *x_base = (const unsigned char *)P.x + (int64_t)kp_lo * 128;
+    // K step kp of the activations starts kp * XSTEP bytes into the operand
+    const int64_t XSTEP = XT ? 64 * P.ldx * 2 : 128;
+    const unsigned char *x_base = (const unsigned char *)P.x + (int64_t)kp_lo * XSTEP;
     uint32_t x_off[XL];
 #pragma unroll
     for (int i = 0; i < XL; i++) {
-        const int row = (wave * XL + i) * 8 + (lane >> 3);
-        const int piece = lane & 7;
-        const int q = piece ^ ((row >> 1) & 7);   // logical 16-byte chunk stored at this piece
-        int64_t tok = t0 + row;
-        if (tok >= P.T) tok = P.T - 1;            // clamped rows are computed, never stored
-        x_off[i] = (uint32_t)((tok * P.ldx + q * 8) * 2);
+        if constexpr (XT) {
+            // a DMA load fills 1 KiB = 1024 / (TT * 2) reduction rows of the tile; piece p (8 tokens)
+            // of row k holds the logical chunk p ^ (4*(k%4) + 2*((k/8)%2)): the 32 lanes of a
+            // transpose read that are served together take rows k .. k+3 and k+8 .. k+11 of one
+            // 16-token block, which then fall into 16 different pieces = every bank once
+            constexpr int PPR = TT / 8;                       // 16-byte pieces per row
+            const int row = (wave * XL + i) * (64 / PPR) + lane / PPR;
+            const int chunk = (lane % PPR) ^ (((row & 3) << 2) | (((row >> 3) & 1) << 1));
+            int64_t tok = t0 + chunk * 8;
+            if (tok > P.T - 8) tok = (P.T - 1) / 8 * 8;       // clamped columns are computed, never stored
+            x_off[i] = (uint32_t)((row * P.ldx + tok) * 2);
+        } else {
+            const int row = (wave * XL + i) * 8 + (lane >> 3);
+            const int piece = lane & 7;
+            const int q = piece ^ ((row >> 1) & 7);   // logical 16-byte chunk stored at this piece
+            int64_t tok = t0 + row;
+            if (tok >= P.T) tok = P.T - 1;            // clamped rows are computed, never stored
+            x_off[i] = (uint32_t)((tok * P.ldx + q * 8) * 2);
+        }
     }
 
     struct WSet {
@@ -266,7 +286,7 @@ __global__ __launch_bounds__(256, 1) void dense16_direct_kernel(DfParams P)
         if (kp >= KP) kp = KP - 1;
         if (i < XL) {
             unsigned char *base = smem + (kp & (DD_NS - 1)) * STAGE;
-            const unsigned char *xb = x_base + (int64_t)kp * 128;
+            const unsigned char *xb = x_base + (int64_t)kp * XSTEP;
 #pragma unroll
             for (int q = 0; q < XL; q++)
                 if (q == i)
@@ -311,9 +331,35 @@ __global__ __launch_bounds__(256, 1) void dense16_direct_kernel(DfParams P)
         u32x4 b[BT];
     };
     BFrags fr[2];
+    // XT: lane (kq, i) of a transpose read supplies the 8 bytes at reduction row 8 kq + i/4 (+ 32 k32
+    // + 4 r), tokens 4 (i%4) .. +3 of the 16-token block, and receives token i at rows
+    // 8 kq + 4 r + 0..3: reads r = 0, 1 are the lane's 8 reduction positions.
+    int t_off[XT ? TB : 1];
+    if constexpr (XT) {
+        const int a = r16 >> 2;
+#pragma unroll
+        for (int tb = 0; tb < TB; tb++) {
+            const int chunk = tb * 2 + ((r16 & 3) >> 1);   // 8-token chunk of the row
+            t_off[tb] = (8 * kq + a) * (TT * 2) + ((chunk ^ ((a << 2) | ((kq & 1) << 1))) << 4) + (r16 & 1) * 8;
+        }
+    }
     auto read_one = [&](BFrags &f, const unsigned char *base, int ph, int t) {
         const int k32 = ph / NH, hh = ph % NH;
-        f.b[t] = *(const u32x4 *)(base + b_off[k32] + (hh * BT + t) * 16 * 128);
+        if constexpr (XT) {
+            typedef short i16x4 __attribute__((ext_vector_type(4)));
+            typedef __attribute__((address_space(3))) i16x4 *lds_i16x4;
+            union {
+                i16x4 h[2];
+                u32x4 u;
+            } c;
+#pragma unroll
+            for (int r = 0; r < 2; r++)
+                c.h[r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_i16x4)(base + t_off[hh * BT + t] + (32 * k32 + 4 * r) * (TT * 2)));
+            f.b[t] = c.u;
+        } else {
+            f.b[t] = *(const u32x4 *)(base + b_off[k32] + (hh * BT + t) * 16 * 128);
+        }
     };
     // MFMA number i of phase PH (i = ab * BT + t)
     auto mma = [&](const WSet &w, const BFrags &f, auto ph_tag, int i) {
@@ -445,20 +491,24 @@ __global__ __launch_bounds__(256, 1) void dense16_direct_kernel(DfParams P)
         return;
     }
     const TileOut out{P.y, P.bias, P.O, P.T, P.ldy};
-    store_tile16<T, AB, TB>(acc, smem + wave * (TT * (AB * 32 + 16)), lane, f0 + wave * 64, t0, out);
+    if constexpr (XT)
+        store_tile16_t<T, AB, TB>(acc, smem + wave * (AB * 16 * (TT * 2 + 16)), lane, f0 + wave * 64, t0, out);
+    else
+        store_tile16<T, AB, TB>(acc, smem + wave * (TT * (AB * 32 + 16)), lane, f0 + wave * 64, t0, out);
 }
 
-template <typename T, int TB, int NH> static int launch_dense16(DfParams &P, hipStream_t s)
+template <typename T, int TB, int NH, bool XT = false> static int launch_dense16(DfParams &P, hipStream_t s)
 {
     constexpr int TT = TB * 16;
     P.tiles_m = (int)((P.O + 255) / 256);
     P.tiles_n = (int)((P.T + TT - 1) / TT);
     const int slices = P.ksplit > 1 ? P.ksplit : 1;
     dim3 grid((unsigned)(P.tiles_m * P.tiles_n * slices));
-    constexpr size_t ring = (size_t)DD_NS * TT * 128, stg = (size_t)4 * TT * (4 * 32 + 16);
+    constexpr size_t ring = (size_t)DD_NS * TT * 128;
+    constexpr size_t stg = XT ? (size_t)4 * 64 * (TT * 2 + 16) : (size_t)4 * TT * (4 * 32 + 16);
     constexpr size_t lds = ring > stg ? ring : stg;
     static_assert(lds <= 160 * 1024, "LDS");
-    auto k = dense16_direct_kernel<T, TB, NH>;
+    auto k = dense16_direct_kernel<T, TB, NH, XT>;
     NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(k, grid, dim3(256), lds, s, P);
     NMG_HIP_TRY(hipGetLastError());
@@ -584,6 +634,35 @@ extern "C" int nmg_spmm_densefrag(const void *d_df, int64_t O, int64_t K, const 
     P.KP = (int)(K / 64);
     hipStream_t s = (hipStream_t)stream;
     return dtype == NMG_F16 ? launch_dense<__half>(P, variant, s) : launch_dense<__hip_bfloat16>(P, variant, s);
+}
+
+extern "C" int nmg_spmm_densefrag_tt(const void *d_df, int64_t O, int64_t K, const void *d_b, int64_t ldb, void *d_c,
+                                     int64_t ldc, const void *d_bias, int64_t T, int dtype, void *stream)
+{
+    NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED, "densefrag takes f16/bf16");
+    NMG_REQUIRE(O >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
+    NMG_REQUIRE(ldb >= T && ldc >= T, NMG_ERR_ARG, "leading dimension smaller than row length");
+    NMG_REQUIRE(K % 64 == 0 && K > 0 && ldb % 8 == 0 && ((uintptr_t)d_b % 16) == 0, NMG_ERR_UNSUPPORTED,
+                "the transposed product needs K %% 64 == 0, ldb %% 8 == 0 and a 16-byte aligned B");
+    NMG_REQUIRE(ldb < ((int64_t)1 << 24), NMG_ERR_UNSUPPORTED, "leading dimension too large");
+    if (O == 0 || T == 0) return NMG_OK;
+    NMG_REQUIRE(d_df && d_b && d_c, NMG_ERR_ARG, "null device pointer");
+    DfParams P{};
+    P.df = d_df;
+    P.x = d_b;
+    P.y = d_c;
+    P.bias = d_bias;
+    P.O = O;
+    P.K = K;
+    P.T = T;
+    P.ldx = ldb;
+    P.ldy = ldc;
+    P.KP = (int)(K / 64);
+    hipStream_t s = (hipStream_t)stream;
+    // 256 x 128 tiles only: the fragments of this form are LDS transpose reads, 8 bytes per lane, and
+    // the 256 x 256 tile, which doubles them per wavefront, measured slower (16384x4096 x 4096
+    // columns: 724 against 582 us; the plain product on a transposed copy: 360 + 60 for the copy).
+    return dtype == NMG_F16 ? launch_dense16<__half, 8, 2, true>(P, s) : launch_dense16<__hip_bfloat16, 8, 2, true>(P, s);
 }
 
 extern "C" int nmg_spmm_densefrag_splitk(const void *d_df, int64_t O, int64_t K, const void *d_x, int64_t ldx,

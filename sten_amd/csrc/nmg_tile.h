@@ -132,32 +132,23 @@ __device__ __forceinline__ void store_tile16(const f32x4 (&acc)[AB][TB], unsigne
 // wavefront's FB*32 features x TB*32 tokens are staged as [feature][token], so that a lane stores
 // 16 bytes = 8 tokens of one feature row and TB*64 bytes per row are contiguous.  The bias of a
 // feature is added to its whole row.
-template <typename T, int FB, int TB>
-__device__ __forceinline__ void smf_store_tile_t(const f32x16 (&acc)[FB][TB], unsigned char *stg, int lane,
-                                                 int64_t fw, int64_t tw, const TileOut &P)
+// Second half of the transposed epilogues: NROWS output rows of TB*64 B (+16 B pad) lie in `stg`
+// as [output][token]; a lane moves 16 bytes = 8 tokens of one output row per pass.  The bias of an
+// output is added to its whole row.
+template <typename T, int TB, int NROWS>
+__device__ __forceinline__ void store_staged_rows_t(const unsigned char *stg, int lane, int64_t fw, int64_t tw,
+                                                    const TileOut &P)
 {
     constexpr int ROW = TB * 64 + 16;       // bytes per staged feature row
     constexpr int CPR = TB * 4;             // 16-byte chunks per row
     constexpr int RPP = 64 / CPR;           // feature rows per pass of the wavefront
-    const int j = lane & 31, h = lane >> 5;
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-    for (int tb = 0; tb < TB; tb++)
-#pragma unroll
-        for (int fb = 0; fb < FB; fb++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int f = fb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                *(uint16_t *)(stg + f * ROW + (tb * 32 + j) * 2) = f32_to_bits16(acc[fb][tb][r], (T *)nullptr);
-            }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     uint16_t *Y = (uint16_t *)P.y;
     const T *bias = (const T *)P.bias;
     const bool vec_ok = (P.ldy & 7) == 0 && ((uintptr_t)P.y & 15) == 0;
     const int tc = lane % CPR;                      // 8-token chunk of the row
     const int64_t tok = tw + tc * 8;
 #pragma unroll 4
-    for (int it = 0; it < FB * 32 / RPP; it++) {
+    for (int it = 0; it < NROWS / RPP; it++) {
         const int fl = it * RPP + lane / CPR;
         const int64_t f = fw + fl;
         u32x4 v = *(const u32x4 *)(stg + fl * ROW + tc * 16);
@@ -185,6 +176,48 @@ __device__ __forceinline__ void smf_store_tile_t(const f32x16 (&acc)[FB][TB], un
                 if (tok + i < P.T) dst[i] = (uint16_t)(w[i >> 1] >> ((i & 1) * 16));
         }
     }
+}
+
+template <typename T, int FB, int TB>
+__device__ __forceinline__ void smf_store_tile_t(const f32x16 (&acc)[FB][TB], unsigned char *stg, int lane,
+                                                 int64_t fw, int64_t tw, const TileOut &P)
+{
+    constexpr int ROW = TB * 64 + 16;       // bytes per staged feature row
+    const int j = lane & 31, h = lane >> 5;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int tb = 0; tb < TB; tb++)
+#pragma unroll
+        for (int fb = 0; fb < FB; fb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int f = fb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                *(uint16_t *)(stg + f * ROW + (tb * 32 + j) * 2) = f32_to_bits16(acc[fb][tb][r], (T *)nullptr);
+            }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    store_staged_rows_t<T, TB, FB * 32>(stg, lane, fw, tw, P);
+}
+
+// The 16 x 16 form, transposed output: AB blocks of 16 outputs x TB16 blocks of 16 tokens (an even
+// number) per wavefront, staged as [output][token].
+template <typename T, int AB, int TB16>
+__device__ __forceinline__ void store_tile16_t(const f32x4 (&acc)[AB][TB16], unsigned char *stg, int lane,
+                                               int64_t fw, int64_t tw, const TileOut &P)
+{
+    static_assert(TB16 % 2 == 0, "whole 32-token pieces of a staged row");
+    constexpr int ROW = TB16 * 32 + 16;
+    const int j = lane & 15, q = lane >> 4;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int tb = 0; tb < TB16; tb++)
+#pragma unroll
+        for (int ab = 0; ab < AB; ab++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                *(uint16_t *)(stg + (ab * 16 + q * 4 + r) * ROW + (tb * 16 + j) * 2) =
+                    f32_to_bits16(acc[ab][tb][r], (T *)nullptr);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    store_staged_rows_t<T, TB16 / 2, AB * 16>(stg, lane, fw, tw, P);
 }
 
 // ---- reductions cut into slices (products with fewer tiles than the GPU has CUs) ----

@@ -8,7 +8,7 @@ functions: this package's own ``dispatch`` module, or a real ``sten``.
 """
 import torch
 
-from .tensor import GroupedNMTensor, spmm, spmm_tt
+from .tensor import GroupedNMTensor, spmm, spmm_tt, spmm_tt_dense
 
 
 class GroupedNMSparsifier:
@@ -124,7 +124,7 @@ def install(api):
         [gc] = grad_outputs
         w = weight.wrapped_tensor
         gc = gc.to(w.dtype)
-        gb = spmm(w, gc.t().contiguous(), reduce_dim=0).t()
+        gb = spmm_tt_dense(w, gc, reduce_dim=0)     # W^T @ grad_out, both as they lie in memory
         if compressed:
             # grad_out [R, N] and B [C, N] are reduction-contiguous as they lie: no transposing copies
             if w.masked_product_supported(gc, b, reduction_last=True):

@@ -54,6 +54,7 @@ SIGNATURES = {
     "nmg_densefrag": (_I, [_P, _P, _I64, _I64, _I, _P, _I, _I, _I, _P]),
     "nmg_spmm_densefrag": (_I, [_P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _P]),
     "nmg_spmm_densefrag_splitk": (_I, [_P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _P, _I64, _P]),
+    "nmg_spmm_densefrag_tt": (_I, [_P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _P]),
     "nmg_w4_sizes": (_I, [_I64, _I64] + [ctypes.POINTER(ctypes.c_int64)] * 3),
     "nmg_w4_pack": (_I, [_P, _I64, _I64, _I64, _P, _P, _P, _P]),
     "nmg_w4_to_dense": (_I, [_P, _P, _P, _I64, _I64, _P, _I64, _P]),

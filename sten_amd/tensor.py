@@ -391,6 +391,40 @@ def spmm_tt(weight, b):
     return c
 
 
+def spmm_tt_dense(weight, b, *, reduce_dim):
+    """C = op(W) @ B with both dense operands as they lie in memory, on the dense matrix cores:
+    ``reduce_dim=0``: B is [R, N], C = W^T @ B is [C, N] (the gradient with respect to B of
+    ``torch.mm(W, B)``); ``reduce_dim=1``: B is [C, N], C = W @ B is [R, N].  Needs 16-bit data, a
+    power-of-two m, a reduction extent that is a multiple of 64, more than 16 columns and a B that is
+    row-contiguous with a row pitch that is a multiple of 8; otherwise through ``spmm`` on the
+    transposed operands."""
+    lay = weight.layout
+    native.require_gpu(b, weight.val)
+    K, O = lay.dense_shape[reduce_dim], lay.dense_shape[1 - reduce_dim]
+    if b.dim() != 2 or b.shape[0] != K:
+        raise native.NmgError(f"B must be [{K}, N], got {tuple(b.shape)}")
+    if b.dtype != weight.val.dtype:
+        raise native.NmgError(f"dtype mismatch: B {b.dtype}, weight {weight.val.dtype}")
+    N = b.shape[1]
+    direct = (b.dtype in (torch.float16, torch.bfloat16) and K % 64 == 0 and N > 16
+              and bool(native.load().nmg_densefrag_supported(lay.n, lay.m))
+              and weight.spmm_opt.get("kernel", "auto") in ("auto", "densefrag")
+              and weight.spmm_opt.get("expand", True))
+    if direct and b.stride(1) != 1:
+        b = b.contiguous()
+    if direct and (b.stride(0) % 8 != 0 or b.data_ptr() % 16 != 0 or b.stride(0) >= 2 ** 24):
+        direct = False
+    if not direct:
+        return spmm(weight, b.t().contiguous(), reduce_dim=reduce_dim).t()
+    df = weight.densefrag(reduce_dim)
+    c = torch.empty((O, N), dtype=b.dtype, device=b.device)
+    with torch.cuda.device(b.device):
+        native.check(native.load().nmg_spmm_densefrag_tt(
+            native.ptr(df), O, K, native.ptr(b), b.stride(0), native.ptr(c), N, None, N,
+            native.dtype_code(b.dtype), native.stream_ptr(b.device)))
+    return c
+
+
 def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
     """Y = X @ op(W) for a 2-D ``GroupedNMTensor`` W of shape [R, C].
 

@@ -415,6 +415,45 @@ def test_product_with_both_dense_operands_transposed(dtype, R, C, N, n, m, g):
     assert bool((out[:, N:] == 7.0).all()), "columns beyond N must stay untouched"
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("R,C,N,n,m,g,rd", [
+    (256, 256, 128, 2, 4, 16, 0),      # one tile; W^T @ B: the gradient with respect to B of torch.mm(W, B)
+    (320, 200, 100, 2, 4, 4, 0),       # ragged outputs and columns (N % 8 != 0 goes through a padded pitch)
+    (576, 520, 264, 4, 8, 2, 0),       # several tiles both ways, a pattern the sparse cores do not take
+    (1024, 1024, 1000, 1, 8, 4, 0),
+    (4096, 1024, 2048, 2, 4, 16, 0),   # 64 K steps, full token tiles
+    (264, 448, 136, 4, 8, 4, 1),       # W @ B on the dense matrix cores
+])
+def test_dense_core_product_with_both_dense_operands_transposed(dtype, R, C, N, n, m, g, rd):
+    print(f"case spmm_tt_dense {dtype} R={R} C={C} N={N} {n}:{m}:{g} reduce_dim={rd}", flush=True)
+    W = seeded((R, C), dtype, seed=R + C, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, 1)
+    w = make(W, n, m, g, 1)
+    K, O = (R, C) if rd == 0 else (C, R)
+    b = seeded((K, N), dtype, seed=9)
+    ref = (Wd.T if rd == 0 else Wd) @ to_np(b).astype(np.float64)
+    pitch = -(-N // 8) * 8
+    bb = torch.zeros(K, pitch, dtype=dtype, device=DEV)[:, :N]
+    bb.copy_(b)
+    c = sten.spmm_tt_dense(w, bb, reduce_dim=rd)
+    assert c.shape == (O, N) and c.is_contiguous()
+    assert rel_l2(to_np(c), ref) <= TOL[dtype]
+    c2 = sten.spmm(w, b.to(DEV).t().contiguous(), reduce_dim=rd).t()
+    assert rel_l2(to_np(c), to_np(c2)) <= 2 * TOL[dtype]
+    # the C ABI with a bias per row and a padded output pitch
+    lib = native.load()
+    df = w.densefrag(rd)
+    bias = seeded((O,), dtype, seed=10).to(DEV)
+    out = torch.full((O, pitch + 8), 7.0, dtype=dtype, device=DEV)
+    native.check(lib.nmg_spmm_densefrag_tt(native.ptr(df), O, K, native.ptr(bb), pitch, native.ptr(out), pitch + 8,
+                                           native.ptr(bias), N, native.dtype_code(dtype), None))
+    torch.cuda.synchronize()
+    assert rel_l2(to_np(out[:, :N]), ref + to_np(bias).astype(np.float64)[:, None]) <= TOL[dtype]
+    assert bool((out[:, N:] == 7.0).all()), "columns beyond N must stay untouched"
+    assert lib.nmg_spmm_densefrag_tt(native.ptr(df), O, K, native.ptr(bb), pitch + 4, native.ptr(out), pitch + 8,
+                                     None, N, native.dtype_code(dtype), None) == 2      # ldb % 8
+
+
 def test_transposed_product_argument_errors():
     lib = native.load()
     w = make(seeded((64, 128), torch.float16, 1), 2, 4, 4, 1)
