@@ -32,7 +32,7 @@ typedef _Float16 df_f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 df_bf16x8 __attribute__((ext_vector_type(8)));
 
 // ------------------------------------------------------------------ rowpack -> densefrag
-constexpr int DFX_L = 64, DFX_P = 128;   // LDS tile: lines x positions
+constexpr int DFX_L = 64, DFX_P = 128;   // LDS tile: lines x positions (at most; a tile holds whole blocks)
 
 struct DfExpandParams {
     const void *pk_val;
@@ -41,7 +41,8 @@ struct DfExpandParams {
     const int8_t *order;
     int64_t G, S, nb;
     int64_t OB, K16;                      // blocks of the operand
-    int n, m, pat_bytes, bpt, transpose;  // bpt = blocks of m positions per tile (bpt * m == 128)
+    int n, m, pat_bytes, bpt, transpose;  // bpt = blocks of m positions per tile
+    int pt;                               // positions per tile: bpt * m, a multiple of 32, at most 128
     int order_bytes;                      // size of the order table (specialised kernels: it fits 2 KiB)
 };
 
@@ -60,7 +61,7 @@ template <typename T, int NV> __global__ __launch_bounds__(256) void densefrag_k
     static_assert(sizeof(T) == 2, "16-bit data");
     const int tid = threadIdx.x;
     const int64_t q0 = (int64_t)blockIdx.y * DFX_L, b0 = (int64_t)blockIdx.x * P.bpt;
-    const int rows = P.transpose ? DFX_P : DFX_L, cols = P.transpose ? DFX_L : DFX_P;
+    const int rows = P.transpose ? P.pt : DFX_L, cols = P.transpose ? DFX_L : P.pt;
     const int pitch = cols + PAD;
     {
         uint4 z = {0, 0, 0, 0};
@@ -541,9 +542,20 @@ template <typename T> static int launch_dense(DfParams &P, int variant, hipStrea
 
 using namespace nmg;
 
+// positions per expansion tile: the largest multiple of lcm(m, 32) that fits 128 (0: none)
+static int densefrag_tile_positions(int m)
+{
+    if (m < 1 || m > 64) return 0;
+    int l = m;
+    while (l % 32 != 0) l += m;   // lcm(m, 32)
+    return l <= DFX_P ? DFX_P / l * l : 0;
+}
+
 extern "C" int nmg_densefrag_supported(int n, int m)
 {
-    return (m >= 1 && m <= 64 && n >= 0 && n <= m && (m & (m - 1)) == 0) ? 1 : 0;
+    // m a power of two, or three times one (3, 6, 12, 24, 48): a tile of whole blocks that is also
+    // a whole number of 32-output blocks and 16-position k-steps
+    return (n >= 0 && n <= m && densefrag_tile_positions(m) > 0) ? 1 : 0;
 }
 
 extern "C" int nmg_densefrag_elems(int64_t O, int64_t K, int64_t *elems)
@@ -558,7 +570,7 @@ extern "C" int nmg_densefrag(const void *d_pk_val, const void *d_pk_pat, int64_t
                              void *d_df, int n, int m, int dtype, void *stream)
 {
     NMG_REQUIRE(nmg_densefrag_supported(n, m), NMG_ERR_UNSUPPORTED,
-                "densefrag needs m to be a power of two, got %d:%d", n, m);
+                "densefrag needs m to be a power of two or three times one (at most 64), got %d:%d", n, m);
     NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED, "densefrag takes f16/bf16");
     NMG_REQUIRE(G >= 0 && S >= 0, NMG_ERR_ARG, "negative extent");
     const int64_t O = transpose ? S : G, K = transpose ? G : S;
@@ -579,11 +591,12 @@ extern "C" int nmg_densefrag(const void *d_pk_val, const void *d_pk_pat, int64_t
     P.n = n;
     P.m = m;
     P.pat_bytes = binom(m, n) <= 256 ? 1 : 2;
-    P.bpt = DFX_P / m;
+    P.pt = densefrag_tile_positions(m);
+    P.bpt = P.pt / m;
     P.transpose = transpose ? 1 : 0;
     // the grid covers the padded operand: outputs up to a multiple of 256
     const int64_t Gp = transpose ? G : P.OB * 32, Sp = transpose ? P.OB * 32 : S;
-    const int64_t gx = (Sp + DFX_P - 1) / DFX_P, gy = (Gp + DFX_L - 1) / DFX_L;
+    const int64_t gx = (Sp + P.pt - 1) / P.pt, gy = (Gp + DFX_L - 1) / DFX_L;
     NMG_REQUIRE(gx <= 0x7fffffffLL && gy <= 65535, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
     dim3 grid((unsigned)gx, (unsigned)gy);
     hipStream_t s = (hipStream_t)stream;

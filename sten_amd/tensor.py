@@ -395,7 +395,7 @@ def spmm_tt_dense(weight, b, *, reduce_dim):
     """C = op(W) @ B with both dense operands as they lie in memory, on the dense matrix cores:
     ``reduce_dim=0``: B is [R, N], C = W^T @ B is [C, N] (the gradient with respect to B of
     ``torch.mm(W, B)``); ``reduce_dim=1``: B is [C, N], C = W @ B is [R, N].  Needs 16-bit data, a
-    power-of-two m, a reduction extent that is a multiple of 64, more than 16 columns and a B that is
+    m that is a power of two or three times one, a reduction extent that is a multiple of 64, more than 16 columns and a B that is
     row-contiguous with a row pitch that is a multiple of 8; otherwise through ``spmm`` on the
     transposed operands."""
     lay = weight.layout
@@ -518,7 +518,7 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
                 native.stream_ptr(x.device)))
         return y
     if kname == "densefrag":
-        raise native.NmgError("the densefrag route needs 16-bit data, more than 16 tokens, a power-of-two m "
+        raise native.NmgError("the densefrag route needs 16-bit data, more than 16 tokens, an m that is a power of two or three times one "
                               "and a reduction extent that is a multiple of 64")
     if kname == "expand":
         if not (dense16 and O * K * 2 < 2 ** 31):

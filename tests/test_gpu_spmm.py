@@ -415,6 +415,21 @@ def test_product_with_both_dense_operands_transposed(dtype, R, C, N, n, m, g):
     assert bool((out[:, N:] == 7.0).all()), "columns beyond N must stay untouched"
 
 
+def test_reference_matmul_test_shape_takes_the_dense_matrix_cores():
+    # M, K, N = 768, 3072, 4096 with 3:6:12 ("BERT sizes", dace_gnm_mult.py:1013-1015, :1183): the
+    # automatic choice must be the dense-matrix-core route, not the untuned fallback
+    print("case reference shape 768x3072x4096 3:6:12", flush=True)
+    W = seeded((768, 3072), torch.float16, seed=3, std=0.05)
+    Wd, _ = dense_ref(W, 3, 6, 12, 1)
+    w = make(W, 3, 6, 12, 1)
+    x = seeded((4096, 3072), torch.float16, seed=4)
+    y = sten.spmm(w, x.to(DEV), reduce_dim=1)
+    assert rel_l2(to_np(y), to_np(x).astype(np.float64) @ Wd.T) <= TOL[torch.float16]
+    assert getattr(w, "_densefrag", None) and 1 in w._densefrag, "the dense-core operand was not built"
+    gx = sten.spmm(w, seeded((4096, 768), torch.float16, seed=5).to(DEV), reduce_dim=0)
+    assert rel_l2(to_np(gx), to_np(seeded((4096, 768), torch.float16, seed=5)).astype(np.float64) @ Wd) <= TOL[torch.float16]
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("R,C,N,n,m,g,rd", [
     (256, 256, 128, 2, 4, 16, 0),      # one tile; W^T @ B: the gradient with respect to B of torch.mm(W, B)
@@ -579,6 +594,9 @@ def test_dense_nt_gemm_entry_point(dtype, O_, K, T):
     (320, 448, 77, 2, 4, 16),     # ragged outputs in both directions
     (1024, 1024, 512, 1, 2, 8),
     (192, 128, 40, 3, 16, 1),
+    (320, 192, 70, 3, 6, 12),     # m = 6: tiles of 96 positions (the pattern of the reference's own matmul test)
+    (384, 384, 130, 2, 3, 4),     # m = 3
+    (192, 576, 33, 5, 12, 1),     # m = 12
 ])
 def test_densefrag_route_both_directions(dense_variant, dtype, M, K, T, n, m, g):
     print(f"case densefrag v{dense_variant} {dtype} M={M} K={K} T={T} {n}:{m}:{g}", flush=True)
