@@ -610,6 +610,145 @@ template <typename T> __global__ __launch_bounds__(256) void expand_kernel(Expan
     }
 }
 
+// -------------------------------------------------------------- single precision, plain NT GEMM
+//   Y[T, O] = X[T, K] * A[O, K]^T (+ bias[o]),  all float, V_MFMA_F32_32X32X2_F32
+// The single-precision matrix instruction is 16 times slower than the 16-bit ones (64 clocks for a
+// 32 x 32 x 2 step), so the operands are no problem: a step of 16 reduction positions of a
+// 128 x 128 tile keeps a wavefront's matrix pipe busy for 2048 clocks and needs 16 KiB.  What
+// the kernel has to do is keep the instructions back to back: the tiles of step k+1 are loaded into
+// registers before the MFMAs of step k and stored to the other LDS buffer after them, one
+// barrier per step.  LDS holds a tile as [k][row], so the 32 lanes that share a k read 32
+// consecutive floats.  BM x BN = 128 x 128 (each of the 2 x 2 wavefronts 64 x 64), or 64 x 64
+// where the larger tile would leave most CUs without work.
+struct GemmF32Params {
+    const float *a, *x, *bias;
+    float *y;
+    int64_t lda, ldx, ldy, O, K, T;
+    int vec;   // rows are 16-byte aligned: load four reduction positions at a time
+};
+
+template <int BM, int BN> __global__ __launch_bounds__(256) void gemm_nt_f32_kernel(GemmF32Params P)
+{
+    constexpr int BK = 16;
+    constexpr int MI = BM / 64, NJ = BN / 64;        // 32 x 32 accumulator blocks per wavefront
+    constexpr int XV = BM * BK / 4 / 256, AV = BN * BK / 4 / 256;   // float4 per thread and tile
+    static_assert(XV >= 1 && AV >= 1, "at least 64 rows per side");
+    __shared__ float Xs[2][BK][BM + 4];
+    __shared__ float As[2][BK][BN + 4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int64_t tok0 = (int64_t)blockIdx.y * BM, o0 = (int64_t)blockIdx.x * BN;
+
+    f32x16 acc[MI][NJ];
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    // element e of a tile's load: row e / 4, reduction positions 4 (e % 4) .. +3
+    float4 xr[XV], ar[AV];
+    auto load_tile = [&](int64_t k0) {
+#pragma unroll
+        for (int v = 0; v < XV; v++) {
+            const int e = tid + v * 256, row = e >> 2, kq = (e & 3) * 4;
+            const int64_t tok = tok0 + row, k = k0 + kq;
+            float4 r = {0.f, 0.f, 0.f, 0.f};
+            if (tok < P.T) {
+                const float *src = P.x + tok * P.ldx + k;
+                if (P.vec && k + 3 < P.K) {
+                    r = *(const float4 *)src;
+                } else {
+                    if (k < P.K) r.x = src[0];
+                    if (k + 1 < P.K) r.y = src[1];
+                    if (k + 2 < P.K) r.z = src[2];
+                    if (k + 3 < P.K) r.w = src[3];
+                }
+            }
+            xr[v] = r;
+        }
+#pragma unroll
+        for (int v = 0; v < AV; v++) {
+            const int e = tid + v * 256, row = e >> 2, kq = (e & 3) * 4;
+            const int64_t o = o0 + row, k = k0 + kq;
+            float4 r = {0.f, 0.f, 0.f, 0.f};
+            if (o < P.O) {
+                const float *src = P.a + o * P.lda + k;
+                if (P.vec && k + 3 < P.K) {
+                    r = *(const float4 *)src;
+                } else {
+                    if (k < P.K) r.x = src[0];
+                    if (k + 1 < P.K) r.y = src[1];
+                    if (k + 2 < P.K) r.z = src[2];
+                    if (k + 3 < P.K) r.w = src[3];
+                }
+            }
+            ar[v] = r;
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int v = 0; v < XV; v++) {
+            const int e = tid + v * 256, row = e >> 2, kq = (e & 3) * 4;
+            Xs[buf][kq + 0][row] = xr[v].x;
+            Xs[buf][kq + 1][row] = xr[v].y;
+            Xs[buf][kq + 2][row] = xr[v].z;
+            Xs[buf][kq + 3][row] = xr[v].w;
+        }
+#pragma unroll
+        for (int v = 0; v < AV; v++) {
+            const int e = tid + v * 256, row = e >> 2, kq = (e & 3) * 4;
+            As[buf][kq + 0][row] = ar[v].x;
+            As[buf][kq + 1][row] = ar[v].y;
+            As[buf][kq + 2][row] = ar[v].z;
+            As[buf][kq + 3][row] = ar[v].w;
+        }
+    };
+
+    const int steps = (int)((P.K + BK - 1) / BK);
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+    const int j = lane & 31, h = lane >> 5;
+    for (int st = 0; st < steps; st++) {
+        const int buf = st & 1;
+        if (st + 1 < steps) load_tile((int64_t)(st + 1) * BK);
+        // X is the A operand of the instruction (rows = tokens), the weight tile the B operand
+        // (columns = outputs): lane (j, h) supplies row / column j at reduction position 2 kk + h
+#pragma unroll
+        for (int kk = 0; kk < BK / 2; kk++) {
+            float a[MI], b[NJ];
+#pragma unroll
+            for (int i = 0; i < MI; i++) a[i] = Xs[buf][2 * kk + h][wm * (BM / 2) + i * 32 + j];
+#pragma unroll
+            for (int q = 0; q < NJ; q++) b[q] = As[buf][2 * kk + h][wn * (BN / 2) + q * 32 + j];
+#pragma unroll
+            for (int i = 0; i < MI; i++)
+#pragma unroll
+                for (int q = 0; q < NJ; q++)
+                    acc[i][q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[q], acc[i][q], 0, 0, 0);
+        }
+        if (st + 1 < steps) store_tile(buf ^ 1);   // its last readers finished before the barrier of the last step
+        __syncthreads();
+    }
+
+    // D[row = token][col = output]: lane holds output j, tokens 8*(r/4) + 4*h + r%4
+#pragma unroll
+    for (int q = 0; q < NJ; q++) {
+        const int64_t o = o0 + wn * (BN / 2) + q * 32 + j;
+        if (o >= P.O) continue;
+        const float bv = P.bias ? P.bias[o] : 0.f;
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int64_t tok = tok0 + wm * (BM / 2) + i * 32 + (r >> 2) * 8 + h * 4 + (r & 3);
+                if (tok < P.T) P.y[tok * P.ldy + o] = acc[i][q][r] + bv;
+            }
+    }
+}
+
 }  // namespace nmg
 
 using namespace nmg;
@@ -618,9 +757,40 @@ extern "C" int nmg_gemm_nt(const void *d_a, int64_t lda, const void *d_x, int64_
                            int64_t ldy, const void *d_bias, int64_t O, int64_t K, int64_t T,
                            int dtype, void *stream)
 {
-    NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED, "gemm_nt takes f16/bf16");
+    NMG_REQUIRE(dtype == NMG_F32 || dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED,
+                "gemm_nt takes f32/f16/bf16");
     NMG_REQUIRE(O >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
     NMG_REQUIRE(lda >= K && ldx >= K && ldy >= O, NMG_ERR_ARG, "leading dimension smaller than row length");
+    if (dtype == NMG_F32) {
+        // single precision: any K and any row pitch
+        if (O == 0 || T == 0) return NMG_OK;
+        NMG_REQUIRE(K > 0, NMG_ERR_UNSUPPORTED, "gemm_nt needs K > 0");
+        NMG_REQUIRE(d_a && d_x && d_y, NMG_ERR_ARG, "null device pointer");
+        GemmF32Params Q{};
+        Q.a = (const float *)d_a;
+        Q.x = (const float *)d_x;
+        Q.bias = (const float *)d_bias;
+        Q.y = (float *)d_y;
+        Q.lda = lda;
+        Q.ldx = ldx;
+        Q.ldy = ldy;
+        Q.O = O;
+        Q.K = K;
+        Q.T = T;
+        Q.vec = (lda % 4 == 0 && ldx % 4 == 0 && ((uintptr_t)d_a % 16) == 0 && ((uintptr_t)d_x % 16) == 0) ? 1 : 0;
+        hipStream_t st = (hipStream_t)stream;
+        const int64_t big = ((O + 127) / 128) * ((T + 127) / 128);
+        NMG_REQUIRE((T + 63) / 64 <= 65535, NMG_ERR_UNSUPPORTED, "too many tokens for one launch");
+        if (big >= 128) {
+            dim3 grid((unsigned)((O + 127) / 128), (unsigned)((T + 127) / 128));
+            hipLaunchKernelGGL((gemm_nt_f32_kernel<128, 128>), grid, dim3(256), 0, st, Q);
+        } else {
+            dim3 grid((unsigned)((O + 63) / 64), (unsigned)((T + 63) / 64));
+            hipLaunchKernelGGL((gemm_nt_f32_kernel<64, 64>), grid, dim3(256), 0, st, Q);
+        }
+        NMG_HIP_TRY(hipGetLastError());
+        return NMG_OK;
+    }
     NMG_REQUIRE(K % 64 == 0 && lda % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)d_a % 16) == 0 &&
                     ((uintptr_t)d_x % 16) == 0,
                 NMG_ERR_UNSUPPORTED, "gemm_nt needs K % 64 == 0 and 16-byte aligned rows");

@@ -261,13 +261,24 @@ class GroupedNMTensor:
             cache[reduce_dim] = df
         return df
 
-    def dense_operand(self, reduce_dim):
+    def dense_operand(self, reduce_dim, cached=False):
         """Dense copy [outputs, reduction] of the weight (transposed when the reduction runs along
-        dim 0), expanded from the rowpack operand into fresh scratch; not cached."""
+        dim 0), expanded from the rowpack operand into fresh scratch.  ``cached``: kept until
+        ``val`` changes, like the densefrag operand (``spmm_opt["cache_dense"] = False`` turns
+        that off)."""
         lay = self.layout
+        keep = cached and self.spmm_opt.get("cache_dense", True)
+        key = (self.val.data_ptr(), self.val._version, self.idx.data_ptr())
+        cache = getattr(self, "_dense_operand", None)
+        if cache is None or cache.get("key") != key:
+            cache = self._dense_operand = {"key": key}
+        if keep and reduce_dim in cache:
+            return cache[reduce_dim]
         pk_val, pk_pat = self.rowpack()
         O, K = lay.dense_shape[1 - reduce_dim], lay.dense_shape[reduce_dim]
         out = torch.empty((O, K), dtype=self.val.dtype, device=self.val.device)
+        if keep:
+            cache[reduce_dim] = out
         # rowpack lines run along the group dim; the scratch has the reduction dim contiguous
         transpose = 1 if lay.group_dim == reduce_dim else 0
         with torch.cuda.device(out.device):
@@ -526,6 +537,17 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
                                   "and a reduction extent that is a multiple of 64")
         # the same idea with a plain row-major dense copy of the weight
         a = weight.dense_operand(reduce_dim)
+        with torch.cuda.device(x.device):
+            native.check(native.load().nmg_gemm_nt(
+                native.ptr(a), K, native.ptr(x), x.stride(0), native.ptr(y), O, native.ptr(bias),
+                O, K, T, native.dtype_code(x.dtype), native.stream_ptr(x.device)))
+        return y
+    if (x.dtype == torch.float32 and T > 16 and kname == "auto" and len(lay.dense_shape) == 2
+            and weight.spmm_opt.get("expand", True)):
+        # single precision: "expand, then multiply" as well -- a dense copy of the weight (kept per
+        # weight version) and the pipelined fp32 matrix-core kernel; the kernel below, which expands
+        # inside its reduction loop, runs at a tenth of that rate
+        a = weight.dense_operand(reduce_dim, cached=True)
         with torch.cuda.device(x.device):
             native.check(native.load().nmg_gemm_nt(
                 native.ptr(a), K, native.ptr(x), x.stride(0), native.ptr(y), O, native.ptr(bias),

@@ -586,6 +586,56 @@ def test_dense_nt_gemm_entry_point(dtype, O_, K, T):
     assert rel_l2(to_np(Y), ref) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("O_,K,T,pad", [
+    (256, 64, 128, 0),        # whole 128-wide tiles
+    (300, 323, 77, 0),        # ragged everywhere, rows not 16-byte aligned (scalar loads)
+    (130, 40, 50, 4),         # small tiles, padded pitches
+    (1024, 1024, 512, 0),
+    (64, 17, 200, 3),         # reduction shorter than two K steps, odd pitch
+])
+def test_dense_nt_gemm_entry_point_single_precision(O_, K, T, pad):
+    from sten_amd import native
+    print(f"case gemm_nt f32 O={O_} K={K} T={T} pad={pad}", flush=True)
+    dtype = torch.float32
+    A = seeded((O_, K + pad), dtype, seed=3, std=0.5).to(DEV)
+    X = seeded((T, K + pad), dtype, seed=4).to(DEV)
+    b = seeded((O_,), dtype, seed=5).to(DEV)
+    Y = torch.full((T, O_ + pad), 7.0, dtype=dtype, device=DEV)
+    native.check(native.load().nmg_gemm_nt(A.data_ptr(), K + pad, X.data_ptr(), K + pad, Y.data_ptr(), O_ + pad,
+                                           b.data_ptr(), O_, K, T, native.dtype_code(dtype),
+                                           native.stream_ptr(X.device)))
+    ref = (to_np(X)[:, :K].astype(np.float64) @ to_np(A)[:, :K].astype(np.float64).T
+           + to_np(b).astype(np.float64))
+    assert rel_l2(to_np(Y)[:, :O_], ref) <= TOL[dtype]
+    if pad:
+        assert torch.all(Y[:, O_:] == 7.0)      # nothing written past the row
+
+
+@pytest.mark.parametrize("sd", [1, 0])
+@pytest.mark.parametrize("M,K,T,n,m,g", [(96, 240, 100, 3, 6, 4), (256, 512, 64, 2, 4, 16), (100, 90, 33, 1, 5, 2)])
+def test_single_precision_large_batch_expands_then_multiplies(M, K, T, n, m, g, sd):
+    print(f"case f32 expand route M={M} K={K} T={T} {n}:{m}:{g} sd={sd}", flush=True)
+    dtype = torch.float32
+    W = seeded((M, K), dtype, seed=M + K, std=0.5)
+    x = seeded((T, K), dtype, seed=1)
+    b = seeded((M,), dtype, seed=2)
+    gy = seeded((T, M), dtype, seed=3)
+    Wd, _ = dense_ref(W, n, m, g, sd)
+    w = make(W, n, m, g, sd)
+    y = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)
+    assert rel_l2(to_np(y), to_np(x).astype(np.float64) @ Wd.T + to_np(b).astype(np.float64)) <= TOL[dtype]
+    gx = sten.spmm(w, gy.to(DEV), reduce_dim=0)
+    assert rel_l2(to_np(gx), to_np(gy).astype(np.float64) @ Wd) <= TOL[dtype]
+    # the expanded operand follows the weight: an in-place update of val must show
+    w.val.mul_(2.0)
+    y2 = sten.spmm(w, x.to(DEV), reduce_dim=1)
+    assert rel_l2(to_np(y2), 2.0 * (to_np(x).astype(np.float64) @ Wd.T)) <= TOL[dtype]
+    # and the kernel that expands inside its loop stays reachable and agrees
+    w.spmm_opt["expand"] = False
+    y3 = sten.spmm(w, x.to(DEV), reduce_dim=1)
+    assert rel_l2(to_np(y3), to_np(y2).astype(np.float64)) <= 2 * TOL[dtype]
+
+
 @pytest.mark.parametrize("dense_variant", [-1, 0, 1])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M,K,T,n,m,g", [
