@@ -18,6 +18,11 @@
 //     ds_write_b128 into the same swizzled layout.
 // One s_barrier per stage.  n and m are template parameters so that the expansion is
 // straight-line code on registers.  Requirements: 16-bit data, K % 64 == 0, m in {4, 8}.
+//
+// The file also holds the two halves of "expand, then multiply": the expansion of the rowpack
+// operand into a dense matrix, and the plain NT GEMMs that multiply it (the 16-bit one on the
+// pipeline above, the single-precision one -- gemm_nt_f32_kernel, V_MFMA_F32_32X32X2_F32 -- with
+// its own three-stage loop; single-precision products with more than 16 tokens run on it).
 #include "nmg_common.h"
 
 #include <type_traits>
@@ -25,6 +30,7 @@
 namespace nmg {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -613,13 +619,19 @@ template <typename T> __global__ __launch_bounds__(256) void expand_kernel(Expan
 // -------------------------------------------------------------- single precision, plain NT GEMM
 //   Y[T, O] = X[T, K] * A[O, K]^T (+ bias[o]),  all float, V_MFMA_F32_32X32X2_F32
 // The single-precision matrix instruction is 16 times slower than the 16-bit ones (64 clocks for a
-// 32 x 32 x 2 step), so the operands are no problem: a step of 16 reduction positions of a
-// 128 x 128 tile keeps a wavefront's matrix pipe busy for 2048 clocks and needs 16 KiB.  What
-// the kernel has to do is keep the instructions back to back: the tiles of step k+1 are loaded into
-// registers before the MFMAs of step k and stored to the other LDS buffer after them, one
-// barrier per step.  LDS holds a tile as [k][row], so the 32 lanes that share a k read 32
-// consecutive floats.  BM x BN = 128 x 128 (each of the 2 x 2 wavefronts 64 x 64), or 64 x 64
-// where the larger tile would leave most CUs without work.
+// 32 x 32 x 2 step), so operand traffic is no problem: 16 reduction positions of a 128 x 128 tile
+// keep a wavefront's matrix pipe busy for 2048 clocks and need 16 KiB.  What the kernel has to do
+// is keep the instructions back to back, with one wavefront per SIMD:
+//   * three stages: while the MFMAs of step s run from registers, the fragments of step s+1 are
+//     read from LDS and the tile of step s+2 is on its way from memory; one barrier per step, in
+//     the middle of the MFMAs, where all waves arrive together;
+//   * LDS holds a tile as [row][k] with a pitch of BKT + 4 floats; lane (j, h) of the instruction
+//     reads row j, reduction positions 8h .. 8h+7 with two 128-bit reads (16 lanes x 4 banks, the
+//     pitch spreads them over all 64), and MFMA number kk pairs position kk with 8 + kk -- any
+//     pairing is right as long as both operands use the same one.
+// The 4 wavefronts are WM x WN x WK: WM x WN sub-tiles of (32 MI) x (32 NJ), and WK ways over the
+// reduction inside the workgroup (BKT = 16 WK positions per step, partial sums added through LDS
+// at the end) for products too small to fill the chip with whole tiles.
 struct GemmF32Params {
     const float *a, *x, *bias;
     float *y;
@@ -627,127 +639,242 @@ struct GemmF32Params {
     int vec;   // rows are 16-byte aligned: load four reduction positions at a time
 };
 
-template <int BM, int BN> __global__ __launch_bounds__(256) void gemm_nt_f32_kernel(GemmF32Params P)
+// FAST: rows 16-byte aligned and K a multiple of BKT -- the loads of a step are one 128-bit load
+// per element through pointers computed once (rows past the end are clamped to the last one; their
+// results are never stored), nothing else stands between the MFMAs.
+template <int WM, int WN, int WK, int MI, int NJ, bool FAST>
+__global__ __launch_bounds__(256) void gemm_nt_f32_kernel(GemmF32Params P)
 {
-    constexpr int BK = 16;
-    constexpr int MI = BM / 64, NJ = BN / 64;        // 32 x 32 accumulator blocks per wavefront
-    constexpr int XV = BM * BK / 4 / 256, AV = BN * BK / 4 / 256;   // float4 per thread and tile
-    static_assert(XV >= 1 && AV >= 1, "at least 64 rows per side");
-    __shared__ float Xs[2][BK][BM + 4];
-    __shared__ float As[2][BK][BN + 4];
+    static_assert(WM * WN * WK == 4, "four wavefronts");
+    constexpr int BM = WM * MI * 32, BN = WN * NJ * 32, BKT = 16 * WK, PITCH = BKT + 4;
+    constexpr int KV = BKT / 4;                                      // float4 per tile row
+    constexpr int XE = BM * KV, AE = BN * KV;                        // float4 per tile
+    constexpr int XV = (XE + 255) / 256, AV = (AE + 255) / 256;      // ... per thread
+    constexpr int TILE_FLOATS = 2 * (BM + BN) * PITCH;
+    constexpr int RED_FLOATS = (WK - 1) * WM * WN * MI * NJ * 16 * 64;
+    __shared__ __align__(16) float lds[TILE_FLOATS > RED_FLOATS ? TILE_FLOATS : RED_FLOATS];
+    float *const Xs = lds;                                           // [2][BM][PITCH]
+    float *const As = lds + 2 * BM * PITCH;                          // [2][BN][PITCH]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wk = wave % WK, wn = (wave / WK) % WN, wm = wave / (WK * WN);
     const int64_t tok0 = (int64_t)blockIdx.y * BM, o0 = (int64_t)blockIdx.x * BN;
 
     f32x16 acc[MI][NJ];
 #pragma unroll
     for (int i = 0; i < MI; i++)
 #pragma unroll
-        for (int j = 0; j < NJ; j++)
+        for (int q = 0; q < NJ; q++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+            for (int r = 0; r < 16; r++) acc[i][q][r] = 0.f;
 
-    // element e of a tile's load: row e / 4, reduction positions 4 (e % 4) .. +3
-    float4 xr[XV], ar[AV];
-    auto load_tile = [&](int64_t k0) {
-#pragma unroll
-        for (int v = 0; v < XV; v++) {
-            const int e = tid + v * 256, row = e >> 2, kq = (e & 3) * 4;
-            const int64_t tok = tok0 + row, k = k0 + kq;
-            float4 r = {0.f, 0.f, 0.f, 0.f};
-            if (tok < P.T) {
-                const float *src = P.x + tok * P.ldx + k;
-                if (P.vec && k + 3 < P.K) {
-                    r = *(const float4 *)src;
-                } else {
-                    if (k < P.K) r.x = src[0];
-                    if (k + 1 < P.K) r.y = src[1];
-                    if (k + 2 < P.K) r.z = src[2];
-                    if (k + 3 < P.K) r.w = src[3];
-                }
+    // element e of a tile's load: row e / KV, reduction positions 4 (e % KV) .. +3
+    auto fetch = [&](const float *base, int64_t ld, int64_t row, int64_t nrows, int64_t k) {
+        f32x4 r = {0.f, 0.f, 0.f, 0.f};
+        if (row < nrows) {
+            const float *src = base + row * ld + k;
+            if (P.vec && k + 3 < P.K) {
+                r = *(const f32x4 *)src;
+            } else {
+                if (k < P.K) r[0] = src[0];
+                if (k + 1 < P.K) r[1] = src[1];
+                if (k + 2 < P.K) r[2] = src[2];
+                if (k + 3 < P.K) r[3] = src[3];
             }
-            xr[v] = r;
         }
+        return r;
+    };
+    struct Stage { f32x4 x[XV], a[AV]; };
+    const float *xp[XV], *ap[AV];
 #pragma unroll
-        for (int v = 0; v < AV; v++) {
-            const int e = tid + v * 256, row = e >> 2, kq = (e & 3) * 4;
-            const int64_t o = o0 + row, k = k0 + kq;
-            float4 r = {0.f, 0.f, 0.f, 0.f};
-            if (o < P.O) {
-                const float *src = P.a + o * P.lda + k;
-                if (P.vec && k + 3 < P.K) {
-                    r = *(const float4 *)src;
-                } else {
-                    if (k < P.K) r.x = src[0];
-                    if (k + 1 < P.K) r.y = src[1];
-                    if (k + 2 < P.K) r.z = src[2];
-                    if (k + 3 < P.K) r.w = src[3];
-                }
-            }
-            ar[v] = r;
+    for (int v = 0; v < XV; v++) {
+        const int e = (XE % 256 == 0 || tid + v * 256 < XE) ? tid + v * 256 : 0;
+        const int64_t row = tok0 + e / KV < P.T ? tok0 + e / KV : P.T - 1;
+        xp[v] = P.x + row * P.ldx + (e % KV) * 4;
+    }
+#pragma unroll
+    for (int v = 0; v < AV; v++) {
+        const int e = (AE % 256 == 0 || tid + v * 256 < AE) ? tid + v * 256 : 0;
+        const int64_t row = o0 + e / KV < P.O ? o0 + e / KV : P.O - 1;
+        ap[v] = P.a + row * P.lda + (e % KV) * 4;
+    }
+    // one load / LDS store of a tile: o < XV the activations, the rest the weight
+    constexpr int NG = XV + AV;
+    auto load_op = [&](Stage &G, int64_t k0, int o) {
+        if (o < XV) {
+            const int e = tid + o * 256;
+            if constexpr (FAST) G.x[o] = *(const f32x4 *)(xp[o] + k0);
+            else if (XE % 256 == 0 || e < XE) G.x[o] = fetch(P.x, P.ldx, tok0 + e / KV, P.T, k0 + (e % KV) * 4);
+        } else {
+            const int v = o - XV, e = tid + v * 256;
+            if constexpr (FAST) G.a[v] = *(const f32x4 *)(ap[v] + k0);
+            else if (AE % 256 == 0 || e < AE) G.a[v] = fetch(P.a, P.lda, o0 + e / KV, P.O, k0 + (e % KV) * 4);
         }
     };
-    auto store_tile = [&](int buf) {
-#pragma unroll
-        for (int v = 0; v < XV; v++) {
-            const int e = tid + v * 256, row = e >> 2, kq = (e & 3) * 4;
-            Xs[buf][kq + 0][row] = xr[v].x;
-            Xs[buf][kq + 1][row] = xr[v].y;
-            Xs[buf][kq + 2][row] = xr[v].z;
-            Xs[buf][kq + 3][row] = xr[v].w;
-        }
-#pragma unroll
-        for (int v = 0; v < AV; v++) {
-            const int e = tid + v * 256, row = e >> 2, kq = (e & 3) * 4;
-            As[buf][kq + 0][row] = ar[v].x;
-            As[buf][kq + 1][row] = ar[v].y;
-            As[buf][kq + 2][row] = ar[v].z;
-            As[buf][kq + 3][row] = ar[v].w;
+    auto store_op = [&](const Stage &G, int buf, int o) {
+        if (o < XV) {
+            const int e = tid + o * 256;
+            if (XE % 256 == 0 || e < XE) *(f32x4 *)(Xs + (buf * BM + e / KV) * PITCH + (e % KV) * 4) = G.x[o];
+        } else {
+            const int v = o - XV, e = tid + v * 256;
+            if (AE % 256 == 0 || e < AE) *(f32x4 *)(As + (buf * BN + e / KV) * PITCH + (e % KV) * 4) = G.a[v];
         }
     };
+    auto load_tile = [&](Stage &G, int64_t k0) {
+#pragma unroll
+        for (int o = 0; o < NG; o++) load_op(G, k0, o);
+    };
+    auto store_tile = [&](const Stage &G, int buf) {
+#pragma unroll
+        for (int o = 0; o < NG; o++) store_op(G, buf, o);
+    };
 
-    const int steps = (int)((P.K + BK - 1) / BK);
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
+    struct Frags { f32x4 a[MI][2], b[NJ][2]; };
     const int j = lane & 31, h = lane >> 5;
-    for (int st = 0; st < steps; st++) {
-        const int buf = st & 1;
-        if (st + 1 < steps) load_tile((int64_t)(st + 1) * BK);
-        // X is the A operand of the instruction (rows = tokens), the weight tile the B operand
-        // (columns = outputs): lane (j, h) supplies row / column j at reduction position 2 kk + h
+    const int x_off = (wm * MI * 32 + j) * PITCH + wk * 16 + h * 8;
+    const int a_off = (wn * NJ * 32 + j) * PITCH + wk * 16 + h * 8;
+    // fragment read number o: first the halves that the MFMAs 0 .. 4 MI NJ - 1 of a step use
+    constexpr int NR = 2 * (MI + NJ);
+    auto read_op = [&](Frags &F, int buf, int o) {
+        const int half = o / (MI + NJ), f = o % (MI + NJ);
+        if (f < MI) F.a[f][half] = *(const f32x4 *)(Xs + buf * BM * PITCH + x_off + f * 32 * PITCH + half * 4);
+        else F.b[f - MI][half] = *(const f32x4 *)(As + buf * BN * PITCH + a_off + (f - MI) * 32 * PITCH + half * 4);
+    };
+    auto read_frags = [&](Frags &F, int buf) {
 #pragma unroll
-        for (int kk = 0; kk < BK / 2; kk++) {
-            float a[MI], b[NJ];
+        for (int o = 0; o < NR; o++) read_op(F, buf, o);
+    };
+    // X is the A operand of the instruction (rows = tokens), the weight tile the B operand (columns
+    // = outputs); MFMA number m of a half step
+    constexpr int NH = 4 * MI * NJ;
+    auto mma_one = [&](const Frags &F, int half, int m) {
+        const int kk = m / (MI * NJ), i = (m / NJ) % MI, q = m % NJ;
+        acc[i][q] = __builtin_amdgcn_mfma_f32_32x32x2f32(F.a[i][half][kk], F.b[q][half][kk], acc[i][q], 0, 0, 0);
+    };
+
+    const int steps = (int)((P.K + BKT - 1) / BKT);
+    Frags F0, F1;
+    Stage G0, G1;            // tile t waits in G(t & 1) from step t-3 (its loads) to step t-1 (its LDS stores)
+    load_tile(G0, 0);
+    store_tile(G0, 0);
+    // unconditional (a short reduction loads its last tile again): a branch here would make the
+    // compiler's wait counts in the loop assume the worst, a wait for every load in flight
+    load_tile(G1, (int64_t)(steps > 1 ? 1 : steps - 1) * BKT);
+    load_tile(G0, (int64_t)(steps > 2 ? 2 : steps - 1) * BKT);
+    __syncthreads();
+    read_frags(F0, 0);
+    // step st: `cur` holds the fragments of tile st, `G` tile st+1, the other stage tile st+2.  The
+    // accumulators are pinned to the accumulation registers at every step (left alone, the compiler
+    // moves all of them to vector registers and back around the loop's branches), and the steps
+    // that have a third-next tile run in a loop without branches.
+    auto pin = [&]() {
 #pragma unroll
-            for (int i = 0; i < MI; i++) a[i] = Xs[buf][2 * kk + h][wm * (BM / 2) + i * 32 + j];
+        for (int i = 0; i < MI; i++)
 #pragma unroll
-            for (int q = 0; q < NJ; q++) b[q] = As[buf][2 * kk + h][wn * (BN / 2) + q * 32 + j];
+            for (int q = 0; q < NJ; q++) asm volatile("" : "+a"(acc[i][q]));
+    };
+    // The memory instructions go out one at a time between the MFMAs (64 clocks each): first half
+    // step the LDS stores of tile st+1 and the loads of tile st+3 (two steps, 4096 matrix clocks,
+    // ahead of their use), then the barrier, second half step the fragment reads of tile st+1.
+    // The fences keep that order; without them the scheduler moves the barrier up to the first
+    // MFMA and the next step's LDS stores up to the loads they wait for.
+    auto step = [&](int st, const Frags &cur, Frags &nxt, Stage &G, bool more, bool more3) {
+        pin();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = 0; m < NH; m++) {
+            mma_one(cur, 0, m);
+#pragma unroll
+            for (int o = 0; o < 2 * NG; o++)
+                if (o * NH / (2 * NG) == m) {
+                    if (o < NG) { if (more) store_op(G, (st + 1) & 1, o); }   // last read before the barrier of step st-1
+                    else if (more3) load_op(G, (int64_t)(st + 3) * BKT, o - NG);
+                }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = 0; m < NH; m++) {
+            mma_one(cur, 1, m);
+#pragma unroll
+            for (int o = 0; o < NR; o++)
+                if (o * NH / (2 * NR) == m && more) read_op(nxt, (st + 1) & 1, o);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    int st = 0;
+    for (; st + 4 < steps; st += 2) {
+        step(st, F0, F1, G1, true, true);
+        step(st + 1, F1, F0, G0, true, true);
+    }
+    for (; st < steps; st += 2) {
+        step(st, F0, F1, G1, st + 1 < steps, st + 3 < steps);
+        if (st + 1 < steps) step(st + 1, F1, F0, G0, st + 2 < steps, st + 4 < steps);
+    }
+    pin();
+
+    if constexpr (WK > 1) {
+        // add the partial sums of the WK wavefronts that share a sub-tile; the tiles in LDS are dead
+        // (no wavefront reads them after the barrier of the last step)
+        __syncthreads();
+        float *red = lds;
+        if (wk > 0) {
 #pragma unroll
             for (int i = 0; i < MI; i++)
 #pragma unroll
                 for (int q = 0; q < NJ; q++)
-                    acc[i][q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[q], acc[i][q], 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        red[((((wk - 1) * WM * WN + wm * WN + wn) * MI * NJ + i * NJ + q) * 16 + r) * 64 + lane] = acc[i][q][r];
         }
-        if (st + 1 < steps) store_tile(buf ^ 1);   // its last readers finished before the barrier of the last step
         __syncthreads();
+        if (wk > 0) return;
+#pragma unroll
+        for (int w = 0; w < WK - 1; w++)
+#pragma unroll
+            for (int i = 0; i < MI; i++)
+#pragma unroll
+                for (int q = 0; q < NJ; q++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        acc[i][q][r] += red[(((w * WM * WN + wm * WN + wn) * MI * NJ + i * NJ + q) * 16 + r) * 64 + lane];
     }
 
     // D[row = token][col = output]: lane holds output j, tokens 8*(r/4) + 4*h + r%4
 #pragma unroll
     for (int q = 0; q < NJ; q++) {
-        const int64_t o = o0 + wn * (BN / 2) + q * 32 + j;
+        const int64_t o = o0 + (wn * NJ + q) * 32 + j;
         if (o >= P.O) continue;
         const float bv = P.bias ? P.bias[o] : 0.f;
 #pragma unroll
         for (int i = 0; i < MI; i++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int64_t tok = tok0 + wm * (BM / 2) + i * 32 + (r >> 2) * 8 + h * 4 + (r & 3);
+                const int64_t tok = tok0 + (wm * MI + i) * 32 + (r >> 2) * 8 + h * 4 + (r & 3);
                 if (tok < P.T) P.y[tok * P.ldy + o] = acc[i][q][r] + bv;
             }
     }
 }
+
+template <int WM, int WN, int WK, int MI, int NJ>
+static void launch_gemm_f32(const GemmF32Params &Q, hipStream_t st)
+{
+    constexpr int BM = WM * MI * 32, BN = WN * NJ * 32, BKT = 16 * WK;
+    dim3 grid((unsigned)((Q.O + BN - 1) / BN), (unsigned)((Q.T + BM - 1) / BM));
+    if (Q.vec && Q.K % BKT == 0)
+        hipLaunchKernelGGL((gemm_nt_f32_kernel<WM, WN, WK, MI, NJ, true>), grid, dim3(256), 0, st, Q);
+    else
+        hipLaunchKernelGGL((gemm_nt_f32_kernel<WM, WN, WK, MI, NJ, false>), grid, dim3(256), 0, st, Q);
+}
+
+// Tile shapes of the single-precision kernel: {tokens, outputs, relative efficiency of a tile}.
+// A CU works its tiles off one after the other as far as the matrix pipe is concerned, so a launch
+// costs ceil(tiles / 256) x the cost of one tile; the shape with the smallest product wins (768
+// outputs x 4096 tokens: 192 tiles of 128 x 128 leave a quarter of the CUs idle, 256 of 128 x 96 none).
+struct GemmF32Shape { int bm, bn; double eff; };
+static const GemmF32Shape kGemmF32Shapes[] = {
+    {128, 128, 1.00}, {128, 96, 0.97}, {128, 64, 0.92}, {64, 64, 0.80}, {32, 32, 0.55},
+};
 
 }  // namespace nmg
 
@@ -779,14 +906,21 @@ extern "C" int nmg_gemm_nt(const void *d_a, int64_t lda, const void *d_x, int64_
         Q.T = T;
         Q.vec = (lda % 4 == 0 && ldx % 4 == 0 && ((uintptr_t)d_a % 16) == 0 && ((uintptr_t)d_x % 16) == 0) ? 1 : 0;
         hipStream_t st = (hipStream_t)stream;
-        const int64_t big = ((O + 127) / 128) * ((T + 127) / 128);
-        NMG_REQUIRE((T + 63) / 64 <= 65535, NMG_ERR_UNSUPPORTED, "too many tokens for one launch");
-        if (big >= 128) {
-            dim3 grid((unsigned)((O + 127) / 128), (unsigned)((T + 127) / 128));
-            hipLaunchKernelGGL((gemm_nt_f32_kernel<128, 128>), grid, dim3(256), 0, st, Q);
-        } else {
-            dim3 grid((unsigned)((O + 63) / 64), (unsigned)((T + 63) / 64));
-            hipLaunchKernelGGL((gemm_nt_f32_kernel<64, 64>), grid, dim3(256), 0, st, Q);
+        NMG_REQUIRE((T + 31) / 32 <= 65535, NMG_ERR_UNSUPPORTED, "too many tokens for one launch");
+        int best = 0;
+        double best_cost = 0;
+        for (int c = 0; c < (int)(sizeof(kGemmF32Shapes) / sizeof(kGemmF32Shapes[0])); c++) {
+            const GemmF32Shape &S = kGemmF32Shapes[c];
+            const int64_t tiles = ((T + S.bm - 1) / S.bm) * ((O + S.bn - 1) / S.bn);
+            const double cost = (double)((tiles + 255) / 256) * S.bm * S.bn / S.eff;
+            if (c == 0 || cost < best_cost) { best = c; best_cost = cost; }
+        }
+        switch (best) {
+        case 0: launch_gemm_f32<2, 2, 1, 2, 2>(Q, st); break;
+        case 1: launch_gemm_f32<4, 1, 1, 1, 3>(Q, st); break;
+        case 2: launch_gemm_f32<2, 2, 1, 2, 1>(Q, st); break;
+        case 3: launch_gemm_f32<2, 2, 1, 1, 1>(Q, st); break;
+        default: launch_gemm_f32<1, 1, 4, 1, 1>(Q, st); break;
         }
         NMG_HIP_TRY(hipGetLastError());
         return NMG_OK;
