@@ -642,7 +642,11 @@ struct GemmF32Params {
 // FAST: rows 16-byte aligned and K a multiple of BKT -- the loads of a step are one 128-bit load
 // per element through pointers computed once (rows past the end are clamped to the last one; their
 // results are never stored), nothing else stands between the MFMAs.
-template <int WM, int WN, int WK, int MI, int NJ, bool FAST>
+// AKM: the weight-side operand is given as A[K, O] (reduction-major: Y = X * A, the dense operand of
+// torch.mm as it lies in memory).  Its loads then run along the outputs and the tile is transposed
+// on the way into LDS: element e = (k = e % BKT, group of 4 outputs e / BKT), four 32-bit stores;
+// 16 reduction positions x 4 groups per wavefront fall on 64 different banks.
+template <int WM, int WN, int WK, int MI, int NJ, bool FAST, bool AKM>
 __global__ __launch_bounds__(256) void gemm_nt_f32_kernel(GemmF32Params P)
 {
     static_assert(WM * WN * WK == 4, "four wavefronts");
@@ -694,11 +698,16 @@ __global__ __launch_bounds__(256) void gemm_nt_f32_kernel(GemmF32Params P)
 #pragma unroll
     for (int v = 0; v < AV; v++) {
         const int e = (AE % 256 == 0 || tid + v * 256 < AE) ? tid + v * 256 : 0;
-        const int64_t row = o0 + e / KV < P.O ? o0 + e / KV : P.O - 1;
-        ap[v] = P.a + row * P.lda + (e % KV) * 4;
+        if constexpr (AKM) {
+            const int64_t o = o0 + (e / BKT) * 4 + 3 < P.O ? o0 + (e / BKT) * 4 : (P.O >= 4 ? P.O - 4 : 0);
+            ap[v] = P.a + (int64_t)(e % BKT) * P.lda + o;
+        } else {
+            const int64_t row = o0 + e / KV < P.O ? o0 + e / KV : P.O - 1;
+            ap[v] = P.a + row * P.lda + (e % KV) * 4;
+        }
     }
-    // one load / LDS store of a tile: o < XV the activations, the rest the weight
-    constexpr int NG = XV + AV;
+    // one load / LDS store of a tile: first the activations, then the weight
+    constexpr int NG = XV + AV, CS = AKM ? 4 : 1, NS = XV + CS * AV;
     auto load_op = [&](Stage &G, int64_t k0, int o) {
         if (o < XV) {
             const int e = tid + o * 256;
@@ -706,8 +715,25 @@ __global__ __launch_bounds__(256) void gemm_nt_f32_kernel(GemmF32Params P)
             else if (XE % 256 == 0 || e < XE) G.x[o] = fetch(P.x, P.ldx, tok0 + e / KV, P.T, k0 + (e % KV) * 4);
         } else {
             const int v = o - XV, e = tid + v * 256;
-            if constexpr (FAST) G.a[v] = *(const f32x4 *)(ap[v] + k0);
-            else if (AE % 256 == 0 || e < AE) G.a[v] = fetch(P.a, P.lda, o0 + e / KV, P.O, k0 + (e % KV) * 4);
+            if constexpr (AKM) {
+                if constexpr (FAST) {
+                    G.a[v] = *(const f32x4 *)(ap[v] + k0 * P.lda);
+                } else if (AE % 256 == 0 || e < AE) {
+                    const int64_t k = k0 + e % BKT, o4 = o0 + (e / BKT) * 4;
+                    f32x4 r = {0.f, 0.f, 0.f, 0.f};
+                    if (k < P.K) {
+                        const float *src = P.a + k * P.lda + o4;
+                        if (o4 < P.O) r[0] = src[0];
+                        if (o4 + 1 < P.O) r[1] = src[1];
+                        if (o4 + 2 < P.O) r[2] = src[2];
+                        if (o4 + 3 < P.O) r[3] = src[3];
+                    }
+                    G.a[v] = r;
+                }
+            } else {
+                if constexpr (FAST) G.a[v] = *(const f32x4 *)(ap[v] + k0);
+                else if (AE % 256 == 0 || e < AE) G.a[v] = fetch(P.a, P.lda, o0 + e / KV, P.O, k0 + (e % KV) * 4);
+            }
         }
     };
     auto store_op = [&](const Stage &G, int buf, int o) {
@@ -715,8 +741,11 @@ __global__ __launch_bounds__(256) void gemm_nt_f32_kernel(GemmF32Params P)
             const int e = tid + o * 256;
             if (XE % 256 == 0 || e < XE) *(f32x4 *)(Xs + (buf * BM + e / KV) * PITCH + (e % KV) * 4) = G.x[o];
         } else {
-            const int v = o - XV, e = tid + v * 256;
-            if (AE % 256 == 0 || e < AE) *(f32x4 *)(As + (buf * BN + e / KV) * PITCH + (e % KV) * 4) = G.a[v];
+            const int v = (o - XV) / CS, c = (o - XV) % CS, e = tid + v * 256;
+            if (AE % 256 == 0 || e < AE) {
+                if constexpr (AKM) As[(buf * BN + (e / BKT) * 4 + c) * PITCH + e % BKT] = G.a[v][c];
+                else *(f32x4 *)(As + (buf * BN + e / KV) * PITCH + (e % KV) * 4) = G.a[v];
+            }
         }
     };
     auto load_tile = [&](Stage &G, int64_t k0) {
@@ -725,7 +754,7 @@ __global__ __launch_bounds__(256) void gemm_nt_f32_kernel(GemmF32Params P)
     };
     auto store_tile = [&](const Stage &G, int buf) {
 #pragma unroll
-        for (int o = 0; o < NG; o++) store_op(G, buf, o);
+        for (int o = 0; o < NS; o++) store_op(G, buf, o);
     };
 
     struct Frags { f32x4 a[MI][2], b[NJ][2]; };
@@ -784,10 +813,10 @@ __global__ __launch_bounds__(256) void gemm_nt_f32_kernel(GemmF32Params P)
         for (int m = 0; m < NH; m++) {
             mma_one(cur, 0, m);
 #pragma unroll
-            for (int o = 0; o < 2 * NG; o++)
-                if (o * NH / (2 * NG) == m) {
-                    if (o < NG) { if (more) store_op(G, (st + 1) & 1, o); }   // last read before the barrier of step st-1
-                    else if (more3) load_op(G, (int64_t)(st + 3) * BKT, o - NG);
+            for (int o = 0; o < NS + NG; o++)
+                if (o * NH / (NS + NG) == m) {
+                    if (o < NS) { if (more) store_op(G, (st + 1) & 1, o); }   // last read before the barrier of step st-1
+                    else if (more3) load_op(G, (int64_t)(st + 3) * BKT, o - NS);
                 }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -857,14 +886,18 @@ __global__ __launch_bounds__(256) void gemm_nt_f32_kernel(GemmF32Params P)
 }
 
 template <int WM, int WN, int WK, int MI, int NJ>
-static void launch_gemm_f32(const GemmF32Params &Q, hipStream_t st)
+static void launch_gemm_f32(const GemmF32Params &Q, bool akm, hipStream_t st)
 {
     constexpr int BM = WM * MI * 32, BN = WN * NJ * 32, BKT = 16 * WK;
     dim3 grid((unsigned)((Q.O + BN - 1) / BN), (unsigned)((Q.T + BM - 1) / BM));
-    if (Q.vec && Q.K % BKT == 0)
-        hipLaunchKernelGGL((gemm_nt_f32_kernel<WM, WN, WK, MI, NJ, true>), grid, dim3(256), 0, st, Q);
-    else
-        hipLaunchKernelGGL((gemm_nt_f32_kernel<WM, WN, WK, MI, NJ, false>), grid, dim3(256), 0, st, Q);
+    const bool fast = Q.vec && Q.K % BKT == 0 && (!akm || (Q.O % 4 == 0 && Q.O >= 4));
+    if (akm) {
+        if (fast) hipLaunchKernelGGL((gemm_nt_f32_kernel<WM, WN, WK, MI, NJ, true, true>), grid, dim3(256), 0, st, Q);
+        else hipLaunchKernelGGL((gemm_nt_f32_kernel<WM, WN, WK, MI, NJ, false, true>), grid, dim3(256), 0, st, Q);
+    } else {
+        if (fast) hipLaunchKernelGGL((gemm_nt_f32_kernel<WM, WN, WK, MI, NJ, true, false>), grid, dim3(256), 0, st, Q);
+        else hipLaunchKernelGGL((gemm_nt_f32_kernel<WM, WN, WK, MI, NJ, false, false>), grid, dim3(256), 0, st, Q);
+    }
 }
 
 // Tile shapes of the single-precision kernel: {tokens, outputs, relative efficiency of a tile}.
@@ -880,6 +913,55 @@ static const GemmF32Shape kGemmF32Shapes[] = {
 
 using namespace nmg;
 
+// single precision: any K and any row pitch; `akm`: A is [K, O]
+static int gemm_f32_host(const void *d_a, int64_t lda, const void *d_x, int64_t ldx, void *d_y, int64_t ldy,
+                         const void *d_bias, int64_t O, int64_t K, int64_t T, bool akm, void *stream)
+{
+    if (O == 0 || T == 0) return NMG_OK;
+    NMG_REQUIRE(K > 0, NMG_ERR_UNSUPPORTED, "the fp32 GEMM needs K > 0");
+    NMG_REQUIRE(d_a && d_x && d_y, NMG_ERR_ARG, "null device pointer");
+    GemmF32Params Q{};
+    Q.a = (const float *)d_a;
+    Q.x = (const float *)d_x;
+    Q.bias = (const float *)d_bias;
+    Q.y = (float *)d_y;
+    Q.lda = lda;
+    Q.ldx = ldx;
+    Q.ldy = ldy;
+    Q.O = O;
+    Q.K = K;
+    Q.T = T;
+    Q.vec = (lda % 4 == 0 && ldx % 4 == 0 && ((uintptr_t)d_a % 16) == 0 && ((uintptr_t)d_x % 16) == 0) ? 1 : 0;
+    hipStream_t st = (hipStream_t)stream;
+    NMG_REQUIRE((T + 31) / 32 <= 65535, NMG_ERR_UNSUPPORTED, "too many tokens for one launch");
+    int best = 0;
+    double best_cost = 0;
+    for (int c = 0; c < (int)(sizeof(kGemmF32Shapes) / sizeof(kGemmF32Shapes[0])); c++) {
+        const GemmF32Shape &S = kGemmF32Shapes[c];
+        const int64_t tiles = ((T + S.bm - 1) / S.bm) * ((O + S.bn - 1) / S.bn);
+        const double cost = (double)((tiles + 255) / 256) * S.bm * S.bn / S.eff;
+        if (c == 0 || cost < best_cost) { best = c; best_cost = cost; }
+    }
+    switch (best) {
+    case 0: launch_gemm_f32<2, 2, 1, 2, 2>(Q, akm, st); break;
+    case 1: launch_gemm_f32<4, 1, 1, 1, 3>(Q, akm, st); break;
+    case 2: launch_gemm_f32<2, 2, 1, 2, 1>(Q, akm, st); break;
+    case 3: launch_gemm_f32<2, 2, 1, 1, 1>(Q, akm, st); break;
+    default: launch_gemm_f32<1, 1, 4, 1, 1>(Q, akm, st); break;
+    }
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
+extern "C" int nmg_gemm_nn(const void *d_a, int64_t lda, const void *d_x, int64_t ldx, void *d_y, int64_t ldy,
+                           const void *d_bias, int64_t O, int64_t K, int64_t T, int dtype, void *stream)
+{
+    NMG_REQUIRE(dtype == NMG_F32, NMG_ERR_UNSUPPORTED, "gemm_nn takes f32");
+    NMG_REQUIRE(O >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
+    NMG_REQUIRE(lda >= O && ldx >= K && ldy >= O, NMG_ERR_ARG, "leading dimension smaller than row length");
+    return gemm_f32_host(d_a, lda, d_x, ldx, d_y, ldy, d_bias, O, K, T, true, stream);
+}
+
 extern "C" int nmg_gemm_nt(const void *d_a, int64_t lda, const void *d_x, int64_t ldx, void *d_y,
                            int64_t ldy, const void *d_bias, int64_t O, int64_t K, int64_t T,
                            int dtype, void *stream)
@@ -888,43 +970,8 @@ extern "C" int nmg_gemm_nt(const void *d_a, int64_t lda, const void *d_x, int64_
                 "gemm_nt takes f32/f16/bf16");
     NMG_REQUIRE(O >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
     NMG_REQUIRE(lda >= K && ldx >= K && ldy >= O, NMG_ERR_ARG, "leading dimension smaller than row length");
-    if (dtype == NMG_F32) {
-        // single precision: any K and any row pitch
-        if (O == 0 || T == 0) return NMG_OK;
-        NMG_REQUIRE(K > 0, NMG_ERR_UNSUPPORTED, "gemm_nt needs K > 0");
-        NMG_REQUIRE(d_a && d_x && d_y, NMG_ERR_ARG, "null device pointer");
-        GemmF32Params Q{};
-        Q.a = (const float *)d_a;
-        Q.x = (const float *)d_x;
-        Q.bias = (const float *)d_bias;
-        Q.y = (float *)d_y;
-        Q.lda = lda;
-        Q.ldx = ldx;
-        Q.ldy = ldy;
-        Q.O = O;
-        Q.K = K;
-        Q.T = T;
-        Q.vec = (lda % 4 == 0 && ldx % 4 == 0 && ((uintptr_t)d_a % 16) == 0 && ((uintptr_t)d_x % 16) == 0) ? 1 : 0;
-        hipStream_t st = (hipStream_t)stream;
-        NMG_REQUIRE((T + 31) / 32 <= 65535, NMG_ERR_UNSUPPORTED, "too many tokens for one launch");
-        int best = 0;
-        double best_cost = 0;
-        for (int c = 0; c < (int)(sizeof(kGemmF32Shapes) / sizeof(kGemmF32Shapes[0])); c++) {
-            const GemmF32Shape &S = kGemmF32Shapes[c];
-            const int64_t tiles = ((T + S.bm - 1) / S.bm) * ((O + S.bn - 1) / S.bn);
-            const double cost = (double)((tiles + 255) / 256) * S.bm * S.bn / S.eff;
-            if (c == 0 || cost < best_cost) { best = c; best_cost = cost; }
-        }
-        switch (best) {
-        case 0: launch_gemm_f32<2, 2, 1, 2, 2>(Q, st); break;
-        case 1: launch_gemm_f32<4, 1, 1, 1, 3>(Q, st); break;
-        case 2: launch_gemm_f32<2, 2, 1, 2, 1>(Q, st); break;
-        case 3: launch_gemm_f32<2, 2, 1, 1, 1>(Q, st); break;
-        default: launch_gemm_f32<1, 1, 4, 1, 1>(Q, st); break;
-        }
-        NMG_HIP_TRY(hipGetLastError());
-        return NMG_OK;
-    }
+    if (dtype == NMG_F32)
+        return gemm_f32_host(d_a, lda, d_x, ldx, d_y, ldy, d_bias, O, K, T, false, stream);
     NMG_REQUIRE(K % 64 == 0 && lda % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)d_a % 16) == 0 &&
                     ((uintptr_t)d_x % 16) == 0,
                 NMG_ERR_UNSUPPORTED, "gemm_nt needs K % 64 == 0 and 16-byte aligned rows");

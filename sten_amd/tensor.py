@@ -372,6 +372,27 @@ class GroupedNMTensor:
                 f"device={self.val.device})")
 
 
+def _mm_f32_expanded(weight, b, reduce_dim):
+    """op(W) @ B in single precision with B and the result as they lie in memory: the dense copy of
+    the weight (kept per weight version) as the row operand of the fp32 matrix-core GEMM, B as its
+    reduction-major operand.  None when the route does not apply."""
+    if (b.dtype != torch.float32 or b.shape[1] <= 16 or weight.spmm_opt.get("kernel", "auto") != "auto"
+            or not weight.spmm_opt.get("expand", True)):
+        return None
+    lay = weight.layout
+    K, O = lay.dense_shape[reduce_dim], lay.dense_shape[1 - reduce_dim]
+    if b.stride(1) != 1:
+        b = b.contiguous()
+    N = b.shape[1]
+    wd = weight.dense_operand(reduce_dim, cached=True)          # [O, K]
+    c = torch.empty((O, N), dtype=b.dtype, device=b.device)
+    with torch.cuda.device(b.device):
+        native.check(native.load().nmg_gemm_nn(
+            native.ptr(b), b.stride(0), native.ptr(wd), K, native.ptr(c), N, None, N, K, O,
+            native.dtype_code(b.dtype), native.stream_ptr(b.device)))
+    return c
+
+
 def spmm_tt(weight, b):
     """C = W @ B for a 2-D ``GroupedNMTensor`` W [R, C] and a dense B [C, N] (``torch.mm``), without
     transposing copies when the sparse matrix cores can take it (16-bit, 2-of-4 compatible pattern
@@ -393,6 +414,9 @@ def spmm_tt(weight, b):
         direct = False
     packed = weight.fragpack() if direct else None
     if packed is None:
+        c = _mm_f32_expanded(weight, b, 1)
+        if c is not None:
+            return c
         return spmm(weight, b.t().contiguous(), reduce_dim=1).t()
     c = torch.empty((R, N), dtype=b.dtype, device=b.device)
     with torch.cuda.device(b.device):
@@ -426,6 +450,9 @@ def spmm_tt_dense(weight, b, *, reduce_dim):
     if direct and (b.stride(0) % 8 != 0 or b.data_ptr() % 16 != 0 or b.stride(0) >= 2 ** 24):
         direct = False
     if not direct:
+        c = _mm_f32_expanded(weight, b, reduce_dim)
+        if c is not None:
+            return c
         return spmm(weight, b.t().contiguous(), reduce_dim=reduce_dim).t()
     df = weight.densefrag(reduce_dim)
     c = torch.empty((O, N), dtype=b.dtype, device=b.device)

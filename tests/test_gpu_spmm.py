@@ -592,6 +592,10 @@ def test_dense_nt_gemm_entry_point(dtype, O_, K, T):
     (130, 40, 50, 4),         # small tiles, padded pitches
     (1024, 1024, 512, 0),
     (64, 17, 200, 3),         # reduction shorter than two K steps, odd pitch
+    (96, 3072, 4096, 0),      # one column of 128 x 96 tiles
+    (768, 768, 64, 0),        # 32 x 32 tiles, reduction split inside the workgroup
+    (768, 100, 64, 0),        # the same with a ragged last step
+    (512, 48, 4096, 0),       # 128 x 64 tiles, three steps: prologue and tail only
 ])
 def test_dense_nt_gemm_entry_point_single_precision(O_, K, T, pad):
     from sten_amd import native
@@ -609,6 +613,51 @@ def test_dense_nt_gemm_entry_point_single_precision(O_, K, T, pad):
     assert rel_l2(to_np(Y)[:, :O_], ref) <= TOL[dtype]
     if pad:
         assert torch.all(Y[:, O_:] == 7.0)      # nothing written past the row
+
+
+@pytest.mark.parametrize("O_,K,T,pad", [
+    (256, 64, 128, 0),        # whole 128-wide tiles
+    (300, 323, 77, 0),        # ragged everywhere
+    (130, 40, 50, 4),         # padded pitches
+    (1024, 1024, 512, 0),
+    (66, 17, 200, 3),         # outputs not a multiple of 4, odd pitch
+    (96, 3072, 4096, 0),      # one column of 128 x 96 tiles
+    (768, 768, 64, 0),        # 32 x 32 tiles, reduction split inside the workgroup
+])
+def test_dense_nn_gemm_entry_point_single_precision(O_, K, T, pad):
+    from sten_amd import native
+    print(f"case gemm_nn f32 O={O_} K={K} T={T} pad={pad}", flush=True)
+    dtype = torch.float32
+    A = seeded((K, O_ + pad), dtype, seed=3, std=0.5).to(DEV)        # reduction-major
+    X = seeded((T, K + pad), dtype, seed=4).to(DEV)
+    b = seeded((O_,), dtype, seed=5).to(DEV)
+    Y = torch.full((T, O_ + pad), 7.0, dtype=dtype, device=DEV)
+    native.check(native.load().nmg_gemm_nn(A.data_ptr(), O_ + pad, X.data_ptr(), K + pad, Y.data_ptr(), O_ + pad,
+                                           b.data_ptr(), O_, K, T, native.dtype_code(dtype),
+                                           native.stream_ptr(X.device)))
+    ref = (to_np(X)[:, :K].astype(np.float64) @ to_np(A)[:, :O_].astype(np.float64)
+           + to_np(b).astype(np.float64))
+    assert rel_l2(to_np(Y)[:, :O_], ref) <= TOL[dtype]
+    if pad:
+        assert torch.all(Y[:, O_:] == 7.0)      # nothing written past the row
+
+
+@pytest.mark.parametrize("R,C,N,n,m,g,sd", [(96, 240, 100, 3, 6, 4, 1), (256, 512, 64, 2, 4, 16, 0),
+                                            (100, 90, 33, 1, 5, 2, 1)])
+def test_single_precision_mm_and_its_gradients_keep_the_operands_as_they_lie(R, C, N, n, m, g, sd):
+    print(f"case f32 torch.mm R={R} C={C} N={N} {n}:{m}:{g} sd={sd}", flush=True)
+    dtype = torch.float32
+    W = seeded((R, C), dtype, seed=R + C, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, sd)
+    w = make(W, n, m, g, sd)
+    b = seeded((C, N), dtype, seed=7).to(DEV)
+    c = sten.spmm_tt(w, b)
+    assert c.shape == (R, N) and c.is_contiguous()
+    assert rel_l2(to_np(c), Wd @ to_np(b).astype(np.float64)) <= TOL[dtype]
+    gc = seeded((R, N), dtype, seed=8).to(DEV)
+    gb = sten.spmm_tt_dense(w, gc, reduce_dim=0)
+    assert gb.shape == (C, N) and gb.is_contiguous()
+    assert rel_l2(to_np(gb), Wd.T @ to_np(gc).astype(np.float64)) <= TOL[dtype]
 
 
 @pytest.mark.parametrize("sd", [1, 0])
