@@ -41,10 +41,13 @@ PEAK_FP32_TFLOPS = 157.3    # MI355X dense fp32 MFMA
 ROTATE_BYTES = 512 * 1024 * 1024
 PEAK_HBM_GBS = 8000.0
 SETTLE_S = 0.08                # untimed load before the timed steps (see measure())
+FP32_WORKLOADS = ("c1", "ref_f32", "big_f32")
 
 WORKLOADS = {
     # name: (kind, M, K, tokens, n, m, g, description)
     "c1": ("fwd", 768, 768, 256, 2, 4, 16, "configs[0]: W 768x768 fp32 2:4:16 x 256 tokens, forward (the reference's own CPU-runnable case; fp32 matrix cores)"),
+    "ref_f32": ("fwd", 768, 3072, 4096, 3, 6, 12, "the reference's matmul-test shape in its own dtype: W 768x3072 fp32 3:6:12 x 4096 tokens, forward (fp32 matrix cores on the expanded weight)"),
+    "big_f32": ("fwd", 8192, 8192, 4096, 2, 4, 16, "W 8192x8192 fp32 2:4:16 x 4096 tokens, forward (fp32 matrix cores on the expanded weight)"),
     "c2": ("fwd", 4096, 4096, 2048, 2, 4, 16, "configs[1]: W 4096x4096 fp16 2:4:16 along K x 2048 tokens, forward"),
     "target_2_4": ("fwd", 4096, 11008, 2048, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 2048 tokens, forward"),
     "target_2_4_4k": ("fwd", 4096, 11008, 4096, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 4096 tokens, forward"),
@@ -84,7 +87,7 @@ PMC_SUMMARIES = {
 }
 
 # measured beside the headline workload in the default run: (workload, steps, warm-up)
-ALSO = [("c1", 50, 10), ("c2", 50, 10), ("c3_1_8", 20, 5), ("c3_2_8", 20, 5), ("c3_4_8", 20, 5),
+ALSO = [("c1", 50, 10), ("ref_f32", 20, 5), ("c2", 50, 10), ("c3_1_8", 20, 5), ("c3_2_8", 20, 5), ("c3_4_8", 20, 5),
         ("decode_1", 50, 10), ("decode_4", 50, 10), ("decode_8", 50, 10), ("decode_16", 50, 10),
         ("c4_b1", 50, 10), ("c4_b4", 50, 10), ("c4_b16", 50, 10),
         ("sparsify_c2", 20, 5), ("c5_step", 10, 3), ("c5_train", 10, 3)]
@@ -259,7 +262,7 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
     # copies of it in turn, more than 512 MiB in all.
     copies, turn = 1, [0]
     torch.manual_seed(0)
-    dt = torch.float32 if workload == "c1" else torch.float16
+    dt = torch.float32 if workload in FP32_WORKLOADS else torch.float16
     W = (torch.randn(M, K) * 0.02).to(dt).to(dev)
 
     if kind in ("step", "train"):
@@ -388,7 +391,7 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
         dense_flops = 2.0 * M * K * N * (3 if kind in ("step", "train") else 1)
         eff_flops = dense_flops * n / m
         achieved = eff_flops / (kern_ms * 1e-3) / 1e12
-        peak = PEAK_FP32_TFLOPS if workload == "c1" else PEAK_FP16_TFLOPS
+        peak = PEAK_FP32_TFLOPS if workload in FP32_WORKLOADS else PEAK_FP16_TFLOPS
         row.update({
             "metric": "nmg sparse x dense GEMM TFLOP/s (dense-equiv)",
             "value": dense_flops / wall / 1e12, "unit": "TFLOP/s",
@@ -454,7 +457,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": row["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32" if args.workload == "c1" else "f16", "data": "synthetic",
+        "dtype": "f32" if args.workload in FP32_WORKLOADS else "f16", "data": "synthetic",
         "config": {"workload": desc, "kernel": args.kernel, "variant": args.variant, "launch": row["launch"],
                    "settle": f"{row['settle_steps']} more untimed steps ({SETTLE_S * 1e3:.0f} ms of load) between the "
                              "warm-up and the timed steps: the clocks dip for 10-60 ms after an idle spell",
@@ -464,7 +467,7 @@ def main():
     for key in ("effective_tflops", "algorithmic_bytes", "weight_copies"):
         if key in row:
             out["config"][key] = row[key]
-    if kind in ("fwd", "grad_x") and not args.no_ceiling and args.workload != "c1":
+    if kind in ("fwd", "grad_x") and not args.no_ceiling and args.workload not in FP32_WORKLOADS:
         # The instruction of the dominant kernel, issued from registers with nothing else going on:
         # the 2.5 PFLOP/s behind `peak` assume 2.4 GHz, which random operands do not sustain, and the
         # 32x32x32 sparse instruction stays below its nominal rate even on zeros.
