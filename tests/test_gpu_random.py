@@ -54,6 +54,15 @@ def one_case(rng, big):
         if b is not None:
             ref = ref + to_np(b).astype(np.float64)
         assert rel_l2(to_np(y), ref) <= 2 * TOL[dt], f"spmm reduce_dim={rd}"
+    # torch.mm(W, B) and its gradient with respect to B, operands as they lie in memory
+    B = torch.randn((C, T), generator=gen).to(dt)
+    prod = sten.spmm_tt(w, B.to(DEV))
+    assert prod.shape == (R, T)
+    assert rel_l2(to_np(prod), Wd64 @ to_np(B).astype(np.float64)) <= 2 * TOL[dt], "W @ B"
+    G = torch.randn((R, T), generator=gen).to(dt)
+    gB = sten.spmm_tt_dense(w, G.to(DEV), reduce_dim=0)
+    assert gB.shape == (C, T)
+    assert rel_l2(to_np(gB), Wd64.T @ to_np(G).astype(np.float64)) <= 2 * TOL[dt], "W^T @ G"
     if dt != torch.float32 and R % 8 == 0 and C % 8 == 0:
         gy = torch.randn((T, R), generator=gen).to(dt)
         x = torch.randn((T, C), generator=gen).to(dt)

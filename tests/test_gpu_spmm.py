@@ -430,6 +430,22 @@ def test_reference_matmul_test_shape_takes_the_dense_matrix_cores():
     assert rel_l2(to_np(gx), to_np(seeded((4096, 768), torch.float16, seed=5)).astype(np.float64) @ Wd) <= TOL[torch.float16]
 
 
+def test_reference_matmul_test_shape_in_single_precision():
+    # the same sizes in the dtype of the reference's own test (fp32, dace_gnm_mult.py:1183): expand
+    # once, then the fp32 matrix cores; B [K, N] and C [M, N] as torch.mm has them
+    print("case reference shape 768x3072x4096 3:6:12 fp32", flush=True)
+    W = seeded((768, 3072), torch.float32, seed=3, std=0.05)
+    Wd, _ = dense_ref(W, 3, 6, 12, 1)
+    w = make(W, 3, 6, 12, 1)
+    x = seeded((4096, 3072), torch.float32, seed=4)
+    y = sten.spmm(w, x.to(DEV), reduce_dim=1)
+    assert rel_l2(to_np(y), to_np(x).astype(np.float64) @ Wd.T) <= TOL[torch.float32]
+    assert 1 in getattr(w, "_dense_operand", {}), "the expanded operand was not kept"
+    B = seeded((3072, 4096), torch.float32, seed=5)
+    c = sten.spmm_tt(w, B.to(DEV))
+    assert c.is_contiguous() and rel_l2(to_np(c), Wd @ to_np(B).astype(np.float64)) <= TOL[torch.float32]
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("R,C,N,n,m,g,rd", [
     (256, 256, 128, 2, 4, 16, 0),      # one tile; W^T @ B: the gradient with respect to B of torch.mm(W, B)
