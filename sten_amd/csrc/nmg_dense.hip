@@ -646,7 +646,9 @@ struct GemmF32Params {
 // torch.mm as it lies in memory).  Its loads then run along the outputs and the tile is transposed
 // on the way into LDS: element e = (k = e % BKT, group of 4 outputs e / BKT), four 32-bit stores;
 // 16 reduction positions x 4 groups per wavefront fall on 64 different banks.
-template <int WM, int WN, int WK, int MI, int NJ, bool FAST, bool AKM>
+// XKM: the same for the activation-side operand, X[K, T] (Y = X^T * A: the weight gradient of a
+// linear layer from the upstream gradient and the activations as they lie).
+template <int WM, int WN, int WK, int MI, int NJ, bool FAST, bool AKM, bool XKM>
 __global__ __launch_bounds__(256) void gemm_nt_f32_kernel(GemmF32Params P)
 {
     static_assert(WM * WN * WK == 4, "four wavefronts");
@@ -671,8 +673,9 @@ __global__ __launch_bounds__(256) void gemm_nt_f32_kernel(GemmF32Params P)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][q][r] = 0.f;
 
-    // element e of a tile's load: row e / KV, reduction positions 4 (e % KV) .. +3
-    auto fetch = [&](const float *base, int64_t ld, int64_t row, int64_t nrows, int64_t k) {
+    // Element e of a tile's load.  Row-major operand: row e / KV, reduction positions 4 (e % KV) .. +3.
+    // Reduction-major operand: position e % BKT, rows 4 (e / BKT) .. +3.
+    auto fetch_rm = [&](const float *base, int64_t ld, int64_t row, int64_t nrows, int64_t k) {
         f32x4 r = {0.f, 0.f, 0.f, 0.f};
         if (row < nrows) {
             const float *src = base + row * ld + k;
@@ -687,61 +690,60 @@ __global__ __launch_bounds__(256) void gemm_nt_f32_kernel(GemmF32Params P)
         }
         return r;
     };
+    auto fetch_km = [&](const float *base, int64_t ld, int64_t row, int64_t nrows, int64_t k) {
+        f32x4 r = {0.f, 0.f, 0.f, 0.f};
+        if (k < P.K) {
+            const float *src = base + k * ld + row;
+            if (row < nrows) r[0] = src[0];
+            if (row + 1 < nrows) r[1] = src[1];
+            if (row + 2 < nrows) r[2] = src[2];
+            if (row + 3 < nrows) r[3] = src[3];
+        }
+        return r;
+    };
+    // pointer of the thread's element in the first step (FAST: rows past the end are clamped)
+    auto first_ptr = [&](const float *base, int64_t ld, int64_t r0, int64_t nrows, int e, bool km) {
+        if (km) {
+            const int64_t row = r0 + (e / BKT) * 4 + 3 < nrows ? r0 + (e / BKT) * 4 : (nrows >= 4 ? nrows - 4 : 0);
+            return base + (int64_t)(e % BKT) * ld + row;
+        }
+        const int64_t row = r0 + e / KV < nrows ? r0 + e / KV : nrows - 1;
+        return base + row * ld + (e % KV) * 4;
+    };
     struct Stage { f32x4 x[XV], a[AV]; };
     const float *xp[XV], *ap[AV];
 #pragma unroll
-    for (int v = 0; v < XV; v++) {
-        const int e = (XE % 256 == 0 || tid + v * 256 < XE) ? tid + v * 256 : 0;
-        const int64_t row = tok0 + e / KV < P.T ? tok0 + e / KV : P.T - 1;
-        xp[v] = P.x + row * P.ldx + (e % KV) * 4;
-    }
+    for (int v = 0; v < XV; v++)
+        xp[v] = first_ptr(P.x, P.ldx, tok0, P.T, (XE % 256 == 0 || tid + v * 256 < XE) ? tid + v * 256 : 0, XKM);
 #pragma unroll
-    for (int v = 0; v < AV; v++) {
-        const int e = (AE % 256 == 0 || tid + v * 256 < AE) ? tid + v * 256 : 0;
-        if constexpr (AKM) {
-            const int64_t o = o0 + (e / BKT) * 4 + 3 < P.O ? o0 + (e / BKT) * 4 : (P.O >= 4 ? P.O - 4 : 0);
-            ap[v] = P.a + (int64_t)(e % BKT) * P.lda + o;
-        } else {
-            const int64_t row = o0 + e / KV < P.O ? o0 + e / KV : P.O - 1;
-            ap[v] = P.a + row * P.lda + (e % KV) * 4;
-        }
-    }
+    for (int v = 0; v < AV; v++)
+        ap[v] = first_ptr(P.a, P.lda, o0, P.O, (AE % 256 == 0 || tid + v * 256 < AE) ? tid + v * 256 : 0, AKM);
     // one load / LDS store of a tile: first the activations, then the weight
-    constexpr int NG = XV + AV, CS = AKM ? 4 : 1, NS = XV + CS * AV;
+    constexpr int NG = XV + AV, CSX = XKM ? 4 : 1, CSA = AKM ? 4 : 1, NS = CSX * XV + CSA * AV;
     auto load_op = [&](Stage &G, int64_t k0, int o) {
         if (o < XV) {
             const int e = tid + o * 256;
-            if constexpr (FAST) G.x[o] = *(const f32x4 *)(xp[o] + k0);
-            else if (XE % 256 == 0 || e < XE) G.x[o] = fetch(P.x, P.ldx, tok0 + e / KV, P.T, k0 + (e % KV) * 4);
+            if constexpr (FAST) G.x[o] = *(const f32x4 *)(xp[o] + (XKM ? k0 * P.ldx : k0));
+            else if (XE % 256 == 0 || e < XE)
+                G.x[o] = XKM ? fetch_km(P.x, P.ldx, tok0 + (e / BKT) * 4, P.T, k0 + e % BKT)
+                             : fetch_rm(P.x, P.ldx, tok0 + e / KV, P.T, k0 + (e % KV) * 4);
         } else {
             const int v = o - XV, e = tid + v * 256;
-            if constexpr (AKM) {
-                if constexpr (FAST) {
-                    G.a[v] = *(const f32x4 *)(ap[v] + k0 * P.lda);
-                } else if (AE % 256 == 0 || e < AE) {
-                    const int64_t k = k0 + e % BKT, o4 = o0 + (e / BKT) * 4;
-                    f32x4 r = {0.f, 0.f, 0.f, 0.f};
-                    if (k < P.K) {
-                        const float *src = P.a + k * P.lda + o4;
-                        if (o4 < P.O) r[0] = src[0];
-                        if (o4 + 1 < P.O) r[1] = src[1];
-                        if (o4 + 2 < P.O) r[2] = src[2];
-                        if (o4 + 3 < P.O) r[3] = src[3];
-                    }
-                    G.a[v] = r;
-                }
-            } else {
-                if constexpr (FAST) G.a[v] = *(const f32x4 *)(ap[v] + k0);
-                else if (AE % 256 == 0 || e < AE) G.a[v] = fetch(P.a, P.lda, o0 + e / KV, P.O, k0 + (e % KV) * 4);
-            }
+            if constexpr (FAST) G.a[v] = *(const f32x4 *)(ap[v] + (AKM ? k0 * P.lda : k0));
+            else if (AE % 256 == 0 || e < AE)
+                G.a[v] = AKM ? fetch_km(P.a, P.lda, o0 + (e / BKT) * 4, P.O, k0 + e % BKT)
+                             : fetch_rm(P.a, P.lda, o0 + e / KV, P.O, k0 + (e % KV) * 4);
         }
     };
     auto store_op = [&](const Stage &G, int buf, int o) {
-        if (o < XV) {
-            const int e = tid + o * 256;
-            if (XE % 256 == 0 || e < XE) *(f32x4 *)(Xs + (buf * BM + e / KV) * PITCH + (e % KV) * 4) = G.x[o];
+        if (o < CSX * XV) {
+            const int v = o / CSX, c = o % CSX, e = tid + v * 256;
+            if (XE % 256 == 0 || e < XE) {
+                if constexpr (XKM) Xs[(buf * BM + (e / BKT) * 4 + c) * PITCH + e % BKT] = G.x[v][c];
+                else *(f32x4 *)(Xs + (buf * BM + e / KV) * PITCH + (e % KV) * 4) = G.x[v];
+            }
         } else {
-            const int v = (o - XV) / CS, c = (o - XV) % CS, e = tid + v * 256;
+            const int v = (o - CSX * XV) / CSA, c = (o - CSX * XV) % CSA, e = tid + v * 256;
             if (AE % 256 == 0 || e < AE) {
                 if constexpr (AKM) As[(buf * BN + (e / BKT) * 4 + c) * PITCH + e % BKT] = G.a[v][c];
                 else *(f32x4 *)(As + (buf * BN + e / KV) * PITCH + (e % KV) * 4) = G.a[v];
@@ -886,18 +888,26 @@ __global__ __launch_bounds__(256) void gemm_nt_f32_kernel(GemmF32Params P)
 }
 
 template <int WM, int WN, int WK, int MI, int NJ>
-static void launch_gemm_f32(const GemmF32Params &Q, bool akm, hipStream_t st)
+static void launch_gemm_f32(const GemmF32Params &Q, int form, hipStream_t st)
 {
+    // form 0: X[T, K], A[O, K];  1: X[T, K], A[K, O];  2: X[K, T], A[K, O]
     constexpr int BM = WM * MI * 32, BN = WN * NJ * 32, BKT = 16 * WK;
     dim3 grid((unsigned)((Q.O + BN - 1) / BN), (unsigned)((Q.T + BM - 1) / BM));
-    const bool fast = Q.vec && Q.K % BKT == 0 && (!akm || (Q.O % 4 == 0 && Q.O >= 4));
-    if (akm) {
-        if (fast) hipLaunchKernelGGL((gemm_nt_f32_kernel<WM, WN, WK, MI, NJ, true, true>), grid, dim3(256), 0, st, Q);
-        else hipLaunchKernelGGL((gemm_nt_f32_kernel<WM, WN, WK, MI, NJ, false, true>), grid, dim3(256), 0, st, Q);
+    const bool fast = Q.vec && Q.K % BKT == 0 && (form < 1 || (Q.O % 4 == 0 && Q.O >= 4)) &&
+                      (form < 2 || (Q.T % 4 == 0 && Q.T >= 4));
+#define NMG_F32_LAUNCH(FAST_, AKM_, XKM_) \
+    hipLaunchKernelGGL((gemm_nt_f32_kernel<WM, WN, WK, MI, NJ, FAST_, AKM_, XKM_>), grid, dim3(256), 0, st, Q)
+    if (form == 0) {
+        if (fast) NMG_F32_LAUNCH(true, false, false);
+        else NMG_F32_LAUNCH(false, false, false);
+    } else if (form == 1) {
+        if (fast) NMG_F32_LAUNCH(true, true, false);
+        else NMG_F32_LAUNCH(false, true, false);
     } else {
-        if (fast) hipLaunchKernelGGL((gemm_nt_f32_kernel<WM, WN, WK, MI, NJ, true, false>), grid, dim3(256), 0, st, Q);
-        else hipLaunchKernelGGL((gemm_nt_f32_kernel<WM, WN, WK, MI, NJ, false, false>), grid, dim3(256), 0, st, Q);
+        if (fast) NMG_F32_LAUNCH(true, true, true);
+        else NMG_F32_LAUNCH(false, true, true);
     }
+#undef NMG_F32_LAUNCH
 }
 
 // Tile shapes of the single-precision kernel: {tokens, outputs, relative efficiency of a tile}.
@@ -913,9 +923,9 @@ static const GemmF32Shape kGemmF32Shapes[] = {
 
 using namespace nmg;
 
-// single precision: any K and any row pitch; `akm`: A is [K, O]
+// single precision: any K and any row pitch; `form` as in launch_gemm_f32
 static int gemm_f32_host(const void *d_a, int64_t lda, const void *d_x, int64_t ldx, void *d_y, int64_t ldy,
-                         const void *d_bias, int64_t O, int64_t K, int64_t T, bool akm, void *stream)
+                         const void *d_bias, int64_t O, int64_t K, int64_t T, int form, void *stream)
 {
     if (O == 0 || T == 0) return NMG_OK;
     NMG_REQUIRE(K > 0, NMG_ERR_UNSUPPORTED, "the fp32 GEMM needs K > 0");
@@ -943,11 +953,11 @@ static int gemm_f32_host(const void *d_a, int64_t lda, const void *d_x, int64_t 
         if (c == 0 || cost < best_cost) { best = c; best_cost = cost; }
     }
     switch (best) {
-    case 0: launch_gemm_f32<2, 2, 1, 2, 2>(Q, akm, st); break;
-    case 1: launch_gemm_f32<4, 1, 1, 1, 3>(Q, akm, st); break;
-    case 2: launch_gemm_f32<2, 2, 1, 2, 1>(Q, akm, st); break;
-    case 3: launch_gemm_f32<2, 2, 1, 1, 1>(Q, akm, st); break;
-    default: launch_gemm_f32<1, 1, 4, 1, 1>(Q, akm, st); break;
+    case 0: launch_gemm_f32<2, 2, 1, 2, 2>(Q, form, st); break;
+    case 1: launch_gemm_f32<4, 1, 1, 1, 3>(Q, form, st); break;
+    case 2: launch_gemm_f32<2, 2, 1, 2, 1>(Q, form, st); break;
+    case 3: launch_gemm_f32<2, 2, 1, 1, 1>(Q, form, st); break;
+    default: launch_gemm_f32<1, 1, 4, 1, 1>(Q, form, st); break;
     }
     NMG_HIP_TRY(hipGetLastError());
     return NMG_OK;
@@ -959,7 +969,16 @@ extern "C" int nmg_gemm_nn(const void *d_a, int64_t lda, const void *d_x, int64_
     NMG_REQUIRE(dtype == NMG_F32, NMG_ERR_UNSUPPORTED, "gemm_nn takes f32");
     NMG_REQUIRE(O >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
     NMG_REQUIRE(lda >= O && ldx >= K && ldy >= O, NMG_ERR_ARG, "leading dimension smaller than row length");
-    return gemm_f32_host(d_a, lda, d_x, ldx, d_y, ldy, d_bias, O, K, T, true, stream);
+    return gemm_f32_host(d_a, lda, d_x, ldx, d_y, ldy, d_bias, O, K, T, 1, stream);
+}
+
+extern "C" int nmg_gemm_tn(const void *d_a, int64_t lda, const void *d_x, int64_t ldx, void *d_y, int64_t ldy,
+                           const void *d_bias, int64_t O, int64_t K, int64_t T, int dtype, void *stream)
+{
+    NMG_REQUIRE(dtype == NMG_F32, NMG_ERR_UNSUPPORTED, "gemm_tn takes f32");
+    NMG_REQUIRE(O >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
+    NMG_REQUIRE(lda >= O && ldx >= T && ldy >= O, NMG_ERR_ARG, "leading dimension smaller than row length");
+    return gemm_f32_host(d_a, lda, d_x, ldx, d_y, ldy, d_bias, O, K, T, 2, stream);
 }
 
 extern "C" int nmg_gemm_nt(const void *d_a, int64_t lda, const void *d_x, int64_t ldx, void *d_y,
@@ -971,7 +990,7 @@ extern "C" int nmg_gemm_nt(const void *d_a, int64_t lda, const void *d_x, int64_
     NMG_REQUIRE(O >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
     NMG_REQUIRE(lda >= K && ldx >= K && ldy >= O, NMG_ERR_ARG, "leading dimension smaller than row length");
     if (dtype == NMG_F32)
-        return gemm_f32_host(d_a, lda, d_x, ldx, d_y, ldy, d_bias, O, K, T, false, stream);
+        return gemm_f32_host(d_a, lda, d_x, ldx, d_y, ldy, d_bias, O, K, T, 0, stream);
     NMG_REQUIRE(K % 64 == 0 && lda % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)d_a % 16) == 0 &&
                     ((uintptr_t)d_x % 16) == 0,
                 NMG_ERR_UNSUPPORTED, "gemm_nt needs K % 64 == 0 and 16-byte aligned rows");

@@ -8,6 +8,7 @@ functions: this package's own ``dispatch`` module, or a real ``sten``.
 """
 import torch
 
+from . import native
 from .tensor import GroupedNMTensor, spmm, spmm_tt, spmm_tt_dense
 
 
@@ -31,13 +32,35 @@ class GroupedNMSparsifier:
 def _masked_weight_grad(weight, lhs_t, rhs):
     """val-layout gradient: the kept positions of ``lhs_t^T @ rhs`` (``lhs_t`` [T, rows of W],
     ``rhs`` [T, columns of W]).  16-bit weights take the fused kernel, which never stores the dense
-    product; fp32 and extents that are not multiples of 8 go through the dense product and the
-    same-pattern gather."""
+    product; fp32 (``nmg_gemm_tn``) and extents that are not multiples of 8 go through the dense
+    product and the same-pattern gather."""
     if rhs.dtype != weight.dtype:
         rhs = rhs.to(weight.dtype)
     if weight.masked_product_supported(lhs_t, rhs):
         return weight.masked_product(lhs_t, rhs)
+    if rhs.dtype == torch.float32 and lhs_t.dtype == torch.float32 and lhs_t.is_cuda and lhs_t.shape[0] > 0:
+        # single precision: the dense product on the fp32 matrix cores, operands as they lie
+        # (both reduction-major), then the gather
+        return weight.clone_layout(_f32_product("tn", lhs_t, rhs))
     return weight.clone_layout(torch.mm(lhs_t.t(), rhs))
+
+
+def _f32_product(form, x, a):
+    """Dense fp32 product on this library's matrix-core GEMM, operands as they lie in memory:
+    ``"tn"``: x [K, T], a [K, O] -> x^T @ a;  ``"nt"``: x [T, K], a [O, K] -> x @ a^T."""
+    x = x if x.stride(1) == 1 else x.contiguous()
+    a = a if a.stride(1) == 1 else a.contiguous()
+    if form == "tn":
+        (K, T), O = x.shape, a.shape[1]
+        entry = native.load().nmg_gemm_tn
+    else:
+        (T, K), O = x.shape, a.shape[0]
+        entry = native.load().nmg_gemm_nt
+    y = torch.empty((T, O), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        native.check(entry(native.ptr(a), a.stride(0), native.ptr(x), x.stride(0), native.ptr(y), O,
+                           None, O, K, T, native.dtype_code(torch.float32), native.stream_ptr(x.device)))
+    return y
 
 
 def install(api):
@@ -129,6 +152,8 @@ def install(api):
             # grad_out [R, N] and B [C, N] are reduction-contiguous as they lie: no transposing copies
             if w.masked_product_supported(gc, b, reduction_last=True):
                 gw = wrap(w.masked_product(gc, b, reduction_last=True), gc)
+            elif gc.dtype == torch.float32 and b.dtype == torch.float32 and gc.shape[1] > 0:
+                gw = wrap(w.clone_layout(_f32_product("nt", gc, b)), gc)     # grad_out @ B^T
             else:
                 gw = wrap(_masked_weight_grad(w, gc.t(), b.t()), gc)
         else:

@@ -82,6 +82,7 @@ SIGNATURES = {
     "nmg_spmm_smfmac_tt": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _P]),
     "nmg_gemm_nt": (_I, [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I, _P]),
     "nmg_gemm_nn": (_I, [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I, _P]),
+    "nmg_gemm_tn": (_I, [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I, _P]),
 }
 
 _lib = None

@@ -73,6 +73,15 @@ def one_case(rng, big):
         got = to_np(gw.val).astype(np.float64)
         assert not got[~real].any(), "padded slots of the weight gradient"
         assert rel_l2(got, ref) <= TOL[dt], "masked weight gradient"
+    if dt == torch.float32:
+        # fp32: dense product on the fp32 matrix cores (both operands reduction-major), then the gather
+        from sten_amd.impls import _masked_weight_grad
+        gy = torch.randn((T, R), generator=gen).to(dt)
+        x = torch.randn((T, C), generator=gen).to(dt)
+        gw = _masked_weight_grad(w, gy.to(DEV), x.to(DEV))
+        full = to_np(gy).astype(np.float64).T @ to_np(x).astype(np.float64)
+        ref = O.gather_merged(O.merge(full, lay), idx, lay.n)
+        assert rel_l2(to_np(gw.val).astype(np.float64), ref) <= 2 * TOL[dt], "fp32 weight gradient"
     pv, pi = O.perfect_nm(to_np(W), n, m, sd)
     p = sten.PerfectNMTensor.from_dense(W.to(DEV), n, m, sparse_dim=sd)
     assert same_bits(p.val, pv) and np.array_equal(to_np(p.idx), pi), "ungrouped n:m"

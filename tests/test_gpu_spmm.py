@@ -658,6 +658,30 @@ def test_dense_nn_gemm_entry_point_single_precision(O_, K, T, pad):
         assert torch.all(Y[:, O_:] == 7.0)      # nothing written past the row
 
 
+@pytest.mark.parametrize("O_,K,T,pad", [
+    (256, 64, 128, 0),
+    (300, 323, 77, 0),        # ragged everywhere
+    (130, 40, 50, 4),
+    (1024, 1024, 512, 0),
+    (66, 17, 202, 3),         # neither extent a multiple of 4, odd pitches
+    (96, 3072, 4096, 0),      # one column of 128 x 96 tiles
+    (768, 768, 64, 0),        # 32 x 32 tiles, reduction split inside the workgroup
+])
+def test_dense_tn_gemm_entry_point_single_precision(O_, K, T, pad):
+    from sten_amd import native
+    print(f"case gemm_tn f32 O={O_} K={K} T={T} pad={pad}", flush=True)
+    dtype = torch.float32
+    A = seeded((K, O_ + pad), dtype, seed=3, std=0.5).to(DEV)        # both reduction-major
+    X = seeded((K, T + pad), dtype, seed=4).to(DEV)
+    Y = torch.full((T, O_ + pad), 7.0, dtype=dtype, device=DEV)
+    native.check(native.load().nmg_gemm_tn(A.data_ptr(), O_ + pad, X.data_ptr(), T + pad, Y.data_ptr(), O_ + pad,
+                                           None, O_, K, T, native.dtype_code(dtype), native.stream_ptr(X.device)))
+    ref = to_np(X)[:, :T].astype(np.float64).T @ to_np(A)[:, :O_].astype(np.float64)
+    assert rel_l2(to_np(Y)[:, :O_], ref) <= TOL[dtype]
+    if pad:
+        assert torch.all(Y[:, O_:] == 7.0)
+
+
 @pytest.mark.parametrize("R,C,N,n,m,g,sd", [(96, 240, 100, 3, 6, 4, 1), (256, 512, 64, 2, 4, 16, 0),
                                             (100, 90, 33, 1, 5, 2, 1)])
 def test_single_precision_mm_and_its_gradients_keep_the_operands_as_they_lie(R, C, N, n, m, g, sd):
