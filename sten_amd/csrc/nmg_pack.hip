@@ -23,7 +23,7 @@ struct PackParams {
     uint32_t *fp_idx;
     int64_t G, S, nb, num_chunks;
     int n, m, g, cols, pat_bytes;
-    int R, NBW;          // lines and blocks per workgroup
+    int R, NBW, PW;      // lines and blocks per workgroup; pitch of a line in LDS, in blocks (odd)
     int KP, MBtot;       // fragpack extents: pairs of 32 positions, blocks of 32 lines
     int m_log2;
     int whole_groups;    // m is 4 or 8 and S % 4 == 0: every group of 4 positions lies in one block
@@ -37,16 +37,16 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr PT ABSENT = (PT)~(PT)0;
     const int tid = threadIdx.x, nthr = blockDim.x;
-    const int n = P.n, cols = P.cols, R = P.R, NBW = P.NBW;
-    T *s_val = (T *)smem;                                        // [R][NBW][n]
-    PT *s_pat = (PT *)(smem + (((size_t)R * NBW * n * sizeof(T) + 15) & ~(size_t)15));   // [R][NBW]
-    uint8_t *s_mask = (uint8_t *)(s_pat + (size_t)R * NBW);      // [c] (fragpack only)
+    const int n = P.n, cols = P.cols, R = P.R, NBW = P.NBW, PW = P.PW;
+    T *s_val = (T *)smem;                                        // [R][PW][n]: an odd pitch spreads the 32 lines of a fragment over the banks
+    PT *s_pat = (PT *)(smem + (((size_t)R * PW * n * sizeof(T) + 15) & ~(size_t)15));   // [R][PW]
+    uint8_t *s_mask = (uint8_t *)(s_pat + (size_t)R * PW);      // [c] (fragpack only)
 
     const int64_t r0 = (int64_t)blockIdx.y * R;       // first line
     const int64_t b0 = (int64_t)blockIdx.x * NBW;     // first block
     const int nbw = (int)(P.nb - b0 < NBW ? P.nb - b0 : NBW);   // blocks that exist
 
-    for (int e = tid; e < R * NBW; e += nthr) s_pat[e] = ABSENT;
+    for (int e = tid; e < R * PW; e += nthr) s_pat[e] = ABSENT;
     if (P.fp_val != nullptr) {
         for (int w = 0; w < 32; w++) {
             const uint32_t four = P.masks[w];
@@ -62,7 +62,34 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
         if (kc >= P.num_chunks) break;
         const int64_t slot0 = (kc * P.nb + b0) * cols;   // first slot of the chunk's tiles here
         const int cnt = nbw * cols;
-        if (n <= 4) {
+        if (n == 2 && sizeof(T) == 2) {
+            // the two values of a slot travel as one 32-bit word, four slots per thread in flight
+            // (-11 % on the whole kernel against two 16-bit loads and stores per slot; pairs of
+            // slots per thread, one 64-bit and one 32-bit load, gained another 2 % at 2:4 and lost
+            // as much at 2:8)
+            const uint32_t *val2 = (const uint32_t *)P.val;
+            uint32_t *s_val2 = (uint32_t *)smem;
+            for (int base = tid; base < cnt; base += 4 * nthr) {
+                int o[4];
+                uint32_t vw[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int e = base + u * nthr;
+                    const bool in = e < cnt;
+                    o[u] = in ? (int)P.idx[slot0 + e] : -1;
+                    vw[u] = val2[slot0 + (in ? e : 0)];
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int e = base + u * nthr;
+                    if (o[u] < 0 || kc * cols + o[u] >= P.G) continue;
+                    const int bl = (int)(((uint64_t)e * P.magic_cols) >> 32), slot = e - bl * cols;
+                    const int at = (kcl * cols + o[u]) * PW + bl;
+                    s_pat[at] = (PT)(((uint64_t)slot * P.magic_g) >> 32);
+                    s_val2[at] = vw[u];
+                }
+            }
+        } else if (n <= 4) {
             // four slots per thread are loaded (index and values) before the first is placed:
             // one round trip to HBM per batch instead of one per slot
             for (int base = tid; base < cnt; base += 4 * nthr) {
@@ -83,7 +110,7 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
                     const int e = base + u * nthr;
                     if (o[u] < 0 || kc * cols + o[u] >= P.G) continue;
                     const int bl = (int)(((uint64_t)e * P.magic_cols) >> 32), slot = e - bl * cols;
-                    const int at = (kcl * cols + o[u]) * NBW + bl;
+                    const int at = (kcl * cols + o[u]) * PW + bl;
                     s_pat[at] = (PT)(((uint64_t)slot * P.magic_g) >> 32);
 #pragma unroll
                     for (int j = 0; j < 4; j++)
@@ -95,7 +122,7 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
                 const int bl = (int)(((uint64_t)e * P.magic_cols) >> 32), slot = e - bl * cols;
                 const int o = P.idx[slot0 + e];
                 if (o < 0 || kc * cols + o >= P.G) continue;
-                const int at = (kcl * cols + o) * NBW + bl;
+                const int at = (kcl * cols + o) * PW + bl;
                 s_pat[at] = (PT)(((uint64_t)slot * P.magic_g) >> 32);
                 const T *v = val + (slot0 + e) * n;
                 for (int j = 0; j < n; j++) s_val[at * n + j] = v[j];
@@ -111,8 +138,8 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
         const int run = nbw * n;
         for (int r = tid >> 6; r < R && r0 + r < P.G; r += nthr >> 6) {
             const int64_t q = r0 + r;
-            for (int i = tid & 63; i < run; i += 64) pk_val[(q * P.nb + b0) * n + i] = s_val[(size_t)r * NBW * n + i];
-            for (int i = tid & 63; i < nbw; i += 64) pk_pat[q * P.nb + b0 + i] = s_pat[r * NBW + i];
+            for (int i = tid & 63; i < run; i += 64) pk_val[(q * P.nb + b0) * n + i] = s_val[(size_t)r * PW * n + i];
+            for (int i = tid & 63; i < nbw; i += 64) pk_pat[q * P.nb + b0 + i] = s_pat[r * PW + i];
         }
     }
     if (P.fp_val == nullptr) return;
@@ -146,7 +173,7 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
                     const bool in = (b0 << P.m_log2) + k0 < P.S;
                     blk[q] = in ? k0 >> P.m_log2 : 0;
                     base[q] = k0 & (m - 1);
-                    pt[q] = in ? s_pat[r * NBW + blk[q]] : ABSENT;
+                    pt[q] = in ? s_pat[r * PW + blk[q]] : ABSENT;
                 }
 #pragma unroll
                 for (int q = 0; q < 4; q++) mkb[q] = pt[q] == ABSENT ? 0 : (int)mask[pt[q]];
@@ -154,7 +181,7 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
                     const int j0 = __popc(mkb[q] & ((1 << base[q]) - 1));
-                    const T *bv = s_val + ((size_t)r * NBW + blk[q]) * n;
+                    const T *bv = s_val + ((size_t)r * PW + blk[q]) * n;
                     const T x0 = bv[j0 < n ? j0 : 0], x1 = bv[j0 + 1 < n ? j0 + 1 : 0];
                     c0[q] = *reinterpret_cast<const uint16_t *>(&x0);
                     c1[q] = *reinterpret_cast<const uint16_t *>(&x1);
@@ -209,7 +236,7 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
                 const int q = e >> 2, i = e & 3;
                 const int k = (kpl * 2 + ks) * 32 + (4 * (q >> 1) + 2 * ga + (q & 1)) * 4 + i;   // from the first block
                 // beyond S the probe reads its line's first block; it is ignored below
-                pat[e] = s_pat[r * NBW + ((b0 << P.m_log2) + k < P.S ? k >> P.m_log2 : 0)];
+                pat[e] = s_pat[r * PW + ((b0 << P.m_log2) + k < P.S ? k >> P.m_log2 : 0)];
             }
 #pragma unroll
             for (int e = 0; e < 16; e++) mk[e] = pat[e] == ABSENT ? 0 : (int)mask[pat[e]];
@@ -218,7 +245,7 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
                 const int q = e >> 2, i = e & 3;
                 const int k = (kpl * 2 + ks) * 32 + (4 * (q >> 1) + 2 * ga + (q & 1)) * 4 + i;
                 const int j = __popc(mk[e] & ((1 << (k & (m - 1))) - 1));
-                const T x = s_val[((size_t)r * NBW + ((b0 << P.m_log2) + k < P.S ? k >> P.m_log2 : 0)) * n + (j < n ? j : 0)];
+                const T x = s_val[((size_t)r * PW + ((b0 << P.m_log2) + k < P.S ? k >> P.m_log2 : 0)) * n + (j < n ? j : 0)];
                 cand[e] = *reinterpret_cast<const uint16_t *>(&x);
             }
             uint16_t vals[8];
@@ -321,7 +348,15 @@ extern "C" int nmg_pack_operands(const void *d_val, const int16_t *d_idx, int64_
     NBW = NBW / nbw_unit * nbw_unit;
     if (NBW < nbw_unit) NBW = nbw_unit;
     if (NBW > 256) NBW = 256 / nbw_unit * nbw_unit;
-    const size_t lds = (((size_t)R64 * NBW * n * elem + 15) & ~(size_t)15) + (size_t)R64 * NBW * pat_bytes + 160;
+    // Pitch of a line in LDS: odd, so that the 32 lines a fragment reads side by side fall on
+    // different banks (-10 % on 2:4:16: 6 workgroups of 23.7 KB per CU instead of 7 of 23.2), but
+    // only where six padded workgroups still fit a CU: at 2:8:32 the padding takes the CU from
+    // four workgroups of 36 KB to three (+3 %).
+    auto lds_for = [&](int64_t pw) {
+        return (((size_t)R64 * pw * n * elem + 15) & ~(size_t)15) + (size_t)R64 * pw * pat_bytes + 160;
+    };
+    const int64_t PW = lds_for(NBW | 1) * 6 <= 156 * 1024 ? (NBW | 1) : NBW;
+    const size_t lds = lds_for(PW);
     const bool one_pass = n >= 1 && lds <= 96 * 1024 && (int64_t)NBW * tg.cols < 65536 && R64 * NBW * (int64_t)(n > 1 ? n : 1) < ((int64_t)1 << 30) &&
                           (!frag || (pow2 && m <= 8 && tg.c <= 128));
     if (!one_pass) {
@@ -348,6 +383,7 @@ extern "C" int nmg_pack_operands(const void *d_val, const int16_t *d_idx, int64_
     P.pat_bytes = pat_bytes;
     P.R = (int)R64;
     P.NBW = (int)NBW;
+    P.PW = (int)PW;
     P.KP = (int)((S + 63) / 64);
     P.MBtot = (int)((G + 255) / 256 * 8);
     P.m_log2 = 0;
