@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
     const int tid = threadIdx.x, nthr = blockDim.x;
     const int n = P.n, cols = P.cols, R = P.R, NBW = P.NBW, PW = P.PW;
     T *s_val = (T *)smem;                                        // [R][PW][n]: an odd pitch spreads the 32 lines of a fragment over the banks
-    PT *s_pat = (PT *)(smem + (((size_t)R * PW * n * sizeof(T) + 15) & ~(size_t)15));   // [R][PW]
+    PT *s_pat = (PT *)(smem + (((size_t)R * PW * n * sizeof(T) + 15) & ~(size_t)15));   // [R][NBW] (rows stay 16-byte aligned where NBW is a multiple of 16)
     uint8_t *s_mask = (uint8_t *)(s_pat + (size_t)R * PW);      // [c] (fragpack only)
 
     const int64_t r0 = (int64_t)blockIdx.y * R;       // first line
@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
                     if (o[u] < 0 || kc * cols + o[u] >= P.G) continue;
                     const int bl = (int)(((uint64_t)e * P.magic_cols) >> 32), slot = e - bl * cols;
                     const int at = (kcl * cols + o[u]) * PW + bl;
-                    s_pat[at] = (PT)(((uint64_t)slot * P.magic_g) >> 32);
+                    s_pat[(kcl * cols + o[u]) * NBW + bl] = (PT)(((uint64_t)slot * P.magic_g) >> 32);
                     s_val2[at] = vw[u];
                 }
             }
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
                     if (o[u] < 0 || kc * cols + o[u] >= P.G) continue;
                     const int bl = (int)(((uint64_t)e * P.magic_cols) >> 32), slot = e - bl * cols;
                     const int at = (kcl * cols + o[u]) * PW + bl;
-                    s_pat[at] = (PT)(((uint64_t)slot * P.magic_g) >> 32);
+                    s_pat[(kcl * cols + o[u]) * NBW + bl] = (PT)(((uint64_t)slot * P.magic_g) >> 32);
 #pragma unroll
                     for (int j = 0; j < 4; j++)
                         if (j < n) s_val[at * n + j] = vv[u][j];
@@ -123,7 +123,7 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
                 const int o = P.idx[slot0 + e];
                 if (o < 0 || kc * cols + o >= P.G) continue;
                 const int at = (kcl * cols + o) * PW + bl;
-                s_pat[at] = (PT)(((uint64_t)slot * P.magic_g) >> 32);
+                s_pat[(kcl * cols + o) * NBW + bl] = (PT)(((uint64_t)slot * P.magic_g) >> 32);
                 const T *v = val + (slot0 + e) * n;
                 for (int j = 0; j < n; j++) s_val[at * n + j] = v[j];
             }
@@ -131,17 +131,48 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
     }
     __syncthreads();
 
-    // ---- rowpack: a wavefront writes the whole run of a line
-    {
-        T *pk_val = (T *)P.pk_val;
-        PT *pk_pat = (PT *)P.pk_pat;
-        const int run = nbw * n;
-        for (int r = tid >> 6; r < R && r0 + r < P.G; r += nthr >> 6) {
-            const int64_t q = r0 + r;
-            for (int i = tid & 63; i < run; i += 64) pk_val[(q * P.nb + b0) * n + i] = s_val[(size_t)r * PW * n + i];
-            for (int i = tid & 63; i < nbw; i += 64) pk_pat[q * P.nb + b0 + i] = s_pat[r * PW + i];
+    // ---- rowpack: the runs of the lines go out as one flat list of pieces -- 16 bytes where the
+    //      ends of a run are aligned (four 32-bit LDS reads each: the odd pitch keeps the rows
+    //      word-aligned only), else 4 bytes, else single elements -- so that every lane has a piece
+    //      (a wavefront per line wrote 2 bytes per lane, and 12 lanes of 64 where a run is 24 bytes)
+    auto write_runs = [&](unsigned char *dst, int64_t row_b, const unsigned char *src, int pitch_b, int run_b,
+                          int unit_b, bool rows16) {
+        // largest piece that divides the run, the rows' distance and both starts
+        const uintptr_t mis = (uintptr_t)dst | (uintptr_t)row_b | (uintptr_t)run_b;
+        const int piece = (mis % 16 == 0 && pitch_b % 4 == 0 && rows16) ? 16 : (mis % 4 == 0 && pitch_b % 4 == 0) ? 4 : unit_b;
+        const int ppl = run_b / piece;   // pieces per line
+        const uint64_t magic = (((uint64_t)1 << 32) + ppl - 1) / (ppl > 0 ? ppl : 1);
+        const int total = R * ppl;       // < 2^22 (the tile fits LDS): the magic division is exact
+        if (piece == 16) {
+            for (int i = tid; i < total; i += nthr) {
+                const int r = (int)(((uint64_t)i * magic) >> 32), ch = i - r * ppl;
+                if (r0 + r >= P.G) continue;
+                const uint32_t *w = (const uint32_t *)(src + (size_t)r * pitch_b + (size_t)ch * 16);
+                *(uint4 *)(dst + (r0 + r) * row_b + (size_t)ch * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        } else if (piece == 4) {
+            for (int i = tid; i < total; i += nthr) {
+                const int r = (int)(((uint64_t)i * magic) >> 32), ch = i - r * ppl;
+                if (r0 + r >= P.G) continue;
+                *(uint32_t *)(dst + (r0 + r) * row_b + (size_t)ch * 4) = *(const uint32_t *)(src + (size_t)r * pitch_b + (size_t)ch * 4);
+            }
+        } else {
+            for (int i = tid; i < total; i += nthr) {
+                const int r = (int)(((uint64_t)i * magic) >> 32), ch = i - r * ppl;
+                if (r0 + r >= P.G) continue;
+                unsigned char *d = dst + (r0 + r) * row_b + (size_t)ch * piece;
+                const unsigned char *sp = src + (size_t)r * pitch_b + (size_t)ch * piece;
+                if (piece == 2) *(uint16_t *)d = *(const uint16_t *)sp;
+                else if (piece == 1) *d = *sp;
+                else for (int e = 0; e < piece; e++) d[e] = sp[e];
+            }
         }
-    }
+    };
+    write_runs((unsigned char *)P.pk_val + b0 * n * sizeof(T), (int64_t)P.nb * n * (int64_t)sizeof(T),
+               (const unsigned char *)s_val, PW * n * (int)sizeof(T), nbw * n * (int)sizeof(T), (int)sizeof(T), true);
+    write_runs((unsigned char *)P.pk_pat + b0 * sizeof(PT), (int64_t)P.nb * (int64_t)sizeof(PT),
+               (const unsigned char *)s_pat, NBW * (int)sizeof(PT), nbw * (int)sizeof(PT), (int)sizeof(PT),
+               (NBW * sizeof(PT)) % 16 == 0);
     if (P.fp_val == nullptr) return;
 
     // ---- fragpack: one wavefront per (32 lines, 64 positions); a lane emits its 2 x 8 values and
@@ -173,11 +204,20 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
                     const bool in = (b0 << P.m_log2) + k0 < P.S;
                     blk[q] = in ? k0 >> P.m_log2 : 0;
                     base[q] = k0 & (m - 1);
-                    pt[q] = in ? s_pat[r * PW + blk[q]] : ABSENT;
+                    pt[q] = in ? s_pat[r * NBW + blk[q]] : ABSENT;
                 }
 #pragma unroll
                 for (int q = 0; q < 4; q++) mkb[q] = pt[q] == ABSENT ? 0 : (int)mask[pt[q]];
                 uint16_t c0[4], c1[4];
+                if (m == 4 && n == 2) {
+                    // a block is a group: its two values are one word
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const uint32_t w = ((const uint32_t *)s_val)[r * PW + blk[q]];
+                        c0[q] = (uint16_t)(w & 0xFFFFu);
+                        c1[q] = (uint16_t)(w >> 16);
+                    }
+                } else
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
                     const int j0 = __popc(mkb[q] & ((1 << base[q]) - 1));
@@ -236,7 +276,7 @@ __global__ __launch_bounds__(256) void pack_kernel(PackParams P)
                 const int q = e >> 2, i = e & 3;
                 const int k = (kpl * 2 + ks) * 32 + (4 * (q >> 1) + 2 * ga + (q & 1)) * 4 + i;   // from the first block
                 // beyond S the probe reads its line's first block; it is ignored below
-                pat[e] = s_pat[r * PW + ((b0 << P.m_log2) + k < P.S ? k >> P.m_log2 : 0)];
+                pat[e] = s_pat[r * NBW + ((b0 << P.m_log2) + k < P.S ? k >> P.m_log2 : 0)];
             }
 #pragma unroll
             for (int e = 0; e < 16; e++) mk[e] = pat[e] == ABSENT ? 0 : (int)mask[pat[e]];
