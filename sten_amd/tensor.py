@@ -374,8 +374,8 @@ class GroupedNMTensor:
 
 def _mm_f32_expanded(weight, b, reduce_dim):
     """op(W) @ B in single precision with B and the result as they lie in memory: the dense copy of
-    the weight (kept per weight version) as the row operand of the fp32 matrix-core GEMM, B as its
-    reduction-major operand.  None when the route does not apply."""
+    the weight (kept per weight version; the same one for both directions) as the row operand of
+    the fp32 matrix-core GEMM, B as its reduction-major operand.  None when the route does not apply."""
     if (b.dtype != torch.float32 or b.shape[1] <= 16 or weight.spmm_opt.get("kernel", "auto") != "auto"
             or not weight.spmm_opt.get("expand", True)):
         return None
@@ -384,11 +384,13 @@ def _mm_f32_expanded(weight, b, reduce_dim):
     if b.stride(1) != 1:
         b = b.contiguous()
     N = b.shape[1]
-    wd = weight.dense_operand(reduce_dim, cached=True)          # [O, K]
+    # the one dense copy [R, C]: row-major row operand of W @ B, reduction-major row operand of W^T @ B
+    wd = weight.dense_operand(1, cached=True)
+    entry = native.load().nmg_gemm_nn if reduce_dim == 1 else native.load().nmg_gemm_tn
     c = torch.empty((O, N), dtype=b.dtype, device=b.device)
     with torch.cuda.device(b.device):
-        native.check(native.load().nmg_gemm_nn(
-            native.ptr(b), b.stride(0), native.ptr(wd), K, native.ptr(c), N, None, N, K, O,
+        native.check(entry(
+            native.ptr(b), b.stride(0), native.ptr(wd), wd.stride(0), native.ptr(c), N, None, N, K, O,
             native.dtype_code(b.dtype), native.stream_ptr(b.device)))
     return c
 
@@ -574,10 +576,13 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
         # single precision: "expand, then multiply" as well -- a dense copy of the weight (kept per
         # weight version) and the pipelined fp32 matrix-core kernel; the kernel below, which expands
         # inside its reduction loop, runs at a tenth of that rate
-        a = weight.dense_operand(reduce_dim, cached=True)
+        # One dense copy [R, C] serves both directions: row-major operand of the product that
+        # reduces along dim 1, reduction-major operand of the one that reduces along dim 0.
+        a = weight.dense_operand(1, cached=True)
+        entry = native.load().nmg_gemm_nt if reduce_dim == 1 else native.load().nmg_gemm_nn
         with torch.cuda.device(x.device):
-            native.check(native.load().nmg_gemm_nt(
-                native.ptr(a), K, native.ptr(x), x.stride(0), native.ptr(y), O, native.ptr(bias),
+            native.check(entry(
+                native.ptr(a), a.stride(0), native.ptr(x), x.stride(0), native.ptr(y), O, native.ptr(bias),
                 O, K, T, native.dtype_code(x.dtype), native.stream_ptr(x.device)))
         return y
     pk_val, pk_pat = weight.rowpack()
