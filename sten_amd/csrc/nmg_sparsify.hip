@@ -1555,39 +1555,61 @@ __global__ __launch_bounds__(256) void scatter_tiled_kernel(TiledParams Q)
     // store is otherwise one round trip to HBM per slot and thread.
     const int total = tiles * cols;
     const int64_t at0 = t0 * (int64_t)cols;
-    const bool pair = sizeof(T) == 2 && n == 2 && ((uintptr_t)P.val % 4) == 0;
-    for (int base = tid; base < total; base += 4 * 256) {
-        int o[4];
+    // NV > 0: n is the constant NV and a slot's NV values are one aligned word of 4 or 8 bytes -- one
+    // load (issued with the index loads) or store per slot instead of NV of 2 or 4 bytes; NV = 0:
+    // any n, value by value.
+    auto run_slots = [&](auto nv_tag) {
+        constexpr int NV = decltype(nv_tag)::value;
+        constexpr int WB = NV * (int)sizeof(T);            // bytes of a slot's word
+        using Word = typename std::conditional<WB == 8, uint2, uint32_t>::type;
+        for (int base = tid; base < total; base += 4 * 256) {
+            int o[4];
+            Word vw[4];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const int e = base + u * 256;
-            o[u] = e < total ? (int)P.idx[at0 + e] : -1;
-        }
+            for (int u = 0; u < 4; u++) {
+                const int e = base + u * 256;
+                o[u] = e < total ? (int)P.idx[at0 + e] : -1;
+                if (!GATHER && NV > 0) vw[u] = ((const Word *)P.val)[at0 + (e < total ? e : 0)];
+            }
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const int e = base + u * 256;
-            if (e >= total) continue;
-            const int tm = (int)(((uint64_t)e * Q.magic_cols) >> 32), slot = e - tm * cols;
-            const int p = (int)(((uint64_t)slot * Q.magic_g) >> 32);
-            const bool ok = o[u] >= 0 && o[u] < cols;
-            T *v = (T *)P.val + (at0 + e) * n;
-            const T *row = tile + (ok ? o[u] : 0) * pitch + tm * m;
-            if (GATHER) {
-                if (pair) {
-                    T w[2];
-                    w[0] = ok ? row[order[p * 2]] : Zero<T>::v();
-                    w[1] = ok ? row[order[p * 2 + 1]] : Zero<T>::v();
-                    uint32_t raw;
-                    __builtin_memcpy(&raw, w, 4);
-                    *(uint32_t *)v = raw;
+            for (int u = 0; u < 4; u++) {
+                const int e = base + u * 256;
+                if (e >= total) continue;
+                const int tm = (int)(((uint64_t)e * Q.magic_cols) >> 32), slot = e - tm * cols;
+                const int p = (int)(((uint64_t)slot * Q.magic_g) >> 32);
+                const bool ok = o[u] >= 0 && o[u] < cols;
+                T *v = (T *)P.val + (at0 + e) * n;
+                T *row = tile + (ok ? o[u] : 0) * pitch + tm * m;
+                if constexpr (NV > 0) {
+                    T w[NV];
+                    if (GATHER) {
+#pragma unroll
+                        for (int j = 0; j < NV; j++) w[j] = ok ? row[order[p * NV + j]] : Zero<T>::v();
+                        Word raw;
+                        __builtin_memcpy(&raw, w, WB);
+                        ((Word *)P.val)[at0 + e] = raw;
+                    } else if (ok) {
+                        __builtin_memcpy(w, &vw[u], WB);
+#pragma unroll
+                        for (int j = 0; j < NV; j++) row[order[p * NV + j]] = w[j];
+                    }
                 } else {
-                    for (int j = 0; j < n; j++) v[j] = ok ? row[order[p * n + j]] : Zero<T>::v();
+                    if (GATHER) {
+                        for (int j = 0; j < n; j++) v[j] = ok ? row[order[p * n + j]] : Zero<T>::v();
+                    } else if (ok) {
+                        for (int j = 0; j < n; j++) row[order[p * n + j]] = v[j];
+                    }
                 }
-            } else if (ok) {
-                for (int j = 0; j < n; j++) tile[o[u] * pitch + tm * m + order[p * n + j]] = v[j];
             }
         }
-    }
+    };
+    const int vbytes = n * (int)sizeof(T);
+    const bool aligned = ((uintptr_t)P.val % 8) == 0;
+    if (aligned && vbytes == 4 && n == 1) run_slots(std::integral_constant<int, (sizeof(T) == 4 ? 1 : 0)>{});
+    else if (aligned && vbytes == 4 && n == 2) run_slots(std::integral_constant<int, (sizeof(T) == 2 ? 2 : 0)>{});
+    else if (aligned && vbytes == 8 && n == 2) run_slots(std::integral_constant<int, (sizeof(T) == 4 ? 2 : 0)>{});
+    else if (aligned && vbytes == 8 && n == 4) run_slots(std::integral_constant<int, (sizeof(T) == 2 ? 4 : 0)>{});
+    else run_slots(std::integral_constant<int, 0>{});
     if (GATHER) return;
     __syncthreads();
     // LDS -> region
