@@ -562,7 +562,7 @@ struct ExpandParams {
     void *out;
     const int8_t *order;
     int64_t G, S, nb, ld;
-    int n, m, pat_bytes, bpt, transpose;   // bpt = blocks per tile
+    int n, m, c, pat_bytes, bpt, transpose;   // c = patterns, bpt = blocks per tile
 };
 
 template <typename T> __global__ __launch_bounds__(256) void expand_kernel(ExpandParams P)
@@ -576,25 +576,73 @@ template <typename T> __global__ __launch_bounds__(256) void expand_kernel(Expan
     const int64_t q0 = (int64_t)blockIdx.y * EX_L, b0 = (int64_t)blockIdx.x * P.bpt;
     const int rows = P.transpose ? tp : EX_L, cols = P.transpose ? EX_L : tp;
     const int pitch = (P.transpose ? EX_L : EX_P) + PAD;
-    for (int i = tid; i < rows * pitch; i += 256) tile[i] = Zero<T>::v();
-    __syncthreads();
-    const T *pv = (const T *)P.pk_val;
-    const int per_line = P.bpt * P.n;
-    for (int i = tid; i < EX_L * per_line; i += 256) {
-        const int ql = i / per_line, r = i - ql * per_line;
-        const int bl = r / P.n, j = r - bl * P.n;
-        const int64_t q = q0 + ql, b = b0 + bl;
-        if (q >= P.G || b >= P.nb) continue;
-        const int64_t blk = q * P.nb + b;
-        const int pat = P.pat_bytes == 1 ? (int)((const uint8_t *)P.pk_pat)[blk]
-                                         : (int)((const uint16_t *)P.pk_pat)[blk];
-        const int pos = bl * P.m + P.order[pat * P.n + j];
-        const T v = pv[blk * P.n + j];
-        if (P.transpose)
-            tile[pos * pitch + ql] = v;
-        else
-            tile[ql * pitch + pos] = v;
+    {
+        const uint4 z = {0, 0, 0, 0};
+        for (int i = tid; i < rows * pitch * (int)sizeof(T) / 16; i += 256) ((uint4 *)tile)[i] = z;   // pitch * sizeof(T) % 16 == 0
     }
+    // the order table in LDS where it fits: pattern -> order entry -> LDS store is otherwise a round
+    // trip to L2 per block
+    __shared__ int8_t s_ord[1024];
+    const int ord_n = P.c * P.n;
+    const bool ord_lds = ord_n <= 1024;
+    if (ord_lds)
+        for (int i = tid; i < ord_n; i += 256) s_ord[i] = P.order[i];
+    const int8_t *order = ord_lds ? s_ord : P.order;
+    __syncthreads();
+    // One item = one (line, block): its pattern number and its n values, the values as one word where
+    // n * sizeof(T) is 4 or 8.  The loads of four items are issued before the first item is placed.
+    const T *pv = (const T *)P.pk_val;
+    const int bpt = P.bpt, n = P.n, m = P.m;
+    const int items = EX_L * bpt;
+    // NV > 0: n is the constant NV and the values of a block are one aligned word of 4 or 8 bytes
+    auto place = [&](auto nv_tag) {
+        constexpr int NV = decltype(nv_tag)::value;
+        constexpr int WB = NV * (int)sizeof(T);
+        using Word = typename std::conditional<WB == 8, uint2, uint32_t>::type;
+        for (int base = tid; base < items; base += 4 * 256) {
+            int pat[4];
+            Word vw[4];
+            int64_t blk[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int it = base + u * 256;
+                const int ql = it / bpt, bl = it - ql * bpt;
+                const int64_t q = q0 + ql, b = b0 + bl;
+                const bool in = it < items && q < P.G && b < P.nb;
+                blk[u] = in ? q * P.nb + b : -1;
+                const int64_t at = in ? blk[u] : 0;
+                pat[u] = P.pat_bytes == 1 ? (int)((const uint8_t *)P.pk_pat)[at] : (int)((const uint16_t *)P.pk_pat)[at];
+                if (NV > 0) vw[u] = ((const Word *)pv)[at];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (blk[u] < 0) continue;
+                const int it = base + u * 256;
+                const int ql = it / bpt, bl = it - ql * bpt;
+                if constexpr (NV > 0) {
+                    T w[NV];
+                    __builtin_memcpy(w, &vw[u], WB);
+#pragma unroll
+                    for (int j = 0; j < NV; j++) {
+                        const int pos = bl * m + order[pat[u] * NV + j];
+                        tile[P.transpose ? pos * pitch + ql : ql * pitch + pos] = w[j];
+                    }
+                } else {
+                    for (int j = 0; j < n; j++) {
+                        const int pos = bl * m + order[pat[u] * n + j];
+                        tile[P.transpose ? pos * pitch + ql : ql * pitch + pos] = pv[blk[u] * n + j];
+                    }
+                }
+            }
+        }
+    };
+    const int vb = n * (int)sizeof(T);
+    const bool aligned = ((uintptr_t)pv % 8) == 0;
+    if (aligned && vb == 4 && n == 1) place(std::integral_constant<int, (sizeof(T) == 4 ? 1 : 0)>{});
+    else if (aligned && vb == 4 && n == 2) place(std::integral_constant<int, (sizeof(T) == 2 ? 2 : 0)>{});
+    else if (aligned && vb == 8 && n == 2) place(std::integral_constant<int, (sizeof(T) == 4 ? 2 : 0)>{});
+    else if (aligned && vb == 8 && n == 4) place(std::integral_constant<int, (sizeof(T) == 2 ? 4 : 0)>{});
+    else place(std::integral_constant<int, 0>{});
     __syncthreads();
     // rows of the tile -> global, 16 bytes per lane where the row is aligned
     T *out = (T *)P.out;
@@ -1039,6 +1087,7 @@ extern "C" int nmg_rowpack_expand(const void *d_pk_val, const void *d_pk_pat, in
     P.ld = ld_out;
     P.n = n;
     P.m = m;
+    P.c = (int)binom(m, n);
     P.pat_bytes = binom(m, n) <= 256 ? 1 : 2;
     P.bpt = EX_P / m;
     P.transpose = transpose ? 1 : 0;
