@@ -1500,7 +1500,10 @@ struct TiledParams {
     uint64_t magic_cols, magic_g;
 };
 
-template <typename T, bool GATHER>
+// GC: the group dim is the contiguous one instead (the reference's default orientation of a Linear
+// weight).  The region of NT tiles that are neighbours along the sparse dim is then NT*m rows (one
+// per position) of c*g contiguous columns; LDS holds it as [position][column].
+template <typename T, bool GATHER, bool GC>
 __global__ __launch_bounds__(256) void scatter_tiled_kernel(TiledParams Q)
 {
     const ScatterParams &P = Q.sp;
@@ -1516,21 +1519,26 @@ __global__ __launch_bounds__(256) void scatter_tiled_kernel(TiledParams Q)
     const int64_t t0 = (b * P.view.num_chunks + kc) * P.view.num_blocks + mb0;
     const int tiles = (int)min((int64_t)nt, P.view.num_blocks - mb0);
     const int64_t g0 = kc * cols, s0 = mb0 * m;
-    const int width = tiles * m;                       // positions of the region
-    const int rows = (int)min((int64_t)cols, P.view.G - g0);
-    const int valid_w = (int)max((int64_t)0, min((int64_t)width, P.view.S - s0));
-    T *dense = (T *)P.dense + b * P.view.stride_b + g0 * P.view.stride_g + s0;
+    // region: `all_rows` rows of `width` contiguous elements; rows / valid_w of them exist
+    const int width = GC ? cols : tiles * m;
+    const int all_rows = GC ? tiles * m : cols;
+    const int rows = GC ? (int)max((int64_t)0, min((int64_t)all_rows, P.view.S - s0))
+                        : (int)min((int64_t)cols, P.view.G - g0);
+    const int valid_w = GC ? (int)min((int64_t)cols, P.view.G - g0)
+                           : (int)max((int64_t)0, min((int64_t)width, P.view.S - s0));
+    const int64_t row_stride = GC ? P.view.stride_s : P.view.stride_g;
+    T *dense = (T *)P.dense + b * P.view.stride_b + g0 * P.view.stride_g + s0 * P.view.stride_s;
     constexpr int V = 16 / sizeof(T);
-    const bool vec = (P.view.stride_g % V) == 0 && (s0 % V) == 0 && (P.view.stride_b % V) == 0 &&
+    const bool vec = (row_stride % V) == 0 && ((GC ? g0 : s0) % V) == 0 && (P.view.stride_b % V) == 0 &&
                      ((uintptr_t)P.dense % 16) == 0 && (pitch % V) == 0;
     const int wv = (width + V - 1) / V;
 
     if (GATHER) {
         // region -> LDS (zeros beyond G / S)
-        for (int i = tid; i < cols * wv; i += 256) {
+        for (int i = tid; i < all_rows * wv; i += 256) {
             const int r = i / wv, cc = (i - r * wv) * V;
             T *dst = tile + r * pitch + cc;
-            const T *src = dense + (int64_t)r * P.view.stride_g + cc;
+            const T *src = dense + (int64_t)r * row_stride + cc;
             if (vec && r < rows && cc + V <= valid_w) {
                 *(uint4 *)dst = *(const uint4 *)src;
             } else {
@@ -1540,7 +1548,7 @@ __global__ __launch_bounds__(256) void scatter_tiled_kernel(TiledParams Q)
         }
     } else {
         const uint4 z = {0, 0, 0, 0};
-        for (int i = tid; i < cols * pitch * (int)sizeof(T) / 16; i += 256) ((uint4 *)tile)[i] = z;
+        for (int i = tid; i < all_rows * pitch * (int)sizeof(T) / 16; i += 256) ((uint4 *)tile)[i] = z;
     }
     // the order table in LDS where it fits: a slot's positions are then one LDS read away instead
     // of a round trip to L2 behind the load of its index
@@ -1579,25 +1587,27 @@ __global__ __launch_bounds__(256) void scatter_tiled_kernel(TiledParams Q)
                 const int p = (int)(((uint64_t)slot * Q.magic_g) >> 32);
                 const bool ok = o[u] >= 0 && o[u] < cols;
                 T *v = (T *)P.val + (at0 + e) * n;
-                T *row = tile + (ok ? o[u] : 0) * pitch + tm * m;
+                // element (column oc, position ps of tile tm) of the region
+                const int oc = ok ? o[u] : 0;
+                auto at = [&](int ps) { return GC ? (tm * m + ps) * pitch + oc : oc * pitch + tm * m + ps; };
                 if constexpr (NV > 0) {
                     T w[NV];
                     if (GATHER) {
 #pragma unroll
-                        for (int j = 0; j < NV; j++) w[j] = ok ? row[order[p * NV + j]] : Zero<T>::v();
+                        for (int j = 0; j < NV; j++) w[j] = ok ? tile[at(order[p * NV + j])] : Zero<T>::v();
                         Word raw;
                         __builtin_memcpy(&raw, w, WB);
                         ((Word *)P.val)[at0 + e] = raw;
                     } else if (ok) {
                         __builtin_memcpy(w, &vw[u], WB);
 #pragma unroll
-                        for (int j = 0; j < NV; j++) row[order[p * NV + j]] = w[j];
+                        for (int j = 0; j < NV; j++) tile[at(order[p * NV + j])] = w[j];
                     }
                 } else {
                     if (GATHER) {
-                        for (int j = 0; j < n; j++) v[j] = ok ? row[order[p * n + j]] : Zero<T>::v();
+                        for (int j = 0; j < n; j++) v[j] = ok ? tile[at(order[p * n + j])] : Zero<T>::v();
                     } else if (ok) {
-                        for (int j = 0; j < n; j++) row[order[p * n + j]] = v[j];
+                        for (int j = 0; j < n; j++) tile[at(order[p * n + j])] = v[j];
                     }
                 }
             }
@@ -1617,7 +1627,7 @@ __global__ __launch_bounds__(256) void scatter_tiled_kernel(TiledParams Q)
         const int r = i / wv, cc = (i - r * wv) * V;
         if (cc >= valid_w) continue;
         const T *src = tile + r * pitch + cc;
-        T *dst = dense + (int64_t)r * P.view.stride_g + cc;
+        T *dst = dense + (int64_t)r * row_stride + cc;
         if (vec && cc + V <= valid_w) {
             *(uint4 *)dst = *(const uint4 *)src;
         } else {
@@ -1631,7 +1641,8 @@ template <typename T>
 static int launch_scatter_tiled(bool gather, ScatterParams &P, hipStream_t s, bool *done)
 {
     *done = false;
-    if (P.view.stride_s != 1 || P.view.num_blocks < 4) return NMG_OK;
+    const bool gc = P.view.stride_s != 1 && P.view.stride_g == 1;   // group dim contiguous
+    if ((P.view.stride_s != 1 && !gc) || P.view.num_blocks < 4) return NMG_OK;
     // Tiles per workgroup: about 8 KiB of LDS (many small workgroups overlap each other's
     // latencies: a 16384 x 4096 2:4:16 gather takes 81 us with 10 tiles, 112 us with 64), but at
     // least 8 tiles so that a row of the region is a decent run of bytes, or 4 where 8 do not fit
@@ -1641,9 +1652,15 @@ static int launch_scatter_tiled(bool gather, ScatterParams &P, hipStream_t s, bo
     int nt = (int)std::min<int64_t>(64, (8 * 1024) / per_tile);
     if (nt < 8) nt = 8;
     nt = (int)std::min<int64_t>(nt, P.view.num_blocks);
-    auto pitch_of = [&](int tiles, bool pad) { return ((tiles * P.m + V - 1) / V) * V + (pad ? V : 0); };
+    auto pitch_of = [&](int tiles, bool pad) { return (((gc ? P.cols : tiles * P.m) + V - 1) / V) * V + (pad ? V : 0); };
     bool pad = true;
-    auto lds_of = [&](int tiles, bool pd) { return (size_t)P.cols * pitch_of(tiles, pd) * sizeof(T); };
+    auto lds_of = [&](int tiles, bool pd) {
+        return (size_t)(gc ? tiles * P.m : P.cols) * pitch_of(tiles, pd) * sizeof(T);
+    };
+    // group dim contiguous, gather: with one large workgroup per CU the slot-per-thread kernel is
+    // ahead (8192^2 2:8:32, 115 KB: 110 us against 70), so the region must stay under 64 KB
+    if (gc && gather && lds_of(nt, pad) > 64 * 1024) nt = (int)std::min<int64_t>(4, P.view.num_blocks);
+    if (gc && gather && lds_of(nt, pad) > 64 * 1024) return NMG_OK;
     if (lds_of(nt, pad) > 150 * 1024) nt = (int)std::min<int64_t>(4, P.view.num_blocks);
     if (lds_of(nt, pad) > 150 * 1024) pad = false;    // rows without the vector of padding
     if (lds_of(nt, pad) > 150 * 1024 || nt < 4) return NMG_OK;
@@ -1659,7 +1676,8 @@ static int launch_scatter_tiled(bool gather, ScatterParams &P, hipStream_t s, bo
     const int64_t chunks = P.outer / P.view.num_blocks;   // batches x group-dim chunks
     const int64_t grid = chunks * Q.groups_per_chunk;
     if (grid > 0x7fffffffLL) return NMG_OK;
-    auto kern = gather ? scatter_tiled_kernel<T, true> : scatter_tiled_kernel<T, false>;
+    auto kern = gc ? (gather ? scatter_tiled_kernel<T, true, true> : scatter_tiled_kernel<T, false, true>)
+                   : (gather ? scatter_tiled_kernel<T, true, false> : scatter_tiled_kernel<T, false, false>);
     if (lds > 64 * 1024)
         NMG_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, s, Q);
