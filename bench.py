@@ -11,8 +11,11 @@ kernel's average launch duration, measured with HIP events on the stream the ker
 on, against the dense fp16 MFMA peak -- i.e. the fraction of the density-scaled MFMA roofline.
 For the bandwidth-bound workloads (decode shapes, sparsifier) value = GB/s of algorithmic bytes
 (weight values + int16 indices + activations + output; dense input + val + idx for the
-sparsifier) and the roofline is HBM.  roofline.traffic is null: HBM traffic comes from rocprofv3
-counter runs, whose summaries are under profiles/ (config.traffic_profile names the file).
+sparsifier) and the roofline is HBM.  roofline.traffic is the HBM bytes per launch that the
+committed rocprofv3 counter summary of the workload reports (its `traffic_bytes_per_launch` line:
+FETCH_SIZE and WRITE_SIZE runs, scaled by a copy of known size; config.traffic_profile names the
+file under profiles/), null for a workload without such a summary -- the counters cannot be read
+from inside this process.
 With the default workload the same run also measures the other benchmark rows (config 2, config 3
 at 1:8 / 2:8 / 4:8, the decode shapes at 1, 4, 8 and 16 tokens, config 4 at 1, 4 and 16 tokens, the
 config 2 sparsifier and the config 5 training step without and with the optimizer update) with the
@@ -91,6 +94,21 @@ ALSO = [("c1", 50, 10), ("ref_f32", 20, 5), ("c2", 50, 10), ("c3_1_8", 20, 5), (
         ("decode_1", 50, 10), ("decode_4", 50, 10), ("decode_8", 50, 10), ("decode_16", 50, 10),
         ("c4_b1", 50, 10), ("c4_b4", 50, 10), ("c4_b16", 50, 10),
         ("sparsify_c2", 20, 5), ("c5_step", 10, 3), ("c5_train", 10, 3)]
+
+
+def profile_traffic(name):
+    """HBM bytes per launch from the `traffic_bytes_per_launch:` line of a committed counter summary."""
+    if not name:
+        return None
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", name)
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return float(line.split(":", 1)[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def cpu_baseline(M, K, N, n, m, g, seconds=15.0):
@@ -384,6 +402,7 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
     kern_ms = e0.elapsed_time(e1) / steps
     launch = "hip graph of the timed steps, replayed" if graph is not None else "eager"
 
+    traffic = profile_traffic(PMC_SUMMARIES.get(workload))
     row = {"ms_per_step": wall * 1e3, "kernel_ms": kern_ms, "launch": launch, "desc": desc, "kind": kind,
            "settle_steps": settle_steps,
            "shape": (M, K, N, n, m, g), "traffic_profile": PMC_SUMMARIES.get(workload)}
@@ -397,7 +416,7 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
             "value": dense_flops / wall / 1e12, "unit": "TFLOP/s",
             "effective_tflops": eff_flops / wall / 1e12,
             "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak,
-                         "unit": "TFLOP/s", "frac": achieved / peak, "traffic": None,
+                         "unit": "TFLOP/s", "frac": achieved / peak, "traffic": traffic,
                          "flops": "effective non-zero (2*M*K*N*n/m); dense-equivalent is m/n times this"},
         })
     else:
@@ -407,7 +426,7 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
             "value": algo_bytes / wall / 1e9, "unit": "GB/s",
             "algorithmic_bytes": algo_bytes, "weight_copies": copies,
             "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": achieved / PEAK_HBM_GBS, "traffic": None},
+                         "frac": achieved / PEAK_HBM_GBS, "traffic": traffic},
         })
     del step
     torch.cuda.empty_cache()
