@@ -261,29 +261,32 @@ class GroupedNMTensor:
             cache[reduce_dim] = df
         return df
 
-    def dense_operand(self, reduce_dim, cached=False):
+    def dense_operand(self, reduce_dim, cached=False, pad_k=1):
         """Dense copy [outputs, reduction] of the weight (transposed when the reduction runs along
         dim 0), expanded from the rowpack operand into fresh scratch.  ``cached``: kept until
         ``val`` changes, like the densefrag operand (``spmm_opt["cache_dense"] = False`` turns
-        that off)."""
+        that off).  ``pad_k``: the rows are padded with zeros to a multiple of it."""
         lay = self.layout
         keep = cached and self.spmm_opt.get("cache_dense", True)
         key = (self.val.data_ptr(), self.val._version, self.idx.data_ptr())
         cache = getattr(self, "_dense_operand", None)
         if cache is None or cache.get("key") != key:
             cache = self._dense_operand = {"key": key}
-        if keep and reduce_dim in cache:
-            return cache[reduce_dim]
-        pk_val, pk_pat = self.rowpack()
         O, K = lay.dense_shape[1 - reduce_dim], lay.dense_shape[reduce_dim]
-        out = torch.empty((O, K), dtype=self.val.dtype, device=self.val.device)
+        Kp = -(-K // pad_k) * pad_k
+        slot = reduce_dim if Kp == K else (reduce_dim, Kp)
+        if keep and slot in cache:
+            return cache[slot]
+        pk_val, pk_pat = self.rowpack()
+        alloc = torch.empty if Kp == K else torch.zeros
+        out = alloc((O, Kp), dtype=self.val.dtype, device=self.val.device)
         if keep:
-            cache[reduce_dim] = out
+            cache[slot] = out
         # rowpack lines run along the group dim; the scratch has the reduction dim contiguous
         transpose = 1 if lay.group_dim == reduce_dim else 0
         with torch.cuda.device(out.device):
             native.check(native.load().nmg_rowpack_expand(
-                native.ptr(pk_val), native.ptr(pk_pat), lay.G, lay.S, native.ptr(out), K, transpose,
+                native.ptr(pk_val), native.ptr(pk_pat), lay.G, lay.S, native.ptr(out), Kp, transpose,
                 lay.n, lay.m, native.dtype_code(out.dtype), native.stream_ptr(out.device)))
         return out
 
@@ -584,6 +587,25 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
             native.check(entry(
                 native.ptr(a), a.stride(0), native.ptr(x), x.stride(0), native.ptr(y), O, native.ptr(bias),
                 O, K, T, native.dtype_code(x.dtype), native.stream_ptr(x.device)))
+        return y
+    Kp = -(-K // 64) * 64
+    if (x.dtype in (torch.float16, torch.bfloat16) and T > 16 and kname == "auto" and len(lay.dense_shape) == 2
+            and weight.spmm_opt.get("expand", True) and O * Kp * 2 < 2 ** 31 and T * Kp * 2 < 2 ** 31):
+        # 16-bit shapes that none of the matrix-core routes above takes as they are (a reduction
+        # extent that is not a multiple of 64 or 8, an m such as 5 or 7, unaligned activations):
+        # a dense copy of the weight with zero-padded rows (kept per weight version) and, where
+        # needed, a zero-padded copy of the activations, through the dense 16-bit GEMM -- the
+        # kernel below runs at a hundredth of its rate
+        a = weight.dense_operand(reduce_dim, cached=True, pad_k=64)
+        if Kp != K or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
+            xp = x.new_zeros((T, Kp))
+            xp[:, :K] = x
+        else:
+            xp = x
+        with torch.cuda.device(x.device):
+            native.check(native.load().nmg_gemm_nt(
+                native.ptr(a), Kp, native.ptr(xp), xp.stride(0), native.ptr(y), O, native.ptr(bias),
+                O, Kp, T, native.dtype_code(x.dtype), native.stream_ptr(x.device)))
         return y
     pk_val, pk_pat = weight.rowpack()
     with torch.cuda.device(x.device):

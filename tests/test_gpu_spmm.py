@@ -430,6 +430,36 @@ def test_reference_matmul_test_shape_takes_the_dense_matrix_cores():
     assert rel_l2(to_np(gx), to_np(seeded((4096, 768), torch.float16, seed=5)).astype(np.float64) @ Wd) <= TOL[torch.float16]
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,K,T,n,m,g,sd", [
+    (300, 1001, 130, 2, 4, 16, 1),     # reduction not a multiple of 8: no sparse-core operand
+    (257, 520, 77, 4, 8, 4, 1),        # 4:8 with a reduction that is not a multiple of 64
+    (192, 455, 40, 2, 5, 3, 1),        # m = 5: no dense-core operand either
+    (130, 333, 64, 3, 7, 2, 0),        # the other orientation
+])
+def test_odd_16_bit_shapes_take_the_padded_dense_route(dtype, M, K, T, n, m, g, sd):
+    print(f"case padded expand {dtype} M={M} K={K} T={T} {n}:{m}:{g} sd={sd}", flush=True)
+    W = seeded((M, K), dtype, seed=M + K, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, sd)
+    w = make(W, n, m, g, sd)
+    x = seeded((T, K), dtype, seed=1)
+    b = seeded((M,), dtype, seed=2)
+    y = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)
+    assert rel_l2(to_np(y), to_np(x).astype(np.float64) @ Wd.T + to_np(b).astype(np.float64)) <= TOL[dtype]
+    assert any(isinstance(k, tuple) for k in getattr(w, "_dense_operand", {})), "the padded operand was not built"
+    gy = seeded((T, M), dtype, seed=3)
+    gx = sten.spmm(w, gy.to(DEV), reduce_dim=0)
+    assert rel_l2(to_np(gx), to_np(gy).astype(np.float64) @ Wd) <= TOL[dtype]
+    # a view of the activations with an odd pitch goes through a padded copy as well
+    xv = seeded((T, K + 3), dtype, seed=4).to(DEV)[:, 1:K + 1]
+    yv = sten.spmm(w, xv, reduce_dim=1)
+    assert rel_l2(to_np(yv), to_np(xv).astype(np.float64) @ Wd.T) <= TOL[dtype]
+    # the kernel that expands inside its loop stays reachable and agrees
+    w.spmm_opt["expand"] = False
+    y2 = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)
+    assert rel_l2(to_np(y2), to_np(y).astype(np.float64)) <= 2 * TOL[dtype]
+
+
 def test_reference_matmul_test_shape_in_single_precision():
     # the same sizes in the dtype of the reference's own test (fp32, dace_gnm_mult.py:1183): expand
     # once, then the fp32 matrix cores; B [K, N] and C [M, N] as torch.mm has them
