@@ -532,8 +532,16 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
                 x.stride(0) if T > 1 else K, native.ptr(y), O, native.ptr(bias), T,
                 native.dtype_code(x.dtype), variant, native.stream_ptr(x.device)))
         return y
-    dense16 = (T > 16 and x.dtype in (torch.float16, torch.bfloat16) and K % 64 == 0
-               and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and T * x.stride(0) * 2 < 2 ** 31)
+    # Few tokens as well when the choice is automatic: without a sparse-core operand (another
+    # pattern, the reduction along the group dim, fp32) the alternative for <= 16 tokens is the untuned
+    # streaming kernel.  4096 x 11008 at 1 / 4 / 16 tokens: 4:8 25 / 25 / 26 us on the dense-core
+    # operand with the reduction cut into slices against 63 / 119 / 342; 2:4 reduced along the
+    # group dim (the reference's default orientation) 24 / 25 / 26 against 1190 / 1203 / 1286; fp32
+    # 65 / 65 / 65 against 70 / 134 / 361.
+    min_t = 1 if kname == "auto" else 17
+    ldx = x.stride(0) if T > 1 else K      # the stride of a dim of extent 1 means nothing
+    dense16 = (T >= min_t and x.dtype in (torch.float16, torch.bfloat16) and K % 64 == 0
+               and ldx % 8 == 0 and x.data_ptr() % 16 == 0 and T * ldx * 2 < 2 ** 31)
     if (kname in ("auto", "mfma", "densefrag") and dense16
             and native.load().nmg_densefrag_supported(lay.n, lay.m)
             and (kname == "densefrag" or weight.spmm_opt.get("expand", True))):
@@ -543,20 +551,22 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
         lib = native.load()
         slices, ws_bytes = ctypes.c_int(1), ctypes.c_int64(0)
         if int(weight.spmm_opt.get("dense_variant", -1)) == -1:
-            native.check(lib.nmg_splitk_plan(O, K, T, ctypes.byref(slices), ctypes.byref(ws_bytes)))
+            # (the plan leaves 16 tokens and fewer to the streaming kernel of the sparse-core operand;
+            # here they are cut like 17)
+            native.check(lib.nmg_splitk_plan(O, K, max(T, 17), ctypes.byref(slices), ctypes.byref(ws_bytes)))
         slices = int(weight.spmm_opt.get("slices", slices.value))
         if slices > 1:
             # few tiles for the chip: the reduction is cut into slices, summed by a second kernel
             ws = torch.empty((slices * T * ((O + 255) // 256) * 256,), dtype=torch.float32, device=x.device)
             with torch.cuda.device(x.device):
                 native.check(lib.nmg_spmm_densefrag_splitk(
-                    native.ptr(df), O, K, native.ptr(x), x.stride(0), native.ptr(y), O, native.ptr(bias), T,
+                    native.ptr(df), O, K, native.ptr(x), ldx, native.ptr(y), O, native.ptr(bias), T,
                     native.dtype_code(x.dtype), slices, native.ptr(ws), ws.numel() * 4,
                     native.stream_ptr(x.device)))
             return y
         with torch.cuda.device(x.device):
             native.check(native.load().nmg_spmm_densefrag(
-                native.ptr(df), O, K, native.ptr(x), x.stride(0), native.ptr(y), O, native.ptr(bias), T,
+                native.ptr(df), O, K, native.ptr(x), ldx, native.ptr(y), O, native.ptr(bias), T,
                 native.dtype_code(x.dtype), int(weight.spmm_opt.get("dense_variant", -1)),
                 native.stream_ptr(x.device)))
         return y
@@ -571,10 +581,10 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
         a = weight.dense_operand(reduce_dim)
         with torch.cuda.device(x.device):
             native.check(native.load().nmg_gemm_nt(
-                native.ptr(a), K, native.ptr(x), x.stride(0), native.ptr(y), O, native.ptr(bias),
+                native.ptr(a), K, native.ptr(x), ldx, native.ptr(y), O, native.ptr(bias),
                 O, K, T, native.dtype_code(x.dtype), native.stream_ptr(x.device)))
         return y
-    if (x.dtype == torch.float32 and T > 16 and kname == "auto" and len(lay.dense_shape) == 2
+    if (x.dtype == torch.float32 and T >= min_t and kname == "auto" and len(lay.dense_shape) == 2
             and weight.spmm_opt.get("expand", True)):
         # single precision: "expand, then multiply" as well -- a dense copy of the weight (kept per
         # weight version) and the pipelined fp32 matrix-core kernel; the kernel below, which expands
@@ -585,19 +595,20 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
         entry = native.load().nmg_gemm_nt if reduce_dim == 1 else native.load().nmg_gemm_nn
         with torch.cuda.device(x.device):
             native.check(entry(
-                native.ptr(a), a.stride(0), native.ptr(x), x.stride(0), native.ptr(y), O, native.ptr(bias),
+                native.ptr(a), a.stride(0), native.ptr(x), ldx, native.ptr(y), O, native.ptr(bias),
                 O, K, T, native.dtype_code(x.dtype), native.stream_ptr(x.device)))
         return y
     Kp = -(-K // 64) * 64
-    if (x.dtype in (torch.float16, torch.bfloat16) and T > 16 and kname == "auto" and len(lay.dense_shape) == 2
+    if (x.dtype in (torch.float16, torch.bfloat16) and T >= 4 and kname == "auto" and len(lay.dense_shape) == 2
             and weight.spmm_opt.get("expand", True) and O * Kp * 2 < 2 ** 31 and T * Kp * 2 < 2 ** 31):
         # 16-bit shapes that none of the matrix-core routes above takes as they are (a reduction
         # extent that is not a multiple of 64 or 8, an m such as 5 or 7, unaligned activations):
         # a dense copy of the weight with zero-padded rows (kept per weight version) and, where
         # needed, a zero-padded copy of the activations, through the dense 16-bit GEMM -- the
-        # kernel below runs at a hundredth of its rate
+        # kernel below runs at a hundredth of its rate (from 4 tokens on: this GEMM does not cut its
+        # reduction, and at 1 token the streaming kernel below is ahead, 81 us against 132)
         a = weight.dense_operand(reduce_dim, cached=True, pad_k=64)
-        if Kp != K or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
+        if Kp != K or ldx % 8 != 0 or x.data_ptr() % 16 != 0:
             xp = x.new_zeros((T, Kp))
             xp[:, :K] = x
         else:

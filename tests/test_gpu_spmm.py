@@ -460,6 +460,32 @@ def test_odd_16_bit_shapes_take_the_padded_dense_route(dtype, M, K, T, n, m, g, 
     assert rel_l2(to_np(y2), to_np(y).astype(np.float64)) <= 2 * TOL[dtype]
 
 
+@pytest.mark.parametrize("T", [1, 3, 16])
+@pytest.mark.parametrize("dtype,M,K,n,m,g,sd", [
+    (torch.float16, 512, 1024, 4, 8, 4, 1),       # no sparse-core operand for 4:8
+    (torch.bfloat16, 768, 640, 2, 4, 16, 0),      # the reference's default orientation: reduction along the group dim
+    (torch.float16, 320, 1152, 3, 6, 12, 1),
+    (torch.float32, 512, 1024, 2, 4, 16, 1),      # fp32: dense copy + fp32 GEMM
+])
+def test_few_tokens_without_a_sparse_core_operand_take_the_dense_routes(dtype, M, K, n, m, g, sd, T):
+    print(f"case few tokens {dtype} M={M} K={K} {n}:{m}:{g} sd={sd} T={T}", flush=True)
+    W = seeded((M, K), dtype, seed=M + K, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, sd)
+    w = make(W, n, m, g, sd)
+    x = seeded((T, K), dtype, seed=T)
+    b = seeded((M,), dtype, seed=2)
+    y = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)
+    assert rel_l2(to_np(y), to_np(x).astype(np.float64) @ Wd.T + to_np(b).astype(np.float64)) <= TOL[dtype]
+    if dtype == torch.float32:
+        assert 1 in getattr(w, "_dense_operand", {}), "the dense copy was not built"
+    else:
+        assert getattr(w, "_densefrag", None) and 1 in w._densefrag, "the dense-core operand was not built"
+    # the streaming kernel stays reachable and agrees
+    alt = "skinny" if dtype != torch.float32 and sd == 1 else "mfma"
+    y2 = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1, kernel=alt)
+    assert rel_l2(to_np(y2), to_np(y).astype(np.float64)) <= 2 * TOL[dtype]
+
+
 def test_reference_matmul_test_shape_in_single_precision():
     # the same sizes in the dtype of the reference's own test (fp32, dace_gnm_mult.py:1183): expand
     # once, then the fp32 matrix cores; B [K, N] and C [M, N] as torch.mm has them
