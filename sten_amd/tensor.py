@@ -393,7 +393,7 @@ def _mm_f32_expanded(weight, b, reduce_dim):
     c = torch.empty((O, N), dtype=b.dtype, device=b.device)
     with torch.cuda.device(b.device):
         native.check(entry(
-            native.ptr(b), b.stride(0), native.ptr(wd), wd.stride(0), native.ptr(c), N, None, N, K, O,
+            native.ptr(b), b.stride(0) if K > 1 else N, native.ptr(wd), wd.stride(0), native.ptr(c), N, None, N, K, O,
             native.dtype_code(b.dtype), native.stream_ptr(b.device)))
     return c
 
@@ -486,6 +486,8 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
     if x.stride(1) != 1:
         x = x.contiguous()
     T = x.shape[0]
+    if T == 1 and x.stride(0) != K:
+        x = x.as_strided((1, K), (K, 1))    # the stride of a dim of extent 1 means nothing; give it the plain one
     y = torch.empty((T, O), dtype=x.dtype, device=x.device)
     if bias is not None:
         bias = bias.to(dtype=x.dtype).contiguous()
@@ -599,14 +601,16 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
                 O, K, T, native.dtype_code(x.dtype), native.stream_ptr(x.device)))
         return y
     Kp = -(-K // 64) * 64
-    if (x.dtype in (torch.float16, torch.bfloat16) and T >= 4 and kname == "auto" and len(lay.dense_shape) == 2
+    if (x.dtype in (torch.float16, torch.bfloat16) and T >= (4 if reduce_sparse == 1 else 1) and kname == "auto"
+            and len(lay.dense_shape) == 2
             and weight.spmm_opt.get("expand", True) and O * Kp * 2 < 2 ** 31 and T * Kp * 2 < 2 ** 31):
         # 16-bit shapes that none of the matrix-core routes above takes as they are (a reduction
         # extent that is not a multiple of 64 or 8, an m such as 5 or 7, unaligned activations):
         # a dense copy of the weight with zero-padded rows (kept per weight version) and, where
         # needed, a zero-padded copy of the activations, through the dense 16-bit GEMM -- the
-        # kernel below runs at a hundredth of its rate (from 4 tokens on: this GEMM does not cut its
-        # reduction, and at 1 token the streaming kernel below is ahead, 81 us against 132)
+        # kernel below runs at a hundredth of its rate (from 4 tokens on where the reduction runs
+        # along the sparse dim: this GEMM does not cut its reduction, and at 1 token the streaming kernel
+        # below is ahead, 81 us against 132; along the group dim that kernel takes 470 us at 4096^2)
         a = weight.dense_operand(reduce_dim, cached=True, pad_k=64)
         if Kp != K or ldx % 8 != 0 or x.data_ptr() % 16 != 0:
             xp = x.new_zeros((T, Kp))
@@ -615,7 +619,7 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
             xp = x
         with torch.cuda.device(x.device):
             native.check(native.load().nmg_gemm_nt(
-                native.ptr(a), Kp, native.ptr(xp), xp.stride(0), native.ptr(y), O, native.ptr(bias),
+                native.ptr(a), Kp, native.ptr(xp), xp.stride(0) if T > 1 else Kp, native.ptr(y), O, native.ptr(bias),
                 O, Kp, T, native.dtype_code(x.dtype), native.stream_ptr(x.device)))
         return y
     pk_val, pk_pat = weight.rowpack()

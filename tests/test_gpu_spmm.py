@@ -450,6 +450,11 @@ def test_odd_16_bit_shapes_take_the_padded_dense_route(dtype, M, K, T, n, m, g, 
     gy = seeded((T, M), dtype, seed=3)
     gx = sten.spmm(w, gy.to(DEV), reduce_dim=0)
     assert rel_l2(to_np(gx), to_np(gy).astype(np.float64) @ Wd) <= TOL[dtype]
+    # a single token along the group dim takes the padded route too (the streaming kernel has no form for it)
+    one = (gy if sd == 1 else x)[:1]
+    g1 = sten.spmm(w, one.to(DEV), reduce_dim=1 - sd)
+    ref1 = to_np(one).astype(np.float64) @ (Wd if sd == 1 else Wd.T)
+    assert rel_l2(to_np(g1), ref1) <= TOL[dtype]
     # a view of the activations with an odd pitch goes through a padded copy as well
     xv = seeded((T, K + 3), dtype, seed=4).to(DEV)[:, 1:K + 1]
     yv = sten.spmm(w, xv, reduce_dim=1)
