@@ -69,6 +69,8 @@ WORKLOADS = {
     "decode_4": ("decode", 4096, 11008, 4, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 4 tokens"),
     "decode_8": ("decode", 4096, 11008, 8, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 8 tokens"),
     "decode_16": ("decode", 4096, 11008, 16, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 16 tokens"),
+    "decode_gdim_1": ("decode_g", 4096, 11008, 1, 2, 4, 16, "W 4096x11008 fp16 2:4:16 with the n:m blocks along the outputs (the reference's default orientation) x 1 token: the reduction runs along the group dim, on the dense-core operand with the reduction cut into slices"),
+    "decode_gdim_16": ("decode_g", 4096, 11008, 16, 2, 4, 16, "the same x 16 tokens"),
     "decode_up_1": ("decode", 11008, 4096, 1, 2, 4, 16, "W 11008x4096 fp16 2:4:16 x 1 token (the up-projection beside the north_star shape)"),
     "decode_up_16": ("decode", 11008, 4096, 16, 2, 4, 16, "W 11008x4096 fp16 2:4:16 x 16 tokens"),
     "c4_b1": ("w4", 11008, 4096, 1, 2, 4, 1, "configs[3]: W 11008x4096 2:4 + int4 (scale per 128) x 1 token"),
@@ -92,6 +94,7 @@ PMC_SUMMARIES = {
 # measured beside the headline workload in the default run: (workload, steps, warm-up)
 ALSO = [("c1", 50, 10), ("ref_f32", 20, 5), ("c2", 50, 10), ("c3_1_8", 20, 5), ("c3_2_8", 20, 5), ("c3_4_8", 20, 5),
         ("decode_1", 50, 10), ("decode_4", 50, 10), ("decode_8", 50, 10), ("decode_16", 50, 10),
+        ("decode_gdim_1", 50, 10), ("decode_gdim_16", 50, 10),
         ("c4_b1", 50, 10), ("c4_b4", 50, 10), ("c4_b16", 50, 10),
         ("sparsify_c2", 20, 5), ("c5_step", 10, 3), ("c5_train", 10, 3)]
 
@@ -330,9 +333,10 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
     else:
         # weight values + one int16 index per (line, block) + activations + output
         algo_bytes = M * K * n // m * 2 + M * K // m * 2 + N * K * 2 + N * M * 2
-        if kind == "decode":
+        if kind in ("decode", "decode_g"):
             copies = copies_arg or -(-ROTATE_BYTES // algo_bytes)
-        ws = [sten.GroupedNMTensor.from_dense(W, n, m, sparse_dim=1, group_size=g, group_dim=0)
+        sdim, gdim = (0, 1) if kind == "decode_g" else (1, 0)
+        ws = [sten.GroupedNMTensor.from_dense(W, n, m, sparse_dim=sdim, group_size=g, group_dim=gdim)
               for _ in range(copies)]
         for w in ws:
             w.spmm_opt["variant"] = variant
@@ -360,7 +364,7 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
     # shapes keep the host busy for less than a step and are launched eagerly (--graph replays
     # them too).
     graph = None
-    short = kind in ("decode", "w4") or (kind == "fwd" and N <= 1024)
+    short = kind in ("decode", "decode_g", "w4") or (kind == "fwd" and N <= 1024)
     if (short and not eager) or (graph_large and kind not in ("step", "train", "sparsify")):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
