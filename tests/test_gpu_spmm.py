@@ -945,6 +945,35 @@ def test_hip_graph_replays_match_eager(M, K, T):
         assert torch.equal(got, want), f"replay with input seed {seed} differs from the eager call"
 
 
+@pytest.mark.parametrize("dtype,n,m,g,sd,T", [
+    (torch.float16, 2, 4, 16, 0, 4),      # reduction along the group dim, few tokens: dense-core operand in slices
+    (torch.float16, 4, 8, 4, 1, 16),      # no sparse-core operand
+    (torch.float32, 2, 4, 16, 1, 4),      # fp32: dense copy + fp32 GEMM
+    (torch.float32, 2, 4, 16, 1, 300),
+])
+def test_hip_graph_replays_of_the_dense_routes_match_eager(dtype, n, m, g, sd, T):
+    # the split reduction allocates its workspace inside the capture; every replay is checked
+    # against an eager call, with eager work and synchronisations between the replays
+    print(f"case graph replay dense routes {dtype} {n}:{m}:{g} sd={sd} T={T}", flush=True)
+    M, K = 1024, 2048
+    w = make(seeded((M, K), dtype, seed=31, std=0.05), n, m, g, sd)
+    x = seeded((T, K), dtype, seed=32).to(DEV)
+    b = seeded((M,), dtype, seed=33).to(DEV)
+    sten.spmm(w, x, b, reduce_dim=1)           # first call: tables and operand caches are set up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = sten.spmm(w, x, b, reduce_dim=1)
+    for seed in (40, 41, 42):
+        x.copy_(seeded((T, K), dtype, seed=seed).to(DEV))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = y.clone()
+        want = sten.spmm(w, x, b, reduce_dim=1)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay with input seed {seed} differs from the eager call"
+
+
 def test_tile_boundary_sweep_default_route():
     # The reference sweeps every size across each tile boundary +-1 (matmul_generator.py:1482-1521).
     # Here the boundaries are those of the default kernels: 32 / 64 / 256 lines, 16 / 128 / 256
