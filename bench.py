@@ -7,15 +7,16 @@ operand resident in HBM.
 
 Prints one JSON line.  For the matmul workloads value = dense-equivalent TFLOP/s (2*M*K*N / step
 time) and roofline.achieved counts the effective (non-zero) flops 2*M*K*N*n/m per launch over the
-kernel's average launch duration, measured with HIP events on the stream the kernel is launched
-on, against the dense fp16 MFMA peak -- i.e. the fraction of the density-scaled MFMA roofline.
+kernel's launch duration (the median over the timed steps, one HIP event pair per step on the
+stream the kernel is launched on), against the dense fp16 MFMA peak -- i.e. the fraction of the
+density-scaled MFMA roofline.
 For the bandwidth-bound workloads (decode shapes, sparsifier) value = GB/s of algorithmic bytes
 (weight values + int16 indices + activations + output; dense input + val + idx for the
 sparsifier) and the roofline is HBM.  roofline.traffic is the HBM bytes per launch that the
 committed rocprofv3 counter summary of the workload reports (its `traffic_bytes_per_launch` line:
-FETCH_SIZE and WRITE_SIZE runs, scaled by a copy of known size; config.traffic_profile names the
-file under profiles/), null for a workload without such a summary -- the counters cannot be read
-from inside this process.
+FETCH_SIZE and WRITE_SIZE runs, scaled by a copy of known size; roofline.traffic_source names the
+file under profiles/ and says that the figure is not measured by this run), null for a workload
+without such a summary -- the counters cannot be read from inside this process.
 With the default workload the same run also measures the other benchmark rows (config 2, config 3
 at 1:8 / 2:8 / 4:8, the decode shapes at 1, 4, 8 and 16 tokens, config 4 at 1, 4 and 16 tokens, the
 config 2 sparsifier and the config 5 training step without and with the optimizer update) with the
@@ -26,10 +27,18 @@ cpu_baseline (headline and config 2) = the CPU restatement of the reference's AV
 for the sparsifier workloads the restatement of the reference's single-threaded sort-and-scan on
 a slab of the weight.
 
+Timing protocol: `warmup` untimed steps, more untimed steps until 80 ms of load have passed, then
+the K timed steps, each between its own pair of HIP events; reported are the median, the minimum
+and the maximum of the K durations (the roofline uses the median) and ms_per_step = wall clock of
+the K steps / K between two synchronisations.  The decode shapes replay their steps from a HIP
+graph (events cannot be recorded into one): there a timed iteration is one replay of a graph of
+GRAPH_STEPS steps, divided by GRAPH_STEPS, and the median is over K such replays.
+
 Other modes: --workload picks another benchmark shape; --calibrate-copy runs a plain device copy
 of known size (the counter calibration for FETCH_SIZE / WRITE_SIZE).
 """
 import argparse
+import gc
 import json
 import os
 import sys
@@ -44,6 +53,7 @@ PEAK_FP32_TFLOPS = 157.3    # MI355X dense fp32 MFMA
 ROTATE_BYTES = 512 * 1024 * 1024
 PEAK_HBM_GBS = 8000.0
 SETTLE_S = 0.08                # untimed load before the timed steps (see measure())
+GRAPH_STEPS = 20               # steps per replayed HIP graph (decode shapes)
 FP32_WORKLOADS = ("c1", "ref_f32", "big_f32")
 
 WORKLOADS = {
@@ -96,7 +106,7 @@ ALSO = [("c1", 50, 10), ("ref_f32", 20, 5), ("c2", 50, 10), ("c3_1_8", 20, 5), (
         ("decode_1", 50, 10), ("decode_4", 50, 10), ("decode_8", 50, 10), ("decode_16", 50, 10),
         ("decode_gdim_1", 50, 10), ("decode_gdim_16", 50, 10),
         ("c4_b1", 50, 10), ("c4_b4", 50, 10), ("c4_b16", 50, 10),
-        ("sparsify_c2", 20, 5), ("c5_step", 10, 3), ("c5_train", 10, 3)]
+        ("sparsify_c2", 20, 5), ("sparsify_c3_2_8", 20, 5), ("c5_step", 20, 3), ("c5_train", 20, 3)]
 
 
 def profile_traffic(name):
@@ -179,10 +189,18 @@ def matrix_ceiling(iters=4000):
     instructions of a 128 x 128 x 64 slab per wavefront, issued from registers, no memory traffic in
     the loop), per instruction, on all-zero operands (the instruction's issue rate) and on N(0,1)
     operands (what the power limit leaves).  TFLOP/s, dense-equivalent for the sparse instructions."""
+    import ctypes
     import torch
     from sten_amd import native
 
-    lib = native.load()
+    path = os.path.join(ROOT, "sten_amd", "libnmg_probe.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it with `python -m sten_amd.build`")
+    lib = ctypes.CDLL(path)
+    lib.nmg_probe_matrix_rate.restype = ctypes.c_int
+    lib.nmg_probe_matrix_rate.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
+    lib.nmg_probe_matrix_rate_flops.restype = ctypes.c_int64
+    lib.nmg_probe_matrix_rate_flops.argtypes = [ctypes.c_int, ctypes.c_int]
     dev = "cuda:0"
     torch.manual_seed(0)
     ops = {"random": torch.randn(512 * 1024, device=dev).half(), "zero": torch.zeros(512 * 1024, device=dev).half()}
@@ -194,7 +212,8 @@ def matrix_ceiling(iters=4000):
         flops = lib.nmg_probe_matrix_rate_flops(kind, iters)
         for label, src in ops.items():
             def launch():
-                native.check(lib.nmg_probe_matrix_rate(kind, native.ptr(src), native.ptr(out), iters, stream))
+                if lib.nmg_probe_matrix_rate(kind, native.ptr(src), native.ptr(out), iters, stream) != 0:
+                    raise RuntimeError(f"nmg_probe_matrix_rate refused kind {kind}")
             settle_end = time.perf_counter() + SETTLE_S
             while time.perf_counter() < settle_end:
                 launch()
@@ -206,56 +225,6 @@ def matrix_ceiling(iters=4000):
             e1.record()
             torch.cuda.synchronize()
             res[name][label] = flops / (e0.elapsed_time(e1) / 3 * 1e-3) / 1e12
-    return res
-
-
-MIX_KINDS = [
-    "dense 256x256, V_MFMA_F32_32X32X16: MFMAs alone", "dense 256x256, 32X32X16: + LDS reads",
-    "dense 256x256, 32X32X16: + LDS reads, weight loads, DMA loads",
-    "dense 256x256, V_MFMA_F32_16X16X32: MFMAs alone", "dense 256x256, 16X16X32: + LDS reads",
-    "dense 256x256, 16X16X32: + LDS reads, weight loads, DMA loads",
-    "dense 256x256, 32X32X16, eight wavefronts: everything", "dense 256x256, 16X16X32, eight wavefronts: everything",
-    "sparse 256x256, V_SMFMAC_F32_32X32X32: everything", "sparse 256x256, V_SMFMAC_F32_16X16X64: everything",
-    "sparse 256x128, 32X32X32: MFMAs alone", "sparse 256x128, 32X32X32: + LDS reads",
-    "sparse 256x128, 32X32X32: + LDS reads, weight loads, DMA loads", "sparse 256x128, 32X32X32: without the DMA loads",
-    "sparse 256x128, 32X32X32: without the weight loads", "sparse 256x128, 32X32X32: without the index loads",
-    "sparse 256x128, 32X32X32: wavefronts 2 x 2", "sparse 256x128, 16X16X64: MFMAs alone",
-    "sparse 256x128, 16X16X64: + LDS reads, weight loads, DMA loads",
-    "sparse 256x256, 32X32X32: MFMAs alone", "sparse 256x256, 16X16X64: MFMAs alone",
-]
-
-
-def instruction_mix(steps=2048):
-    """What a K step of the large-batch kernels costs beyond its matrix instructions
-    (nmg_probe_instruction_mix: the step's instruction mix on L2-resident N(0,1) data, parts of it
-    left out, the instruction exchanged).  TFLOP/s over the chip, dense-equivalent."""
-    import torch
-    from sten_amd import native
-
-    lib = native.load()
-    dev = "cuda:0"
-    torch.manual_seed(0)
-    data = torch.randn(8 * 1024 * 1024, device=dev).half()
-    out = torch.empty(256 * 512, dtype=torch.float32, device=dev)
-    stream = native.stream_ptr(out.device)
-    res = {}
-    for kind, name in enumerate(MIX_KINDS):
-        flops = lib.nmg_probe_instruction_mix_flops(kind, steps)
-
-        def launch():
-            native.check(lib.nmg_probe_instruction_mix(kind, native.ptr(data), data.numel() * 2, native.ptr(out),
-                                                       out.numel(), steps, stream))
-        settle_end = time.perf_counter() + SETTLE_S
-        while time.perf_counter() < settle_end:
-            launch()
-            torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(5):
-            launch()
-        e1.record()
-        torch.cuda.synchronize()
-        res[name] = round(flops / (e0.elapsed_time(e1) / 5 * 1e-3) / 1e12, 1)
     return res
 
 
@@ -364,21 +333,17 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
     # shapes keep the host busy for less than a step and are launched eagerly (--graph replays
     # them too).
     graph = None
+    per = 1                      # steps per timed iteration
     short = kind in ("decode", "decode_g", "w4") or (kind == "fwd" and N <= 1024)
     if (short and not eager) or (graph_large and kind not in ("step", "train", "sparsify")):
+        per = max(GRAPH_STEPS, copies)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            for _ in range(steps):
+            for _ in range(per):
                 step()
         graph.replay()
         torch.cuda.synchronize()
-
-    def run_steps():
-        if graph is not None:
-            graph.replay()
-        else:
-            for _ in range(steps):
-                step()
+    run_once = graph.replay if graph is not None else step
 
     # Settling: after an idle spell the chip's power management overshoots -- the headline kernel
     # runs at 104 us for its first 2 ms, at 118-125 us for the next 10 ms and at 104 us from then
@@ -388,27 +353,36 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
     settle_end = time.perf_counter() + SETTLE_S
     settle_steps = 0
     while time.perf_counter() < settle_end:
-        run_steps()
+        for _ in range(steps):
+            run_once()
         torch.cuda.synchronize()
-        settle_steps += steps
+        settle_steps += steps * per
 
-    # The timed region: K back-to-back steps between two synchronisations.  The average duration
-    # of a step on the device comes from one HIP event pair around the same K steps, recorded on
-    # the stream they are launched on (torch's current stream).
+    # The timed region: K back-to-back iterations between two synchronisations, each between its
+    # own pair of HIP events recorded on the stream the kernels are launched on (torch's current
+    # stream): event i+1 closes iteration i and opens iteration i+1, so the K durations add up to
+    # the whole region.  The median is what the roofline uses; min and max are reported beside it.
     stream = torch.cuda.current_stream()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    events = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    gc.collect()
+    gc.disable()            # no collector pause of the host inside the timed region
     t0 = time.perf_counter()
-    e0.record(stream)
-    run_steps()
-    e1.record(stream)
+    events[0].record(stream)
+    for i in range(steps):
+        run_once()
+        events[i + 1].record(stream)
     torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / steps
-    kern_ms = e0.elapsed_time(e1) / steps
-    launch = "hip graph of the timed steps, replayed" if graph is not None else "eager"
+    wall = (time.perf_counter() - t0) / (steps * per)
+    gc.enable()
+    durs = sorted(events[i].elapsed_time(events[i + 1]) / per for i in range(steps))
+    kern_ms = durs[len(durs) // 2] if len(durs) % 2 else 0.5 * (durs[len(durs) // 2 - 1] + durs[len(durs) // 2])
+    launch = (f"hip graph of {per} steps, replayed once per timed iteration" if graph is not None else "eager")
 
     traffic = profile_traffic(PMC_SUMMARIES.get(workload))
-    row = {"ms_per_step": wall * 1e3, "kernel_ms": kern_ms, "launch": launch, "desc": desc, "kind": kind,
-           "settle_steps": settle_steps,
+    traffic_source = (f"profiles/{PMC_SUMMARIES[workload]} (committed rocprofv3 --pmc summary of this workload; "
+                      "not measured by this run)") if traffic is not None else None
+    row = {"ms_per_step": wall * 1e3, "kernel_ms": kern_ms, "kernel_ms_min": durs[0], "kernel_ms_max": durs[-1],
+           "launch": launch, "desc": desc, "kind": kind, "settle_steps": settle_steps,
            "shape": (M, K, N, n, m, g), "traffic_profile": PMC_SUMMARIES.get(workload)}
     if kind in ("fwd", "grad_x", "step", "train"):
         dense_flops = 2.0 * M * K * N * (3 if kind in ("step", "train") else 1)
@@ -420,7 +394,7 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
             "value": dense_flops / wall / 1e12, "unit": "TFLOP/s",
             "effective_tflops": eff_flops / wall / 1e12,
             "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak,
-                         "unit": "TFLOP/s", "frac": achieved / peak, "traffic": traffic,
+                         "unit": "TFLOP/s", "frac": achieved / peak, "traffic": traffic, "traffic_source": traffic_source,
                          "flops": "effective non-zero (2*M*K*N*n/m); dense-equivalent is m/n times this"},
         })
     else:
@@ -430,7 +404,7 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
             "value": algo_bytes / wall / 1e9, "unit": "GB/s",
             "algorithmic_bytes": algo_bytes, "weight_copies": copies,
             "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": achieved / PEAK_HBM_GBS, "traffic": traffic},
+                         "frac": achieved / PEAK_HBM_GBS, "traffic": traffic, "traffic_source": traffic_source},
         })
     del step
     torch.cuda.empty_cache()
@@ -453,8 +427,6 @@ def main():
     ap.add_argument("--matrix-ceiling", action="store_true",
                     help="only measure what the matrix cores sustain from registers, per instruction")
     ap.add_argument("--no-ceiling", action="store_true", help="skip that measurement in the default run")
-    ap.add_argument("--instruction-mix", action="store_true",
-                    help="only measure what a K step of the large-batch kernels costs beyond its MFMAs")
     ap.add_argument("--copies", type=int, default=0,
                     help="decode shapes: separate copies of the weight that the steps take in turn "
                          "(0: as many as exceed 512 MiB, so that no step finds its weight in a cache)")
@@ -467,9 +439,6 @@ def main():
         return
     if args.matrix_ceiling:
         print(json.dumps({"matrix_ceiling_tflops": matrix_ceiling()}))
-        return
-    if args.instruction_mix:
-        print(json.dumps({"instruction_mix_tflops": instruction_mix()}, indent=1))
         return
 
     row = measure(args.workload, args.steps, args.warmup, args.kernel, args.variant, args.eager, args.graph,
@@ -484,7 +453,10 @@ def main():
         "config": {"workload": desc, "kernel": args.kernel, "variant": args.variant, "launch": row["launch"],
                    "settle": f"{row['settle_steps']} more untimed steps ({SETTLE_S * 1e3:.0f} ms of load) between the "
                              "warm-up and the timed steps: the clocks dip for 10-60 ms after an idle spell",
-                   "kernel_ms": row["kernel_ms"], "traffic_profile": row["traffic_profile"]},
+                   "kernel_ms": row["kernel_ms"], "kernel_ms_min": row["kernel_ms_min"],
+                   "kernel_ms_max": row["kernel_ms_max"],
+                   "timing": "kernel_ms = median over the timed steps, one HIP event pair per step; "
+                             "ms_per_step = wall clock of the timed steps / steps"},
         "roofline": row["roofline"],
     }
     for key in ("effective_tflops", "algorithmic_bytes", "weight_copies"):
@@ -507,7 +479,8 @@ def main():
         also = {}
         for name, steps, warmup in ALSO:
             r = measure(name, steps, warmup)
-            also[name] = {"us": r["kernel_ms"] * 1e3, "value": r["value"], "unit": r["unit"],
+            also[name] = {"us": r["kernel_ms"] * 1e3, "us_min": r["kernel_ms_min"] * 1e3,
+                          "us_max": r["kernel_ms_max"] * 1e3, "steps": steps, "value": r["value"], "unit": r["unit"],
                           "frac": r["roofline"]["frac"], "bound": r["roofline"]["bound"]}
         out["config"]["also"] = also
     if not args.no_cpu and args.workload in ("c1", "c2", "target_2_4"):

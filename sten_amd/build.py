@@ -7,8 +7,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libnmg_hip.so")
 SOURCES = ["nmg_runtime.hip", "nmg_sparsify.hip", "nmg_spmm.hip", "nmg_smfmac.hip", "nmg_dense.hip",
-           "nmg_densefrag.hip", "nmg_w4.hip", "nmg_pack.hip", "nmg_sddmm.hip", "nmg_perfect.hip", "nmg_probe.hip",
-           "nmg_probe_mix.hip"]
+           "nmg_densefrag.hip", "nmg_w4.hip", "nmg_pack.hip", "nmg_sddmm.hip", "nmg_perfect.hip"]
+# bench.py's measurement aid: a library of its own, outside the product ABI
+PROBE_LIB = os.path.join(HERE, "libnmg_probe.so")
+PROBE_SOURCES = ["nmg_probe.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -25,9 +27,10 @@ def build(verbose=False, jobs=8, check=True):
     os.makedirs(objdir, exist_ok=True)
     procs = []
     objs = []
-    for src in SOURCES:
+    for src in SOURCES + PROBE_SOURCES:
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        objs.append(obj)
+        if src in SOURCES:
+            objs.append(obj)
         cmd = [hipcc] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), file=sys.stderr)
@@ -37,6 +40,8 @@ def build(verbose=False, jobs=8, check=True):
     _drain(procs)
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB]
     subprocess.run(cmd, check=True)
+    probe_objs = [os.path.join(objdir, src.replace(".hip", ".o")) for src in PROBE_SOURCES]
+    subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + probe_objs + ["-o", PROBE_LIB], check=True)
     if check:
         from . import isa_check
         if isa_check.main([]) != 0:

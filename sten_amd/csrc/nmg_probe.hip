@@ -6,14 +6,19 @@
 // The measured rates are what a product kernel's fraction of the nominal peak has to be read
 // against (gfx950, MI355X, measured: dense f16 32x32x16 1.71 PFLOP/s on random operands and 2.45 on
 // zeros, 16x16x32 1.94 / 2.43; sparse 32x32x32 2.6 / 3.6 dense-equivalent, 16x16x64 3.45 / 4.9).
-#include "nmg_common.h"
-#include "nmg_tile.h"
+// Built into its own library (libnmg_probe.so, declared in include/nmg_probe.h): it serves bench.py
+// only and is not part of the product's C ABI.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/nmg_probe.h"
 
 namespace nmg {
 
 typedef _Float16 pb_f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 pb_f16x16 __attribute__((ext_vector_type(16)));
 typedef float pb_f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 // KIND 0: V_MFMA_F32_32X32X16_F16, 1: V_MFMA_F32_16X16X32_F16,
 //      2: V_SMFMAC_F32_32X32X32_F16, 3: V_SMFMAC_F32_16X16X64_F16
@@ -126,10 +131,10 @@ extern "C" int64_t nmg_probe_matrix_rate_flops(int kind, int iters)
 
 extern "C" int nmg_probe_matrix_rate(int kind, const void *d_operands, float *d_out, int iters, void *stream)
 {
-    NMG_REQUIRE(kind >= 0 && kind <= 3, NMG_ERR_ARG, "unknown instruction kind %d", kind);
-    NMG_REQUIRE(iters >= 1 && iters <= (1 << 24), NMG_ERR_ARG, "iters out of range");
-    NMG_REQUIRE(d_operands && d_out, NMG_ERR_ARG, "null device pointer");
-    NMG_REQUIRE(((uintptr_t)d_operands % 16) == 0, NMG_ERR_ARG, "operands must be 16-byte aligned");
+    // 1: bad argument, 2: the launch failed
+    if (kind < 0 || kind > 3 || iters < 1 || iters > (1 << 24) || !d_operands || !d_out ||
+        ((uintptr_t)d_operands % 16) != 0)
+        return 1;
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid(PB_GROUPS), block(256);
     const pb_f16x8 *src = (const pb_f16x8 *)d_operands;
@@ -139,6 +144,5 @@ extern "C" int nmg_probe_matrix_rate(int kind, const void *d_operands, float *d_
     case 2: hipLaunchKernelGGL(probe_kernel<2>, grid, block, 0, s, src, d_out, iters); break;
     default: hipLaunchKernelGGL(probe_kernel<3>, grid, block, 0, s, src, d_out, iters); break;
     }
-    NMG_HIP_TRY(hipGetLastError());
-    return NMG_OK;
+    return hipGetLastError() == hipSuccess ? 0 : 2;
 }

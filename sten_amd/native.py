@@ -73,10 +73,6 @@ SIGNATURES = {
     "nmg_perfect_nm": (_I, [_P, _I64, _I64, _I64, _P, _P, _I, _I, _I, _P]),
     "nmg_perfect_nm_to_dense": (_I, [_P, _P, _I64, _I64, _I64, _P, _I, _I, _I, _P]),
     "nmg_noalloc_scratch_bytes": (_I64, []),
-    "nmg_probe_matrix_rate": (_I, [_I, _P, _P, _I, _P]),
-    "nmg_probe_matrix_rate_flops": (_I64, [_I, _I]),
-    "nmg_probe_instruction_mix": (_I, [_I, _P, _I64, _P, _I64, _I, _P]),
-    "nmg_probe_instruction_mix_flops": (_I64, [_I, _I]),
     "nmg_noalloc_prepare": (_I, []),
     "nmg_spmm_smfmac_splitk_noalloc": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _P]),
     "nmg_spmm_smfmac_tt": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _P]),

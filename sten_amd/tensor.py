@@ -7,6 +7,7 @@ a GPU: ``dtype`` / ``device`` / ``shape`` / ``to``, same-pattern re-compression
 All compute goes through libnmg_hip.so; tensors must live on the GPU.
 """
 import ctypes
+import weakref
 
 import torch
 
@@ -24,6 +25,23 @@ class GroupedNMTensor:
         self.layout = layout
         self.spmm_opt = {"kernel": "auto"}
         self._rowpack = None
+
+    def _version_key(self):
+        """Identity and version of ``val`` and ``idx``: what every derived operand depends on.  The
+        tensors are named by weak reference, not by address -- the allocator hands a freed block
+        back at the same address, and tensors written by the library's kernels all carry version 0."""
+        return (weakref.ref(self.val), self.val._version, weakref.ref(self.idx), self.idx._version)
+
+    def _key_current(self, key):
+        return (key is not None and key[0]() is self.val and key[1] == self.val._version
+                and key[2]() is self.idx and key[3] == self.idx._version)
+
+    def _drop_operands(self):
+        """Forget every operand derived from ``val`` (in-place updates call this)."""
+        self._rowpack = None
+        self._fragpack = None
+        self._densefrag = None
+        self._dense_operand = None
 
     # ---- construction ----------------------------------------------------------------------
     @staticmethod
@@ -148,12 +166,15 @@ class GroupedNMTensor:
         if other.idx is self.idx or (other.idx.data_ptr() == self.idx.data_ptr()
                                      and other.idx.shape == self.idx.shape):
             return True
-        key = (other.idx.data_ptr(), other.idx._version, self.idx._version)
         cached = getattr(self, "_pattern_eq", None)
-        if cached is None or cached[0] != key:
-            same = other.idx.device == self.idx.device and bool(torch.equal(other.idx, self.idx))
-            self._pattern_eq = cached = (key, same)
-        return cached[1]
+        if (cached is not None and cached[0]() is other.idx and cached[1] == other.idx._version
+                and cached[2] == self.idx._version):
+            return cached[3]
+        same = other.idx.device == self.idx.device and bool(torch.equal(other.idx, self.idx))
+        # remembered per tensor object (weak reference), not per address: a freed idx block comes
+        # back at the same address with another pattern in it
+        self._pattern_eq = (weakref.ref(other.idx), other.idx._version, self.idx._version, same)
+        return same
 
     def _other_val(self, other):
         if isinstance(other, GroupedNMTensor):
@@ -175,22 +196,22 @@ class GroupedNMTensor:
 
     def add_(self, other, *, alpha=1):
         self.val.add_(self._other_val(other), alpha=alpha)
-        self._rowpack = None
+        self._drop_operands()
         return self
 
     def mul_(self, other):
         self.val.mul_(self._other_val(other))
-        self._rowpack = None
+        self._drop_operands()
         return self
 
     def zero_(self):
         self.val.zero_()
-        self._rowpack = None
+        self._drop_operands()
         return self
 
     def copy_(self, other):
         self.val.copy_(self._other_val(other))
-        self._rowpack = None
+        self._drop_operands()
         return self
 
     # ---- matmul operand ---------------------------------------------------------------------------
@@ -200,9 +221,9 @@ class GroupedNMTensor:
         lay = self.layout
         if len(lay.dense_shape) != 2:
             raise native.NmgError("matmul needs a 2-D grouped n:m tensor")
-        key = (self.val.data_ptr(), self.val._version, self.idx.data_ptr())
-        if self._rowpack is not None and self._rowpack[0] == key:
+        if self._rowpack is not None and self._key_current(self._rowpack[0]):
             return
+        key = self._version_key()
         native.require_gpu(self.val)
         lib = native.load()
         dev, dt = self.val.device, self.val.dtype
@@ -240,11 +261,10 @@ class GroupedNMTensor:
         the compressed format."""
         lay = self.layout
         lib = native.load()
-        key = (self.val.data_ptr(), self.val._version, self.idx.data_ptr())
         keep = self.spmm_opt.get("cache_dense", True)
         cache = getattr(self, "_densefrag", None)
-        if cache is None or cache.get("key") != key or not keep:
-            cache = self._densefrag = {"key": key}
+        if cache is None or not self._key_current(cache.get("key")) or not keep:
+            cache = self._densefrag = {"key": self._version_key()}
         if reduce_dim in cache:
             return cache[reduce_dim]
         pk_val, pk_pat = self.rowpack()
@@ -268,10 +288,9 @@ class GroupedNMTensor:
         that off).  ``pad_k``: the rows are padded with zeros to a multiple of it."""
         lay = self.layout
         keep = cached and self.spmm_opt.get("cache_dense", True)
-        key = (self.val.data_ptr(), self.val._version, self.idx.data_ptr())
         cache = getattr(self, "_dense_operand", None)
-        if cache is None or cache.get("key") != key:
-            cache = self._dense_operand = {"key": key}
+        if cache is None or not self._key_current(cache.get("key")):
+            cache = self._dense_operand = {"key": self._version_key()}
         O, K = lay.dense_shape[1 - reduce_dim], lay.dense_shape[reduce_dim]
         Kp = -(-K // pad_k) * pad_k
         slot = reduce_dim if Kp == K else (reduce_dim, Kp)
@@ -280,14 +299,14 @@ class GroupedNMTensor:
         pk_val, pk_pat = self.rowpack()
         alloc = torch.empty if Kp == K else torch.zeros
         out = alloc((O, Kp), dtype=self.val.dtype, device=self.val.device)
-        if keep:
-            cache[slot] = out
         # rowpack lines run along the group dim; the scratch has the reduction dim contiguous
         transpose = 1 if lay.group_dim == reduce_dim else 0
         with torch.cuda.device(out.device):
             native.check(native.load().nmg_rowpack_expand(
                 native.ptr(pk_val), native.ptr(pk_pat), lay.G, lay.S, native.ptr(out), Kp, transpose,
                 lay.n, lay.m, native.dtype_code(out.dtype), native.stream_ptr(out.device)))
+        if keep:
+            cache[slot] = out       # only an operand that was written is kept
         return out
 
     def slotmap(self):
@@ -297,10 +316,10 @@ class GroupedNMTensor:
         lay = self.layout
         if len(lay.dense_shape) != 2:
             raise native.NmgError("the slot map needs a 2-D grouped n:m tensor")
-        key = (self.idx.data_ptr(), self.idx._version)
         cached = getattr(self, "_slotmap", None)
-        if cached is not None and cached[0] == key:
+        if cached is not None and cached[0][0]() is self.idx and cached[0][1] == self.idx._version:
             return cached[1]
+        key = (weakref.ref(self.idx), self.idx._version)
         native.require_gpu(self.idx)
         slot = torch.empty((lay.num_blocks, lay.num_chunks * lay.cols), dtype=torch.int16, device=self.idx.device)
         with torch.cuda.device(slot.device):
@@ -358,7 +377,8 @@ class GroupedNMTensor:
                       for t in (rows_op, cols_op)))
         if reduction_last:
             return ok and rows_op.shape[1] % 8 == 0 and max(rows_op.stride(0), cols_op.stride(0)) < 2 ** 22
-        return ok and lay.dense_shape[0] % 8 == 0 and lay.dense_shape[1] % 8 == 0
+        return (ok and lay.dense_shape[0] % 8 == 0 and lay.dense_shape[1] % 8 == 0
+                and max(rows_op.stride(0), cols_op.stride(0)) < 2 ** 25)
 
     def fragpack(self):
         """Operand of the sparse-matrix-core kernel (values + 2-bit positions in instruction
@@ -375,12 +395,15 @@ class GroupedNMTensor:
                 f"device={self.val.device})")
 
 
+F32_GEMM_MAX_TOKENS = 65535 * 32      # one launch of the fp32 GEMM: token tiles of 32 in grid.y
+
+
 def _mm_f32_expanded(weight, b, reduce_dim):
     """op(W) @ B in single precision with B and the result as they lie in memory: the dense copy of
     the weight (kept per weight version; the same one for both directions) as the row operand of
     the fp32 matrix-core GEMM, B as its reduction-major operand.  None when the route does not apply."""
     if (b.dtype != torch.float32 or b.shape[1] <= 16 or weight.spmm_opt.get("kernel", "auto") != "auto"
-            or not weight.spmm_opt.get("expand", True)):
+            or not weight.spmm_opt.get("expand", True) or b.shape[1] > F32_GEMM_MAX_TOKENS):
         return None
     lay = weight.layout
     K, O = lay.dense_shape[reduce_dim], lay.dense_shape[1 - reduce_dim]
@@ -587,7 +610,7 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
                 O, K, T, native.dtype_code(x.dtype), native.stream_ptr(x.device)))
         return y
     if (x.dtype == torch.float32 and T >= min_t and kname == "auto" and len(lay.dense_shape) == 2
-            and weight.spmm_opt.get("expand", True)):
+            and weight.spmm_opt.get("expand", True) and T <= F32_GEMM_MAX_TOKENS):
         # single precision: "expand, then multiply" as well -- a dense copy of the weight (kept per
         # weight version) and the pipelined fp32 matrix-core kernel; the kernel below, which expands
         # inside its reduction loop, runs at a tenth of that rate
@@ -612,7 +635,7 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
         # along the sparse dim: this GEMM does not cut its reduction, and at 1 token the streaming kernel
         # below is ahead, 81 us against 132; along the group dim that kernel takes 470 us at 4096^2)
         a = weight.dense_operand(reduce_dim, cached=True, pad_k=64)
-        if Kp != K or ldx % 8 != 0 or x.data_ptr() % 16 != 0:
+        if Kp != K or ldx % 8 != 0 or x.data_ptr() % 16 != 0 or T * ldx * 2 >= 2 ** 31:
             xp = x.new_zeros((T, Kp))
             xp[:, :K] = x
         else:

@@ -15,7 +15,8 @@ from helpers import oracle_sparsify, rel_l2, same_bits, to_np
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
-# rel-L2 against fp64: fp16 / bf16 inputs with fp32 accumulation, fp32 inputs
+# rel-L2 against fp64: fp16 and fp32 as the benchmark contract states them (1e-3 with fp32
+# accumulation, 1e-5); it states none for bf16, which has three mantissa bits fewer than fp16: 8 x 1e-3
 TOL = {torch.float16: 1e-3, torch.bfloat16: 8e-3, torch.float32: 1e-5}
 
 
@@ -53,16 +54,16 @@ def one_case(rng, big):
         ref = to_np(X).astype(np.float64) @ (Wd64.T if rd == 1 else Wd64)
         if b is not None:
             ref = ref + to_np(b).astype(np.float64)
-        assert rel_l2(to_np(y), ref) <= 2 * TOL[dt], f"spmm reduce_dim={rd}"
+        assert rel_l2(to_np(y), ref) <= TOL[dt], f"spmm reduce_dim={rd}"
     # torch.mm(W, B) and its gradient with respect to B, operands as they lie in memory
     B = torch.randn((C, T), generator=gen).to(dt)
     prod = sten.spmm_tt(w, B.to(DEV))
     assert prod.shape == (R, T)
-    assert rel_l2(to_np(prod), Wd64 @ to_np(B).astype(np.float64)) <= 2 * TOL[dt], "W @ B"
+    assert rel_l2(to_np(prod), Wd64 @ to_np(B).astype(np.float64)) <= TOL[dt], "W @ B"
     G = torch.randn((R, T), generator=gen).to(dt)
     gB = sten.spmm_tt_dense(w, G.to(DEV), reduce_dim=0)
     assert gB.shape == (C, T)
-    assert rel_l2(to_np(gB), Wd64.T @ to_np(G).astype(np.float64)) <= 2 * TOL[dt], "W^T @ G"
+    assert rel_l2(to_np(gB), Wd64.T @ to_np(G).astype(np.float64)) <= TOL[dt], "W^T @ G"
     if dt != torch.float32 and R % 8 == 0 and C % 8 == 0:
         gy = torch.randn((T, R), generator=gen).to(dt)
         x = torch.randn((T, C), generator=gen).to(dt)
@@ -81,7 +82,7 @@ def one_case(rng, big):
         gw = _masked_weight_grad(w, gy.to(DEV), x.to(DEV))
         full = to_np(gy).astype(np.float64).T @ to_np(x).astype(np.float64)
         ref = O.gather_merged(O.merge(full, lay), idx, lay.n)
-        assert rel_l2(to_np(gw.val).astype(np.float64), ref) <= 2 * TOL[dt], "fp32 weight gradient"
+        assert rel_l2(to_np(gw.val).astype(np.float64), ref) <= TOL[dt], "fp32 weight gradient"
     pv, pi = O.perfect_nm(to_np(W), n, m, sd)
     p = sten.PerfectNMTensor.from_dense(W.to(DEV), n, m, sparse_dim=sd)
     assert same_bits(p.val, pv) and np.array_equal(to_np(p.idx), pi), "ungrouped n:m"

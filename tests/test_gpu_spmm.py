@@ -209,6 +209,42 @@ def test_in_place_updates_with_an_independently_sparsified_tensor():
     assert torch.equal(a.val, (before + 2.0) + 2.0)
 
 
+def test_pattern_comparison_is_not_remembered_by_address():
+    # The comparison of two idx tensors is remembered per tensor object.  A tensor with an equal
+    # pattern is freed, and a tensor with another pattern, created right after it, gets its idx at
+    # the freed address (same size, caching allocator) with version 0 like every kernel output: the
+    # remembered "equal" must not be served for it.
+    a = make(seeded((96, 64), torch.float32, seed=1), 2, 4, 4, 1)
+    da = a.to_dense().clone()
+    mask = a.clone_layout(torch.ones(96, 64, device=DEV)).to_dense() != 0
+    twin = sten.GroupedNMTensor(a.val.clone(), a.idx.clone(), a.layout)
+    old_ptr = twin.idx.data_ptr()
+    a.add_(twin)                                   # equal pattern: slot by slot, and remembered
+    assert torch.equal(a.to_dense(), da + da)
+    del twin
+    b = make(seeded((96, 64), torch.float32, seed=2), 2, 4, 4, 1)
+    hit = b.idx.data_ptr() == old_ptr
+    other = b if hit else sten.GroupedNMTensor(b.val, b.idx.clone(), b.layout)
+    assert not torch.equal(other.idx, a.idx)
+    db = other.to_dense().clone()
+    a.add_(other)
+    assert torch.equal(a.to_dense(), torch.where(mask, da + da + db, torch.zeros_like(da))), \
+        f"idx of the second tensor at the freed address: {hit}"
+
+
+def test_derived_operands_follow_in_place_changes_of_the_pattern():
+    # the matmul operands are keyed on the versions of val and idx: a pattern written in place
+    # (idx.copy_) must not leave the operands of the old pattern behind
+    a = make(seeded((128, 64), torch.float16, seed=3), 2, 4, 16, 1)
+    b = make(seeded((128, 64), torch.float16, seed=4), 2, 4, 16, 1)
+    x = seeded((32, 64), torch.float16, seed=5).to(DEV)
+    y0 = sten.spmm(a, x, reduce_dim=1)
+    a.idx.copy_(b.idx)
+    a.val.copy_(b.val)
+    assert torch.equal(sten.spmm(a, x, reduce_dim=1), sten.spmm(b, x, reduce_dim=1))
+    assert not torch.equal(y0, sten.spmm(a, x, reduce_dim=1))
+
+
 def test_unregistered_op_raises_in_raise_mode():
     sten.set_dispatch_failure("raise")
     w = sten.SparseTensorWrapper.wrapped_from_dense(
@@ -1046,38 +1082,3 @@ def test_direct_kernels_on_a_full_chip_with_a_long_reduction():
         for _ in range(4):
             got = sten.spmm(w, g, reduce_dim=0, kernel="densefrag").float()
             assert float((got - want).norm() / want.norm()) <= 1e-4, f"dense variant {dense_variant}"
-
-
-def test_matrix_rate_probe_runs_every_instruction():
-    # measurement aid of bench.py: launches and finishes for every kind, refuses a bad one
-    lib = native.load()
-    src = torch.randn(512 * 1024, device=DEV).half()
-    out = torch.empty(256 * 1024, dtype=torch.float32, device=DEV)
-    for kind in range(4):
-        print(f"case matrix rate probe kind {kind}", flush=True)
-        assert lib.nmg_probe_matrix_rate_flops(kind, 10) == 2 * 128 * 128 * 64 * 10 * 4096
-        native.check(lib.nmg_probe_matrix_rate(kind, native.ptr(src), native.ptr(out), 10, None))
-    torch.cuda.synchronize()
-    assert bool(torch.isfinite(out).all())
-    assert lib.nmg_probe_matrix_rate(7, native.ptr(src), native.ptr(out), 10, None) == 1
-    assert lib.nmg_probe_matrix_rate_flops(7, 10) == -1
-
-
-def test_instruction_mix_probe_runs_every_kind():
-    # measurement aid of bench.py: launches and finishes for every kind, refuses bad arguments
-    lib = native.load()
-    data = torch.randn(8 * 1024 * 1024, device=DEV).half()
-    out = torch.empty(256 * 512, dtype=torch.float32, device=DEV)
-    for kind in range(21):
-        print(f"case instruction mix {kind}", flush=True)
-        tok = 128 if 10 <= kind <= 18 else 256
-        assert lib.nmg_probe_instruction_mix_flops(kind, 4) == 2 * 256 * tok * 64 * 4 * 256
-        native.check(lib.nmg_probe_instruction_mix(kind, native.ptr(data), data.numel() * 2, native.ptr(out),
-                                                   out.numel(), 4, None))
-    torch.cuda.synchronize()
-    assert bool(torch.isfinite(out).all())
-    args = (native.ptr(data), data.numel() * 2, native.ptr(out), out.numel())
-    assert lib.nmg_probe_instruction_mix(21, *args, 4, None) == 1          # unknown kind
-    assert lib.nmg_probe_instruction_mix(0, *args, 3, None) == 1           # odd step count
-    assert lib.nmg_probe_instruction_mix(0, native.ptr(data), 1 << 20, native.ptr(out), out.numel(), 4, None) == 1
-    assert lib.nmg_probe_instruction_mix_flops(21, 4) == -1
