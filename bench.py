@@ -28,11 +28,12 @@ for the sparsifier workloads the restatement of the reference's single-threaded 
 a slab of the weight.
 
 Timing protocol: `warmup` untimed steps, more untimed steps until 80 ms of load have passed, then
-the K timed steps, each between its own pair of HIP events; reported are the median, the minimum
-and the maximum of the K durations (the roofline uses the median) and ms_per_step = wall clock of
-the K steps / K between two synchronisations.  The decode shapes replay their steps from a HIP
-graph (events cannot be recorded into one): there a timed iteration is one replay of a graph of
-GRAPH_STEPS steps, divided by GRAPH_STEPS, and the median is over K such replays.
+the K timed steps back to back between two synchronisations, cut by HIP events into groups that
+last about 0.5 ms each (one step where a step is longer; see measure()).  Reported are the median,
+the minimum and the maximum over the groups of duration / steps in the group (the roofline uses the
+median), the mean from the first to the last event, and ms_per_step = wall clock of the K steps /
+K.  The decode shapes replay their steps from a HIP graph (events cannot be recorded into one): a
+timed iteration is one replay of a graph of GRAPH_STEPS steps, divided by GRAPH_STEPS.
 
 Other modes: --workload picks another benchmark shape; --calibrate-copy runs a plain device copy
 of known size (the counter calibration for FETCH_SIZE / WRITE_SIZE).
@@ -79,7 +80,9 @@ WORKLOADS = {
     "decode_4": ("decode", 4096, 11008, 4, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 4 tokens"),
     "decode_8": ("decode", 4096, 11008, 8, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 8 tokens"),
     "decode_16": ("decode", 4096, 11008, 16, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 16 tokens"),
-    "decode_gdim_1": ("decode_g", 4096, 11008, 1, 2, 4, 16, "W 4096x11008 fp16 2:4:16 with the n:m blocks along the outputs (the reference's default orientation) x 1 token: the reduction runs along the group dim, on the dense-core operand with the reduction cut into slices"),
+    "decode_gdim_1": ("decode_g", 4096, 11008, 1, 2, 4, 16, "W 4096x11008 fp16 2:4:16 with the n:m blocks along the outputs (the reference's default orientation) x 1 token: the reduction runs along the group dim, the compressed lines are streamed and expanded in registers"),
+    "decode_gdim_4": ("decode_g", 4096, 11008, 4, 2, 4, 16, "the same x 4 tokens"),
+    "decode_gdim_8": ("decode_g", 4096, 11008, 8, 2, 4, 16, "the same x 8 tokens"),
     "decode_gdim_16": ("decode_g", 4096, 11008, 16, 2, 4, 16, "the same x 16 tokens"),
     "decode_up_1": ("decode", 11008, 4096, 1, 2, 4, 16, "W 11008x4096 fp16 2:4:16 x 1 token (the up-projection beside the north_star shape)"),
     "decode_up_16": ("decode", 11008, 4096, 16, 2, 4, 16, "W 11008x4096 fp16 2:4:16 x 16 tokens"),
@@ -102,11 +105,11 @@ PMC_SUMMARIES = {
 }
 
 # measured beside the headline workload in the default run: (workload, steps, warm-up)
-ALSO = [("c1", 50, 10), ("ref_f32", 20, 5), ("c2", 50, 10), ("c3_1_8", 20, 5), ("c3_2_8", 20, 5), ("c3_4_8", 20, 5),
+ALSO = [("c1", 50, 10), ("ref_f32", 80, 5), ("c2", 240, 10), ("c3_1_8", 40, 5), ("c3_2_8", 40, 5), ("c3_4_8", 40, 5),
         ("decode_1", 50, 10), ("decode_4", 50, 10), ("decode_8", 50, 10), ("decode_16", 50, 10),
         ("decode_gdim_1", 50, 10), ("decode_gdim_16", 50, 10),
         ("c4_b1", 50, 10), ("c4_b4", 50, 10), ("c4_b16", 50, 10),
-        ("sparsify_c2", 20, 5), ("sparsify_c3_2_8", 20, 5), ("c5_step", 20, 3), ("c5_train", 20, 3)]
+        ("sparsify_c2", 100, 5), ("sparsify_c3_2_8", 20, 5), ("c5_step", 20, 3), ("c5_train", 20, 3)]
 
 
 def profile_traffic(name):
@@ -352,36 +355,54 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
     # see the clocks a workload that keeps running sees.
     settle_end = time.perf_counter() + SETTLE_S
     settle_steps = 0
+    est = 1.0
     while time.perf_counter() < settle_end:
+        ts = time.perf_counter()
         for _ in range(steps):
             run_once()
         torch.cuda.synchronize()
+        est = (time.perf_counter() - ts) / steps      # seconds per timed iteration, roughly
         settle_steps += steps * per
 
-    # The timed region: K back-to-back iterations between two synchronisations, each between its
-    # own pair of HIP events recorded on the stream the kernels are launched on (torch's current
-    # stream): event i+1 closes iteration i and opens iteration i+1, so the K durations add up to
-    # the whole region.  The median is what the roofline uses; min and max are reported beside it.
+    # The timed region: K back-to-back iterations between two synchronisations.  HIP events on the
+    # stream the kernels are launched on (torch's current stream) cut the region into groups of
+    # consecutive iterations, every group between its own pair of events: event g+1 closes group g
+    # and opens group g+1, so the durations add up to the whole region.  A group is one iteration
+    # where an iteration lasts 0.5 ms or more and as many as fill about 0.5 ms otherwise (at most a
+    # quarter of K): an event marker between two kernels keeps the second from starting under the
+    # tail of the first and costs 5-7 us, which a 0.1 ms kernel shows as 7 % (measured: headline
+    # 102 us with a marker after every launch, 95 us back to back, 95.5 us in the rocprofv3 kernel
+    # trace).  The median over the groups is what the roofline uses -- one stall of the host or the
+    # allocator lands in one group and does not move it -- min and max are reported beside it.
+    group = max(1, min(int(round(0.5e-3 / max(est, 1e-9))), max(1, steps // 4)))
+    bounds = list(range(0, steps, group))
+    if len(bounds) > 1 and steps - bounds[-1] < group:
+        bounds.pop()                                   # the last group takes the leftover iterations
+    bounds.append(steps)
     stream = torch.cuda.current_stream()
-    events = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    events = [torch.cuda.Event(enable_timing=True) for _ in bounds]
     gc.collect()
     gc.disable()            # no collector pause of the host inside the timed region
     t0 = time.perf_counter()
     events[0].record(stream)
-    for i in range(steps):
-        run_once()
-        events[i + 1].record(stream)
+    for g in range(len(bounds) - 1):
+        for _ in range(bounds[g], bounds[g + 1]):
+            run_once()
+        events[g + 1].record(stream)
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / (steps * per)
     gc.enable()
-    durs = sorted(events[i].elapsed_time(events[i + 1]) / per for i in range(steps))
+    durs = sorted(events[g].elapsed_time(events[g + 1]) / ((bounds[g + 1] - bounds[g]) * per)
+                  for g in range(len(bounds) - 1))
     kern_ms = durs[len(durs) // 2] if len(durs) % 2 else 0.5 * (durs[len(durs) // 2 - 1] + durs[len(durs) // 2])
+    kern_mean = events[0].elapsed_time(events[-1]) / (steps * per)
     launch = (f"hip graph of {per} steps, replayed once per timed iteration" if graph is not None else "eager")
 
     traffic = profile_traffic(PMC_SUMMARIES.get(workload))
     traffic_source = (f"profiles/{PMC_SUMMARIES[workload]} (committed rocprofv3 --pmc summary of this workload; "
                       "not measured by this run)") if traffic is not None else None
     row = {"ms_per_step": wall * 1e3, "kernel_ms": kern_ms, "kernel_ms_min": durs[0], "kernel_ms_max": durs[-1],
+           "kernel_ms_mean": kern_mean, "timed_groups": len(durs), "steps_per_group": group * per,
            "launch": launch, "desc": desc, "kind": kind, "settle_steps": settle_steps,
            "shape": (M, K, N, n, m, g), "traffic_profile": PMC_SUMMARIES.get(workload)}
     if kind in ("fwd", "grad_x", "step", "train"):
@@ -455,7 +476,11 @@ def main():
                              "warm-up and the timed steps: the clocks dip for 10-60 ms after an idle spell",
                    "kernel_ms": row["kernel_ms"], "kernel_ms_min": row["kernel_ms_min"],
                    "kernel_ms_max": row["kernel_ms_max"],
-                   "timing": "kernel_ms = median over the timed steps, one HIP event pair per step; "
+                   "kernel_ms_mean": row["kernel_ms_mean"], "timed_groups": row["timed_groups"],
+                   "steps_per_group": row["steps_per_group"],
+                   "timing": "the timed steps are cut into groups by HIP events (a group lasts about 0.5 ms, one step "
+                             "where a step is longer); kernel_ms = median over the groups of duration / steps in "
+                             "the group, min / max beside it, kernel_ms_mean = first to last event / steps; "
                              "ms_per_step = wall clock of the timed steps / steps"},
         "roofline": row["roofline"],
     }
@@ -480,7 +505,8 @@ def main():
         for name, steps, warmup in ALSO:
             r = measure(name, steps, warmup)
             also[name] = {"us": r["kernel_ms"] * 1e3, "us_min": r["kernel_ms_min"] * 1e3,
-                          "us_max": r["kernel_ms_max"] * 1e3, "steps": steps, "value": r["value"], "unit": r["unit"],
+                          "us_max": r["kernel_ms_max"] * 1e3, "us_mean": r["kernel_ms_mean"] * 1e3,
+                          "groups": r["timed_groups"], "steps_per_group": r["steps_per_group"], "value": r["value"], "unit": r["unit"],
                           "frac": r["roofline"]["frac"], "bound": r["roofline"]["bound"]}
         out["config"]["also"] = also
     if not args.no_cpu and args.workload in ("c1", "c2", "target_2_4"):

@@ -286,17 +286,17 @@ template <typename T> __global__ __launch_bounds__(256) void splitk_sum_kernel(S
     if (gid >= P.T * quads) return;
     const int64_t tok = gid / quads, f = (gid - tok * quads) * 4;
     const float *src = P.part + tok * P.part_ld + f;
-    // four slices are fetched at a time (the kernel is a chain of round trips to L2 / HBM
-    // otherwise) and added in slice order
+    // sixteen slices are fetched at a time (the kernel is a chain of round trips to memory otherwise:
+    // the sums were written through other L2s) and added in slice order
     const int64_t step = P.T * P.part_ld;
     float4 sum = {0.f, 0.f, 0.f, 0.f};
-    for (int s0 = 0; s0 < P.slices; s0 += 4) {
-        float4 v[4];
+    for (int s0 = 0; s0 < P.slices; s0 += 16) {
+        float4 v[16];
 #pragma unroll
-        for (int u = 0; u < 4; u++)
+        for (int u = 0; u < 16; u++)
             v[u] = s0 + u < P.slices ? *(const float4 *)(src + (int64_t)(s0 + u) * step) : float4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < 16; u++) {
             sum.x += v[u].x;
             sum.y += v[u].y;
             sum.z += v[u].z;

@@ -35,6 +35,7 @@ CHECKED = {
     "nmg_smfmac.hip": ["spmm_smfmac_direct_kernel", "decode_staged_kernel"],
     "nmg_w4.hip": ["w4_linear_staged_kernel"],
     "nmg_sddmm.hip": ["sddmm16_kernel"],
+    "nmg_gstream.hip": ["gstream_kernel"],
 }
 
 REG = re.compile(r"\b([va])(\d+)\b|\b([va])\[(\d+):(\d+)\]")

@@ -395,6 +395,7 @@ class GroupedNMTensor:
                 f"device={self.val.device})")
 
 
+GSTREAM_MAX_TOKENS = 16               # nmg_spmm_gstream: tokens up to which the stream of the weight bounds the product
 F32_GEMM_MAX_TOKENS = 65535 * 32      # one launch of the fp32 GEMM: token tiles of 32 in grid.y
 
 
@@ -565,6 +566,28 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
     # 65 / 65 / 65 against 70 / 134 / 361.
     min_t = 1 if kname == "auto" else 17
     ldx = x.stride(0) if T > 1 else K      # the stride of a dim of extent 1 means nothing
+    # Few tokens with the reduction along the group dim (what F.linear does with a weight in the
+    # reference's default orientation): the compressed lines are streamed once and expanded in
+    # registers -- 56 MB instead of the 90 MB of the dense-core operand for 4096 x 11008 at 2:4.
+    if (kname in ("auto", "gstream") and reduce_sparse == 0 and T <= GSTREAM_MAX_TOKENS
+            and x.dtype in (torch.float16, torch.bfloat16) and len(lay.dense_shape) == 2
+            and native.load().nmg_spmm_gstream_supported(lay.n, lay.m)
+            and K % 8 == 0 and ldx % 8 == 0 and x.data_ptr() % 16 == 0 and T * ldx * 2 < 2 ** 31
+            and lay.num_blocks % (16 // lay.m) == 0):
+        lib = native.load()
+        pk_val, pk_pat = weight.rowpack()
+        slices, ws_bytes = ctypes.c_int(1), ctypes.c_int64(0)
+        native.check(lib.nmg_spmm_gstream_plan(K, O, T, lay.n, lay.m, ctypes.byref(slices), ctypes.byref(ws_bytes)))
+        ws = torch.empty((max(ws_bytes.value, 4) // 4,), dtype=torch.float32, device=x.device)
+        with torch.cuda.device(x.device):
+            native.check(lib.nmg_spmm_gstream(
+                native.ptr(pk_val), native.ptr(pk_pat), K, O, native.ptr(x), ldx, native.ptr(y), O,
+                native.ptr(bias), T, lay.n, lay.m, native.dtype_code(x.dtype), native.ptr(ws), ws.numel() * 4,
+                native.stream_ptr(x.device)))
+        return y
+    if kname == "gstream":
+        raise native.NmgError("the streaming product along the group dim needs 16-bit data, at most "
+                              f"{GSTREAM_MAX_TOKENS} tokens, m = 4 or 8 with n = 1 or 2 and a reduction extent that is a multiple of 8")
     dense16 = (T >= min_t and x.dtype in (torch.float16, torch.bfloat16) and K % 64 == 0
                and ldx % 8 == 0 and x.data_ptr() % 16 == 0 and T * ldx * 2 < 2 ** 31)
     if (kname in ("auto", "mfma", "densefrag") and dense16

@@ -504,7 +504,7 @@ def test_odd_16_bit_shapes_take_the_padded_dense_route(dtype, M, K, T, n, m, g, 
 @pytest.mark.parametrize("T", [1, 3, 16])
 @pytest.mark.parametrize("dtype,M,K,n,m,g,sd", [
     (torch.float16, 512, 1024, 4, 8, 4, 1),       # no sparse-core operand for 4:8
-    (torch.bfloat16, 768, 640, 2, 4, 16, 0),      # the reference's default orientation: reduction along the group dim
+    (torch.bfloat16, 760, 640, 2, 4, 16, 0),      # the reference's default orientation (reduction along the group dim) with 190 blocks: not whole groups of 4
     (torch.float16, 320, 1152, 3, 6, 12, 1),
     (torch.float32, 512, 1024, 2, 4, 16, 1),      # fp32: dense copy + fp32 GEMM
 ])
@@ -525,6 +525,50 @@ def test_few_tokens_without_a_sparse_core_operand_take_the_dense_routes(dtype, M
     alt = "skinny" if dtype != torch.float32 and sd == 1 else "mfma"
     y2 = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1, kernel=alt)
     assert rel_l2(to_np(y2), to_np(y).astype(np.float64)) <= 2 * TOL[dtype]
+
+
+@pytest.mark.parametrize("T", [1, 3, 16])
+@pytest.mark.parametrize("dtype,M,K,n,m,g", [
+    (torch.float16, 768, 640, 2, 4, 16),       # three spans of 256 outputs, 640 lines
+    (torch.bfloat16, 768, 640, 2, 4, 16),
+    (torch.float16, 272, 328, 1, 4, 8),        # 68 blocks: part of a span; 41 groups of 8 lines
+    (torch.float16, 512, 1000, 2, 8, 4),
+    (torch.bfloat16, 1040, 2056, 1, 8, 32),    # 130 blocks of 8, ragged chunks of the group dim
+    (torch.float16, 4096, 2816, 2, 4, 16),     # sixteen spans, several slices of the reduction
+])
+def test_few_tokens_along_the_group_dim_stream_the_compressed_lines(dtype, M, K, n, m, g, T):
+    # F.linear with a weight in the reference's default orientation (n:m blocks along the outputs):
+    # the reduction runs along the group dim; <= 16 tokens stream the rowpack operand
+    print(f"case gstream {dtype} M={M} K={K} {n}:{m}:{g} T={T}", flush=True)
+    W = seeded((M, K), dtype, seed=M + K, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, 0)
+    w = make(W, n, m, g, 0)
+    x = seeded((T, K), dtype, seed=T)
+    b = seeded((M,), dtype, seed=2)
+    ref = to_np(x).astype(np.float64) @ Wd.T
+    y = sten.spmm(w, x.to(DEV), reduce_dim=1)
+    assert rel_l2(to_np(y), ref) <= TOL[dtype]
+    assert not getattr(w, "_densefrag", None), "the dense-core operand was built"
+    yb = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1, kernel="gstream")
+    assert rel_l2(to_np(yb), ref + to_np(b).astype(np.float64)) <= TOL[dtype]
+    # a view with a row pitch (every second row of a larger buffer) and repeated calls agree bit for bit
+    xs = torch.zeros((2 * T, K + 8), dtype=dtype, device=DEV)[::2, :K]
+    xs.copy_(x.to(DEV))
+    for _ in range(3):
+        assert torch.equal(sten.spmm(w, xs, reduce_dim=1), y)
+
+
+@pytest.mark.parametrize("T", [1, 16])
+def test_streamed_product_along_the_group_dim_at_full_size(T):
+    # 4096 x 11008 at 2:4:16 in the reference's default orientation against the dense form (which the
+    # sparsifier tests hold bit-exact against the oracle), in fp64 on the host
+    print(f"case gstream full size T={T}", flush=True)
+    W = seeded((4096, 11008), torch.float16, seed=5, std=0.02).to(DEV)
+    w = sten.GroupedNMTensor.from_dense(W, 2, 4, sparse_dim=0, group_size=16, group_dim=1)
+    x = seeded((T, 11008), torch.float16, seed=T)
+    y = sten.spmm(w, x.to(DEV), reduce_dim=1)
+    ref = to_np(x).astype(np.float64) @ to_np(w.to_dense()).astype(np.float64).T
+    assert rel_l2(to_np(y), ref) <= TOL[torch.float16]
 
 
 def test_reference_matmul_test_shape_in_single_precision():
