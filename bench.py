@@ -73,6 +73,7 @@ WORKLOADS = {
     "c3_4_8": ("fwd", 8192, 8192, 4096, 4, 8, 32, "configs[2]: W 8192x8192 fp16 4:8:32 x 4096 tokens, forward"),
     "c5_fwd": ("fwd", 16384, 4096, 4096, 2, 4, 16, "configs[4]: W 16384x4096 fp16 2:4:16 x 4096 tokens, forward"),
     "c5_grad_x": ("grad_x", 16384, 4096, 4096, 2, 4, 16, "configs[4]: dY 4096x16384 x W 16384x4096 fp16 2:4:16, grad_input"),
+    "c5_grad_w_dense": ("gw_dense", 16384, 4096, 4096, 2, 4, 16, "configs[4] shapes: the dense weight gradient dY^T X (default gradient format), dY 4096x16384, X 4096x4096, fp16, nmg_gemm_tn (the kernel of the masked product without its mask)"),
     "c5_step": ("step", 16384, 4096, 4096, 2, 4, 16, "configs[4]: training step of a sparse linear 4096 -> 16384, 4096 tokens: forward, grad_input, masked grad_weight in val layout"),
     "c5_train": ("train", 16384, 4096, 4096, 2, 4, 16, "configs[4] + optimizer: the training step of c5_step followed by an SGD update of the compressed weight (pattern kept) and the re-derivation of the matmul operands"),
     "c2_grad_x": ("grad_x", 4096, 4096, 2048, 2, 4, 16, "configs[1] shape: dY 2048x4096 x W 4096x4096 fp16 2:4:16, grad_input"),
@@ -286,6 +287,15 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
                 X.grad = None
                 slin(X).backward(dY)
         algo_bytes = 0
+    elif kind == "gw_dense":
+        from sten_amd.impls import _dense_product
+        del W
+        X = torch.randn(N, K).half().to(dev)
+        dY = torch.randn(N, M).half().to(dev)
+
+        def step():
+            return _dense_product("tn", dY, X)
+        algo_bytes = 0
     elif kind == "w4":
         # int4 kept values + 2-bit positions + fp16 scales + activations + output
         algo_bytes = M * K // 4 + M * K // 8 + (K // 128) * M * 2 + N * K * 2 + N * M * 2
@@ -338,7 +348,7 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
     graph = None
     per = 1                      # steps per timed iteration
     short = kind in ("decode", "decode_g", "w4") or (kind == "fwd" and N <= 1024)
-    if (short and not eager) or (graph_large and kind not in ("step", "train", "sparsify")):
+    if (short and not eager) or (graph_large and kind not in ("step", "train", "sparsify", "gw_dense")):
         per = max(GRAPH_STEPS, copies)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
@@ -405,9 +415,9 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
            "kernel_ms_mean": kern_mean, "timed_groups": len(durs), "steps_per_group": group * per,
            "launch": launch, "desc": desc, "kind": kind, "settle_steps": settle_steps,
            "shape": (M, K, N, n, m, g), "traffic_profile": PMC_SUMMARIES.get(workload)}
-    if kind in ("fwd", "grad_x", "step", "train"):
+    if kind in ("fwd", "grad_x", "step", "train", "gw_dense"):
         dense_flops = 2.0 * M * K * N * (3 if kind in ("step", "train") else 1)
-        eff_flops = dense_flops * n / m
+        eff_flops = dense_flops if kind == "gw_dense" else dense_flops * n / m
         achieved = eff_flops / (kern_ms * 1e-3) / 1e12
         peak = PEAK_FP32_TFLOPS if workload in FP32_WORKLOADS else PEAK_FP16_TFLOPS
         row.update({

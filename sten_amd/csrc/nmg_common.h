@@ -41,6 +41,10 @@ int device_order(int n, int m, const int8_t **d_order);
 int device_zero_page(const void **d_zero);
 
 
+// Y[G, S] = L[T, G]^T P[T, S] (+ bias[s]) in a 16-bit type on the matrix cores (nmg_sddmm.hip).
+int dense_tn16(const void *d_lines, int64_t ld_lines, const void *d_pos, int64_t ld_pos, int64_t T, int64_t G, int64_t S,
+               void *d_y, int64_t ldy, const void *d_bias, int dtype, void *stream);
+
 inline size_t dtype_size(int dtype)
 {
     switch (dtype) {

@@ -1023,9 +1023,11 @@ extern "C" int nmg_gemm_nn(const void *d_a, int64_t lda, const void *d_x, int64_
 extern "C" int nmg_gemm_tn(const void *d_a, int64_t lda, const void *d_x, int64_t ldx, void *d_y, int64_t ldy,
                            const void *d_bias, int64_t O, int64_t K, int64_t T, int dtype, void *stream)
 {
-    NMG_REQUIRE(dtype == NMG_F32, NMG_ERR_UNSUPPORTED, "gemm_tn takes f32");
+    NMG_REQUIRE(dtype == NMG_F32 || dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED, "gemm_tn takes f32/f16/bf16");
     NMG_REQUIRE(O >= 0 && K >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
     NMG_REQUIRE(lda >= O && ldx >= T && ldy >= O, NMG_ERR_ARG, "leading dimension smaller than row length");
+    // 16-bit: the kernel of the masked weight gradient without its mask (rows of Y = the operand X)
+    if (dtype != NMG_F32) return dense_tn16(d_x, ldx, d_a, lda, K, T, O, d_y, ldy, d_bias, dtype, stream);
     return gemm_f32_host(d_a, lda, d_x, ldx, d_y, ldy, d_bias, O, K, T, 2, stream);
 }
 

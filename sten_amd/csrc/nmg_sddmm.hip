@@ -88,7 +88,9 @@ struct SddmmParams {
     const int16_t *slot;
     const int8_t *order;
     const void *zero;  // 16 zero bytes: source of the tokens beyond T
+    const void *bias;  // dense product: bias per position, or null
     int64_t ldl, ldp, G, S, T, Gpad, nb;
+    int64_t ldv;       // dense product: elements between two lines of the result
     int n, m, g, cg;
     uint32_t inv_g;    // ceil(2^32 / g) for g > 1
     uint64_t ord4;     // m == 4: byte p = the kept positions of pattern p, 2 bits each
@@ -180,6 +182,9 @@ __device__ __forceinline__ void sd_staged_walk(const SddmmParams &P, const unsig
 // MODE 8 + n (n = 1, 2, 4): m == 8; the two lanes that hold the halves of a block exchange them
 // first (V_PERMLANE16_SWAP), then two byte permutes per output word.
 // MODE 0: any n:m, through the staged tile.
+// MODE 5: no pattern at all -- the dense product L^T P [G, S] (the weight gradient of a linear layer
+// in a dense format), staged like MODE 0 and stored as rows of `val` with a pitch of `ldv` elements
+// (+ bias per position).
 // NT = true: the operands are given with the reduction (tokens) as their fast dim, L^T [G, T] and
 // P^T [S, T] (the weight gradient of torch.mm(W, B): grad_out [R, N] and B [C, N] as they lie in
 // memory).  An operand tile of a K step is then 256 feature rows of 64 bytes; a fragment -- the
@@ -199,7 +204,8 @@ template <typename T, int MODE, bool NT = false>
 __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
 {
     using Mm = SdMma16<T>;
-    static_assert((MODE >= 0 && MODE <= 4) || MODE == 9 || MODE == 10 || MODE == 12, "the staged tile; m == 4, n == MODE; m == 8, n == MODE - 8");
+    static_assert((MODE >= 0 && MODE <= 5) || MODE == 9 || MODE == 10 || MODE == 12,
+                  "the staged tile; m == 4, n == MODE; the dense product; m == 8, n == MODE - 8");
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -225,7 +231,7 @@ __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
     // MODE 8 + n: a block of 8 positions lies in the lanes q = l/16 even (positions 0..3) and odd
     // (4..7) of one accumulator block; after the exchange in the epilogue a lane owns, per pair of
     // position blocks xp, block p0/8 + wm*16 + 4 xp + 2 (q%2) + q/2 of its line (xp even in the low half).
-    uint32_t my_slot[MODE == 0 ? 1 : (MODE <= 4 ? 32 : 16)];
+    uint32_t my_slot[(MODE == 0 || MODE == 5) ? 1 : (MODE <= 4 ? 32 : 16)];
     if constexpr (MODE >= 1 && MODE <= 4) {
         uint32_t *s_sel = (uint32_t *)(smem + 256 * SD_PITCH);
         if (tid < 16) {
@@ -511,6 +517,46 @@ __global__ __launch_bounds__(256, 1) void sddmm16_kernel(SddmmParams P)
             }
         __syncthreads();
         sd_staged_walk(P, smem, tid, l0, p0);
+    } else if constexpr (MODE == 5) {
+        // ---- dense product: stage [line][position] in the output type, then whole rows: a
+        // wavefront stores two lines per instruction, 16 bytes per lane
+        asm volatile("s_barrier" ::: "memory");   // every wavefront is done with the ring
+#pragma unroll
+        for (int y = 0; y < 8; y++)
+#pragma unroll
+            for (int x = 0; x < 8; x++) {
+                uint16_t hh[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) hh[r] = sd_bits16<T>(sd_from_acc(acc[x][y][r]));
+                uint2 pk;
+                pk.x = (uint32_t)hh[0] | ((uint32_t)hh[1] << 16);
+                pk.y = (uint32_t)hh[2] | ((uint32_t)hh[3] << 16);
+                const int line = wn * 128 + y * 16 + j16, pos = wm * 128 + x * 16 + kq * 4;
+                *(uint2 *)(smem + line * SD_PITCH + pos * 2) = pk;
+            }
+        __syncthreads();
+        const int64_t pos = p0 + (lane & 31) * 8;
+        float bv[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) bv[e] = (P.bias && pos + e < P.S) ? to_f32(((const T *)P.bias)[pos + e]) : 0.f;
+        for (int it = wave; it < 128; it += 4) {
+            const int row = 2 * it + (lane >> 5);
+            const int64_t line = l0 + row;
+            const unsigned char *src = smem + row * SD_PITCH + (lane & 31) * 16;
+            uint2 lo = *(const uint2 *)src, hi = *(const uint2 *)(src + 8);   // (rows are 8-byte aligned)
+            if (line >= P.G || pos >= P.S) continue;                          // S % 8 == 0: a piece is whole or absent
+            uint32_t w[4] = {lo.x, lo.y, hi.x, hi.y};
+            if (P.bias) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    uint16_t a = (uint16_t)w[e], b = (uint16_t)(w[e] >> 16);
+                    a = sd_bits16<T>(to_f32(__builtin_bit_cast(T, a)) + bv[2 * e]);
+                    b = sd_bits16<T>(to_f32(__builtin_bit_cast(T, b)) + bv[2 * e + 1]);
+                    w[e] = (uint32_t)a | ((uint32_t)b << 16);
+                }
+            }
+            *(u32x4 *)((uint16_t *)P.val + line * P.ldv + pos) = u32x4{w[0], w[1], w[2], w[3]};
+        }
     } else if constexpr (MODE > 8) {
         // ---- epilogue in registers, m == 8.  The lanes q even / odd round and pack their halves of
         // the blocks in the accumulator blocks 2 xp and 2 xp + 1 and exchange them
@@ -776,6 +822,57 @@ static int sddmm_impl(bool nt, const void *d_lines, int64_t ld_lines, const void
     NMG_HIP_TRY(hipGetLastError());
     return NMG_OK;
 }
+
+namespace nmg {
+// Dense product on the same kernel: Y[G, S] = L[T, G]^T P[T, S] (+ bias[s]) in a 16-bit type, fp32
+// accumulation, rounded once.  Both operands token-major with extents and pitches that are
+// multiples of 8 and 16-byte aligned bases (NMG_ERR_UNSUPPORTED otherwise).
+int dense_tn16(const void *d_lines, int64_t ld_lines, const void *d_pos, int64_t ld_pos, int64_t T, int64_t G, int64_t S,
+               void *d_y, int64_t ldy, const void *d_bias, int dtype, void *stream)
+{
+    NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED, "the 16-bit product takes f16/bf16");
+    if (G == 0 || S == 0) return NMG_OK;
+    NMG_REQUIRE(T > 0, NMG_ERR_UNSUPPORTED, "no tokens: clear the result instead");
+    NMG_REQUIRE(G % 8 == 0 && S % 8 == 0 && ld_lines % 8 == 0 && ld_pos % 8 == 0 && ldy % 8 == 0 &&
+                    ((uintptr_t)d_lines % 16) == 0 && ((uintptr_t)d_pos % 16) == 0 && ((uintptr_t)d_y % 16) == 0,
+                NMG_ERR_UNSUPPORTED, "needs extents and leading dimensions that are multiples of 8 and 16-byte aligned operands");
+    NMG_REQUIRE(ld_lines < ((int64_t)1 << 25) && ld_pos < ((int64_t)1 << 25), NMG_ERR_UNSUPPORTED, "leading dimension too large");
+    NMG_REQUIRE(d_lines && d_pos && d_y, NMG_ERR_ARG, "null device pointer");
+    SddmmParams P{};
+    if (int rc = device_zero_page(&P.zero)) return rc;
+    P.lop = d_lines;
+    P.pop = d_pos;
+    P.val = d_y;
+    P.bias = d_bias;
+    P.ldl = ld_lines;
+    P.ldp = ld_pos;
+    P.ldv = ldy;
+    P.G = G;
+    P.S = S;
+    P.T = T;
+    P.nb = S;
+    P.Gpad = G;
+    P.n = P.m = P.g = 1;
+    P.cg = 1;
+    P.KP = (int)((T + SD_KS - 1) / SD_KS);
+    P.tiles_p = (int)((S + 255) / 256);
+    P.tiles_l = (int)((G + 255) / 256);
+    NMG_REQUIRE((int64_t)P.tiles_p * P.tiles_l <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "product too large for one launch");
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid((unsigned)(P.tiles_p * P.tiles_l));
+    if (dtype == NMG_F16) {
+        auto k = sddmm16_kernel<__half, 5>;
+        NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, SD_LDS));
+        hipLaunchKernelGGL(k, grid, dim3(256), SD_LDS, s, P);
+    } else {
+        auto k = sddmm16_kernel<__hip_bfloat16, 5>;
+        NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, SD_LDS));
+        hipLaunchKernelGGL(k, grid, dim3(256), SD_LDS, s, P);
+    }
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+}  // namespace nmg
 
 extern "C" int nmg_sddmm(const void *d_lines, int64_t ld_lines, const void *d_pos, int64_t ld_pos, int64_t T,
                          const int16_t *d_slot, int64_t G, int64_t S, void *d_val, int n, int m, int g,

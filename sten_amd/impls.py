@@ -42,24 +42,44 @@ def _masked_weight_grad(weight, lhs_t, rhs):
         # single precision: the dense product on the fp32 matrix cores, operands as they lie
         # (both reduction-major), then the gather
         return weight.clone_layout(_f32_product("tn", lhs_t, rhs))
-    return weight.clone_layout(torch.mm(lhs_t.t(), rhs))
+    return weight.clone_layout(_dense_product("tn", lhs_t, rhs))
 
 
 def _f32_product(form, x, a):
     """Dense fp32 product on this library's matrix-core GEMM, operands as they lie in memory:
     ``"tn"``: x [K, T], a [K, O] -> x^T @ a;  ``"nt"``: x [T, K], a [O, K] -> x @ a^T."""
-    x = x if x.stride(1) == 1 else x.contiguous()
-    a = a if a.stride(1) == 1 else a.contiguous()
+    return _dense_product(form, x, a)
+
+
+def _dense_product(form, x, a):
+    """Dense product on this library's matrix-core kernels, operands as they lie in memory:
+    ``"tn"``: x [K, T], a [K, O] -> x^T @ a (``nmg_gemm_tn``);  ``"nt"``: x [T, K], a [O, K] -> x @ a^T
+    (``nmg_gemm_nt``).  fp32 always; 16-bit types where the kernels take the shape (extents and
+    pitches that are multiples of 8, 16-byte aligned bases; ``"nt"``: K a multiple of 64) -- what
+    they do not take goes to ``torch.mm``."""
+    dt = x.dtype
     if form == "tn":
         (K, T), O = x.shape, a.shape[1]
-        entry = native.load().nmg_gemm_tn
     else:
         (T, K), O = x.shape, a.shape[0]
-        entry = native.load().nmg_gemm_nt
-    y = torch.empty((T, O), dtype=torch.float32, device=x.device)
+    ok = x.is_cuda and a.dtype == dt and dt in native.DTYPE_CODE and dt != torch.float64 and T > 0 and O > 0 and K > 0
+    if ok:
+        x = x if x.stride(1) == 1 else x.contiguous()
+        a = a if a.stride(1) == 1 else a.contiguous()
+    if ok and dt != torch.float32:
+        ok = (x.stride(0) % 8 == 0 and a.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and a.data_ptr() % 16 == 0
+              and O % 8 == 0 and max(x.stride(0), a.stride(0)) < 2 ** 24)
+        if form == "tn":
+            ok = ok and T % 8 == 0
+        else:
+            ok = ok and K % 64 == 0 and O * a.stride(0) * 2 < 2 ** 31 and T * x.stride(0) * 2 < 2 ** 31
+    if not ok:
+        return torch.mm(x.t(), a) if form == "tn" else torch.mm(x, a.t())
+    entry = native.load().nmg_gemm_tn if form == "tn" else native.load().nmg_gemm_nt
+    y = torch.empty((T, O), dtype=dt, device=x.device)
     with torch.cuda.device(x.device):
         native.check(entry(native.ptr(a), a.stride(0), native.ptr(x), x.stride(0), native.ptr(y), O,
-                           None, O, K, T, native.dtype_code(torch.float32), native.stream_ptr(x.device)))
+                           None, O, K, T, native.dtype_code(dt), native.stream_ptr(x.device)))
     return y
 
 
@@ -117,7 +137,8 @@ def install(api):
         if compressed:
             gw = wrap(_masked_weight_grad(w, gy2, x2), x2)
         else:
-            gw = torch.mm(gy2.t(), x2)
+            # the dense weight gradient dY^T X from the operands as they lie (both token-major)
+            gw = _dense_product("tn", gy2, x2 if x2.dtype == gy2.dtype else x2.to(gy2.dtype))
         grads = [gx, gw]
         if len(saved) > 2:
             grads.append(gy2.sum(dim=0))
@@ -157,7 +178,7 @@ def install(api):
             else:
                 gw = wrap(_masked_weight_grad(w, gc.t(), b.t()), gc)
         else:
-            gw = torch.mm(gc, b.t())
+            gw = _dense_product("nt", gc, b if b.dtype == gc.dtype else b.to(gc.dtype))     # grad_out @ B^T
         return gw, gb
 
     api.register_bwd_op_impl(

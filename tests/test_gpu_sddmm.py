@@ -227,3 +227,56 @@ def test_weight_gradient_of_torch_mm_from_its_operands_as_they_lie():
     got = w.masked_product(gc, B, reduction_last=True)
     ref = w.clone_layout((gc.double() @ B.double().t()).half())
     assert float((got.val.float() - ref.val.float()).norm() / ref.val.float().norm()) <= 1e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("R,C,T,bias", [
+    (256, 256, 64, False),       # one tile, whole K steps
+    (200, 136, 37, True),        # ragged lines, positions and tokens
+    (520, 776, 100, False),      # several tiles both ways
+    (8, 8, 1, True),             # smallest extents the kernel takes
+    (1024, 512, 4096, False),    # 128 K steps
+])
+def test_dense_weight_gradient_in_16_bit(dtype, R, C, T, bias):
+    # the dense weight gradient dY^T X of a linear layer (default gradient format) on the kernel of
+    # the masked product without its mask: nmg_gemm_tn in f16 / bf16 against the fp64 product
+    print(f"case gemm_tn16 {dtype} R={R} C={C} T={T} bias={bias}", flush=True)
+    gy = seeded((T, R), dtype, seed=R + T).to(DEV)
+    x = seeded((T, C), dtype, seed=C + T + 1).to(DEV)
+    b = seeded((C,), dtype, seed=3).to(DEV) if bias else None
+    # a result with a row pitch: every second row of a larger buffer stays untouched
+    buf = torch.full((R, 2 * C), 7.0, dtype=dtype, device=DEV)
+    out = buf[:, :C]
+    native.check(native.load().nmg_gemm_tn(
+        native.ptr(x), x.stride(0), native.ptr(gy), gy.stride(0), native.ptr(out), out.stride(0),
+        native.ptr(b), C, T, R, native.dtype_code(dtype), None))
+    torch.cuda.synchronize()
+    ref = to_np(gy).astype(np.float64).T @ to_np(x).astype(np.float64)
+    if bias:
+        ref = ref + to_np(b).astype(np.float64)
+    assert rel_l2(to_np(out), ref) <= TOL[dtype]
+    assert bool((buf[:, C:] == 7.0).all()), "wrote beyond the rows of the result"
+
+
+def test_default_gradient_format_takes_no_library_gemm(monkeypatch):
+    # F.linear backward with the default (dense) weight-gradient format in fp16: forward, grad_input and
+    # the dense dY^T X all run on this library's kernels -- torch.mm must not be called
+    torch.manual_seed(0)
+    lin = torch.nn.Linear(256, 384, bias=True).half().to(DEV)
+    sb = sten.SparsityBuilder()
+    sb.set_weight("weight", initial_sparsifier=sten.GroupedNMSparsifier(2, 4, 16, sparse_dim=1, group_dim=0),
+                  out_format=sten.GroupedNMTensor)
+    sp = sb.get_sparse_model(lin)
+    Wd = sp.weight.wrapped_tensor.to_dense().detach().float()
+    x = torch.randn(72, 256, device=DEV).half().requires_grad_(True)
+    gy = torch.randn(72, 384, device=DEV).half()
+
+    def no_mm(*a, **k):
+        raise AssertionError("torch.mm was called in the backward of the sparse linear")
+    monkeypatch.setattr(torch, "mm", no_mm)
+    y = sp(x)
+    y.backward(gy)
+    monkeypatch.undo()
+    gw = sp.weight.grad.wrapped_tensor.to_dense().float()
+    assert rel_l2(to_np(gw), to_np(gy.float().t() @ x.detach().float())) <= 1e-3
+    assert rel_l2(to_np(x.grad.float()), to_np(gy.float() @ Wd)) <= 1e-3
