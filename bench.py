@@ -85,6 +85,8 @@ WORKLOADS = {
     "decode_gdim_4": ("decode_g", 4096, 11008, 4, 2, 4, 16, "the same x 4 tokens"),
     "decode_gdim_8": ("decode_g", 4096, 11008, 8, 2, 4, 16, "the same x 8 tokens"),
     "decode_gdim_16": ("decode_g", 4096, 11008, 16, 2, 4, 16, "the same x 16 tokens"),
+    "decode_2_8_1": ("decode", 8192, 8192, 1, 2, 8, 32, "north_star: W 8192x8192 fp16 2:8:32 x 1 token"),
+    "decode_2_8_16": ("decode", 8192, 8192, 16, 2, 8, 32, "north_star: W 8192x8192 fp16 2:8:32 x 16 tokens"),
     "decode_up_1": ("decode", 11008, 4096, 1, 2, 4, 16, "W 11008x4096 fp16 2:4:16 x 1 token (the up-projection beside the north_star shape)"),
     "decode_up_16": ("decode", 11008, 4096, 16, 2, 4, 16, "W 11008x4096 fp16 2:4:16 x 16 tokens"),
     "c4_b1": ("w4", 11008, 4096, 1, 2, 4, 1, "configs[3]: W 11008x4096 2:4 + int4 (scale per 128) x 1 token"),

@@ -155,36 +155,42 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
     static_assert((NS - 1) * OPS < 64, "vmcnt is a 6-bit counter");
     static_assert(TB == 1, "the wait lists one activation fragment");
 
+    // (`s_nop 4` in front of every load: the bases are scalar registers, and where the compiler
+    // parks one in a lane of a vector register it reads it back with a vector instruction right
+    // before the use -- a scalar register written by the vector unit needs five wait states before
+    // a memory instruction may read it, and the compiler does not look into instruction statements)
     auto issue_tile = [&](Regs &R, uint32_t rel) __attribute__((always_inline)) {
         // ranges are multiples of 8 lines: a group of 8 is whole or absent
         const bool in_range = rel < nlines && rel + 8 * kq < nlines;
         const uint32_t lrel = in_range ? rel + 8 * kq : 0u;      // lines from the range's first
         // (24-bit factors, checked by the host: one multiply-add each)
-        const uint32_t v_off = __umul24(lrel, (uint32_t)val_pitch) + bl_lane * (N * 2);
-        const uint32_t p_off = __umul24(lrel, (uint32_t)pat_pitch) + bl_lane;
+        // (beyond the whole range every lane reads the first bytes of the base: one cache line)
+        const bool none = rel >= nlines;
+        const uint32_t v_off = none ? 0u : __umul24(lrel, (uint32_t)val_pitch) + bl_lane * (N * 2);
+        const uint32_t p_off = none ? 0u : __umul24(lrel, (uint32_t)pat_pitch) + bl_lane;
 #pragma unroll
         for (int u = 0; u < 8; u++) {
             const unsigned char *vp = vwave + u * val_pitch;
             const unsigned char *pp = pwave + u * pat_pitch;
             if constexpr (VB == 16)
-                asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(R.vals[u]) : "v"(v_off), "s"(vp) : "memory");
+                asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2" : "=v"(R.vals[u]) : "v"(v_off), "s"(vp) : "memory");
             else if constexpr (VB == 8)
-                asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(R.vals[u]) : "v"(v_off), "s"(vp) : "memory");
+                asm volatile("s_nop 4\n\tglobal_load_dwordx2 %0, %1, %2" : "=v"(R.vals[u]) : "v"(v_off), "s"(vp) : "memory");
             else if constexpr (VB == 4)
-                asm volatile("global_load_dword %0, %1, %2" : "=v"(R.vals[u]) : "v"(v_off), "s"(vp) : "memory");
+                asm volatile("s_nop 4\n\tglobal_load_dword %0, %1, %2" : "=v"(R.vals[u]) : "v"(v_off), "s"(vp) : "memory");
             else
-                asm volatile("global_load_ushort %0, %1, %2" : "=v"(R.vals[u]) : "v"(v_off), "s"(vp) : "memory");
+                asm volatile("s_nop 4\n\tglobal_load_ushort %0, %1, %2" : "=v"(R.vals[u]) : "v"(v_off), "s"(vp) : "memory");
             if constexpr (BL == 4)
-                asm volatile("global_load_dword %0, %1, %2" : "=v"(R.pats[u]) : "v"(p_off), "s"(pp) : "memory");
+                asm volatile("s_nop 4\n\tglobal_load_dword %0, %1, %2" : "=v"(R.pats[u]) : "v"(p_off), "s"(pp) : "memory");
             else if constexpr (BL == 2)
-                asm volatile("global_load_ushort %0, %1, %2" : "=v"(R.pats[u]) : "v"(p_off), "s"(pp) : "memory");
+                asm volatile("s_nop 4\n\tglobal_load_ushort %0, %1, %2" : "=v"(R.pats[u]) : "v"(p_off), "s"(pp) : "memory");
             else
-                asm volatile("global_load_ubyte %0, %1, %2" : "=v"(R.pats[u]) : "v"(p_off), "s"(pp) : "memory");
+                asm volatile("s_nop 4\n\tglobal_load_ubyte %0, %1, %2" : "=v"(R.pats[u]) : "v"(p_off), "s"(pp) : "memory");
         }
 #pragma unroll
         for (int tb = 0; tb < TB; tb++) {
-            const uint32_t xo = x_tok[tb] + lrel * 2;
-            asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(R.xf[tb]) : "v"(xo), "s"(xwave) : "memory");
+            const uint32_t xo = none ? 0u : x_tok[tb] + lrel * 2;
+            asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2" : "=v"(R.xf[tb]) : "v"(xo), "s"(xwave) : "memory");
             R.xmask[tb] = in_range ? x_live[tb] : 0u;
         }
     };

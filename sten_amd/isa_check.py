@@ -8,11 +8,13 @@ error.  This tool re-reads the device assembly the compiler produced and proves,
 
   * no instruction touches a register that a still-outstanding load will write (a spill of such a
     register is an instruction that reads it), and
+  * no hand-issued load reads a scalar register less than five wait states after a vector
+    instruction wrote it (the compiler keeps that distance for its own instructions only), and
   * no loop that streams operands holds scratch traffic, which would break the per-step count
     of operations the waits rely on (spills outside those loops are reported, not refused),
 
-by simulating the in-order vector-memory counter along every kernel (loop bodies are walked twice,
-so the state a loop carries into its next iteration is checked too).
+by simulating the in-order vector-memory counter along every kernel (loop bodies are walked again
+with the state their back edge carries, so what a loop hands to its next iteration is checked too).
 
     python -m sten_amd.isa_check                  # all sources that contain hand-issued loads
     python -m sten_amd.isa_check file.s --kernels dense_direct   # an assembly file made elsewhere
@@ -36,9 +38,11 @@ CHECKED = {
     "nmg_w4.hip": ["w4_linear_staged_kernel"],
     "nmg_sddmm.hip": ["sddmm16_kernel"],
     "nmg_gstream.hip": ["gstream_kernel"],
+    "nmg_sstream.hip": ["sstream_kernel"],
 }
 
 REG = re.compile(r"\b([va])(\d+)\b|\b([va])\[(\d+):(\d+)\]")
+SREG = re.compile(r"\bs(\d+)\b|\bs\[(\d+):(\d+)\]")
 VMEM = re.compile(r"^(global|buffer|scratch|flat)_(load|store|atomic)")
 LABEL = re.compile(r"^(\.?[A-Za-z_][\w.$]*):")
 
@@ -52,6 +56,44 @@ def regs_of(text):
             for r in range(int(m.group(4)), int(m.group(5)) + 1):
                 out.add((m.group(3), r))
     return out
+
+
+def sregs_of(text):
+    out = set()
+    for m in SREG.finditer(text):
+        if m.group(1):
+            out.add(int(m.group(1)))
+        else:
+            out.update(range(int(m.group(2)), int(m.group(3)) + 1))
+    return out
+
+
+def scalar_hazards(name, prog):
+    """A scalar register written by a vector instruction (a lane read that brings back a parked
+    base, a compare) must rest five wait states before a vector-memory instruction reads it.  The
+    compiler inserts them for its own instructions; it does not look into instruction statements,
+    so the hand-issued loads are checked here, in layout order."""
+    problems = []
+    age = {}      # scalar register -> wait states since a vector instruction wrote it
+    for i, (kind, inst, by_hand) in enumerate(prog):
+        if kind != "inst":
+            continue
+        op = inst.split()[0]
+        if by_hand and VMEM.match(op):
+            young = sorted(r for r in sregs_of(inst) if age.get(r, 99) < 5)
+            if young:
+                problems.append(f"{name[:60]} @{i}: `{inst}` reads s{young[:4]} less than five wait states after a "
+                                "vector instruction wrote them")
+        states = 1
+        if op == "s_nop":
+            states = int(inst.split()[1], 0) + 1
+        for r in list(age):
+            age[r] += states
+        if op.startswith("v_") and len(inst.split(None, 1)) > 1:
+            first = inst.split(None, 1)[1].split(",")[0]
+            for r in sregs_of(first):
+                age[r] = 0
+    return problems
 
 
 def kernels_of(asm_text):
@@ -75,20 +117,27 @@ def kernels_of(asm_text):
 
 
 def parse(body):
-    """[(kind, payload)] with kind in label / inst."""
+    """[(kind, payload, by_hand)] with kind in label / inst; by_hand: the instruction stands inside
+    an instruction statement of the source (between the compiler's ASMSTART / ASMEND marks)."""
     prog = []
+    by_hand = False
     for raw in body:
-        line = raw.split(";")[0].rstrip() if not raw.strip().startswith(";;#") else ""
+        mark = raw.strip()
+        if mark.startswith(";;#ASMSTART"):
+            by_hand = True
+        elif mark.startswith(";;#ASMEND"):
+            by_hand = False
+        line = raw.split(";")[0].rstrip() if not mark.startswith(";;#") else ""
         if not line.strip():
             continue
         m = LABEL.match(line.strip())
         if m and not line.startswith("\t"):
-            prog.append(("label", m.group(1)))
+            prog.append(("label", m.group(1), False))
             continue
         t = line.strip()
         if t.startswith("."):
             continue
-        prog.append(("inst", t))
+        prog.append(("inst", t, by_hand))
     return prog
 
 
@@ -99,10 +148,14 @@ def check_kernel(name, body):
     """List of problems of one kernel (empty = clean); remarks that are no problems go to `notes`."""
     prog = parse(body)
     labels = {p[1]: i for i, p in enumerate(prog) if p[0] == "label"}
-    problems = []
+    problems = scalar_hazards(name, prog)
     seen = set()
+    # Only the loads of instruction statements are tracked by register: the compiler waits for its
+    # own loads itself, they only take their place in the queue.  (An assembly text without the
+    # compiler's marks -- a test, a hand-written file -- has every load tracked.)
+    marked = any(p[2] for p in prog)
 
-    def step(inst, queue, where):
+    def step(inst, queue, where, by_hand=True):
         op = inst.split()[0]
         if op == "s_waitcnt":
             m = re.search(r"vmcnt\((\d+)\)", inst)
@@ -116,7 +169,7 @@ def check_kernel(name, body):
             is_load = "_load" in op or "atomic" in op
             to_lds = "_lds_" in op or op.endswith("_lds")
             dest = set()
-            if is_load and not to_lds:
+            if is_load and not to_lds and (by_hand or not marked):
                 first = inst.split(None, 1)[1].split(",")[0]
                 dest = regs_of(first)
             # the address / data registers it reads must not be in flight either
@@ -127,6 +180,8 @@ def check_kernel(name, body):
             # a load into registers that an older outstanding load also writes would be ordered by the
             # hardware (in-order return), not a hazard
             queue.append(dest)
+            if len(queue) > 63:          # the counter holds 63: older operations have completed
+                del queue[:len(queue) - 63]
             return
         for entry in queue:
             hit = entry & touched
@@ -134,30 +189,57 @@ def check_kernel(name, body):
                 seen.add((where, inst))
                 problems.append(f"{where}: `{inst}` touches {sorted(hit)[:4]} while a load into them is outstanding")
 
-    # linear walk; at a backward branch, walk the loop body once more with the state at the branch
-    queue = []
-    i = 0
-    revisited = set()
-    while i < len(prog):
-        kind, payload = prog[i]
-        if kind == "inst":
-            step(payload, queue, f"{name[:60]} @{i}")
-            m = re.match(r"s_cbranch_\w+\s+(\S+)|s_branch\s+(\S+)", payload)
-            if m:
-                target = m.group(1) or m.group(2)
-                if target in labels and labels[target] < i and (target, i) not in revisited:
-                    revisited.add((target, i))
-                    q2 = list(queue)
-                    for j in range(labels[target], i):
-                        if prog[j][0] == "inst":
-                            step(prog[j][1], q2, f"{name[:60]} @{j} (second iteration)")
-        i += 1
+    # Walk in layout order, which for these kernels is execution order, with two corrections.  An
+    # unconditional forward branch is followed (what lies behind it is never fallen into: a rotated
+    # loop has its body there, entered from its header further down).  At a backward branch the
+    # stretch from its target to the branch is walked twice more, each time with the state the
+    # previous walk ended in: what a loop hands to its next iteration is checked too.  Conditional
+    # forward branches (loop exits, guards) are not followed: their conditions are correlated in
+    # ways a path search cannot see, and it would report paths that never run.
+    flagged = set()
+
+    def step_once(pc, inst, queue, looped):
+        before = len(problems)
+        step(inst, queue, f"{name[:60]} @{pc}" + (" (second iteration)" if looped else ""), prog[pc][2])
+        if len(problems) > before:
+            if pc in flagged:
+                del problems[before:]
+            else:
+                flagged.add(pc)
+                del problems[before + 1:]
+
+    BR = re.compile(r"s_cbranch_\w+\s+(\S+)|s_branch\s+(\S+)")
+
+    def walk(pc, stop, queue, looped, rewalks):
+        """Walk from pc until `stop` (exclusive) is reached or passed; returns the queue at the end."""
+        while pc < stop:
+            kind, payload = prog[pc][0], prog[pc][1]
+            if kind == "inst":
+                step_once(pc, payload, queue, looped)
+                m = BR.match(payload)
+                if m:
+                    target = m.group(1) or m.group(2)
+                    if target in labels:
+                        t = labels[target]
+                        if t < pc and rewalks > 0 and (t, pc) not in done_loops:
+                            done_loops.add((t, pc))
+                            q2 = list(queue)
+                            for _ in range(rewalks):
+                                q2 = walk(t, pc + 1, q2, True, 0)
+                        elif t > pc and m.group(2):
+                            pc = t
+                            continue
+            pc += 1
+        return queue
+
+    done_loops = set()
+    walk(0, len(prog), [], False, 2)
     # Spills: a spilled register with a load in flight is caught above (the scratch operation reads
     # it).  Scratch traffic inside a loop that streams operands would also disturb the counted
     # waits' budget of operations per step, so there it is an error; before and after the loops
     # (a value parked across the product) it is only reported.
     loops = []
-    for i, (kind, payload) in enumerate(prog):
+    for i, (kind, payload, _) in enumerate(prog):
         if kind != "inst":
             continue
         m = re.match(r"s_cbranch_\w+\s+(\S+)|s_branch\s+(\S+)", payload)
@@ -165,7 +247,7 @@ def check_kernel(name, body):
             target = m.group(1) or m.group(2)
             if target in labels and labels[target] < i:
                 loops.append((labels[target], i))
-    for i, (kind, payload) in enumerate(prog):
+    for i, (kind, payload, _) in enumerate(prog):
         if kind == "inst" and payload.startswith("scratch_"):
             inside = [lp for lp in loops if lp[0] <= i <= lp[1]
                       and any(prog[j][0] == "inst" and prog[j][1].startswith("global_load") for j in range(lp[0], lp[1]))]

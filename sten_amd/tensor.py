@@ -42,6 +42,7 @@ class GroupedNMTensor:
         self._fragpack = None
         self._densefrag = None
         self._dense_operand = None
+        self._lanepack8 = None
 
     # ---- construction ----------------------------------------------------------------------
     @staticmethod
@@ -309,6 +310,29 @@ class GroupedNMTensor:
             cache[slot] = out       # only an operand that was written is kept
         return out
 
+    def lanepack8(self):
+        """Operand of the streaming product on blocks of 8 along the reduction (1:8, 2:8, 4:8 with at
+        most 16 tokens): the rowpack values and pattern bytes in the order in which the lanes of
+        ``nmg_spmm_sstream`` take them; as large as the rowpack operand (0.625 bytes per dense weight
+        at 2:8), kept until ``val`` changes."""
+        lay = self.layout
+        cached = getattr(self, "_lanepack8", None)
+        if cached is not None and self._key_current(cached[0]):
+            return cached[1], cached[2]
+        pk_val, pk_pat = self.rowpack()
+        lib = native.load()
+        G, S = lay.G, lay.S
+        ve, pb = ctypes.c_int64(), ctypes.c_int64()
+        native.check(lib.nmg_lanepack8_sizes(G, S, lay.n, ctypes.byref(ve), ctypes.byref(pb)))
+        lp_val = torch.empty(ve.value, dtype=self.val.dtype, device=self.val.device)
+        lp_pat = torch.empty(pb.value, dtype=torch.uint8, device=self.val.device)
+        with torch.cuda.device(lp_val.device):
+            native.check(lib.nmg_lanepack8(native.ptr(pk_val), native.ptr(pk_pat), G, S, lay.n, native.ptr(lp_val),
+                                           native.ptr(lp_pat), native.dtype_code(lp_val.dtype),
+                                           native.stream_ptr(lp_val.device)))
+        self._lanepack8 = (self._version_key(), lp_val, lp_pat)
+        return lp_val, lp_pat
+
     def slotmap(self):
         """int16 [num_blocks, Gpad]: for every line of the (padded) group dim and block of the
         sparse dim, the slot that holds it -- the inverse of ``idx``.  Operand of the masked
@@ -521,6 +545,25 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
               and x.dtype in (torch.float16, torch.bfloat16))
     if kname == "skinny" and T > 16:
         raise native.NmgError("the skinny kernel serves at most 16 tokens")
+    # Few tokens on blocks of 8 along the reduction (1:8, 2:8, 4:8): the rowpack operand holds 0.375 /
+    # 0.625 / 1.125 bytes per dense weight where the operand of the sparse matrix cores holds 1.125
+    # (and 4:8 has none): streamed once, expanded in registers, one kernel.
+    if (kname in ("auto", "sstream") and reduce_sparse == 1 and T <= 16 and len(lay.dense_shape) == 2
+            and x.dtype in (torch.float16, torch.bfloat16)
+            and native.load().nmg_spmm_sstream_supported(lay.n, lay.m)
+            and K % 256 == 0 and K <= (6144 if lay.n == 4 else 8192)
+            and (T == 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0
+            and T * max(x.stride(0), K) * 2 < 2 ** 31 and 32 * (K // 8) * lay.n * 2 < 2 ** 31):
+        lp_val, lp_pat = weight.lanepack8()
+        with torch.cuda.device(x.device):
+            native.check(native.load().nmg_spmm_sstream(
+                native.ptr(lp_val), native.ptr(lp_pat), O, K, native.ptr(x), x.stride(0) if T > 1 else K,
+                native.ptr(y), O, native.ptr(bias), T, lay.n, lay.m, native.dtype_code(x.dtype),
+                native.stream_ptr(x.device)))
+        return y
+    if kname == "sstream":
+        raise native.NmgError("the streaming product along the sparse dim needs 16-bit data, at most 16 tokens, "
+                              "1:8, 2:8 or 4:8 and a reduction extent that is a multiple of 256, at most 8192 (4:8: 6144)")
     packed = None
     if smf_ok and kname in ("auto", "skinny", "smfmac"):
         packed = weight.fragpack()

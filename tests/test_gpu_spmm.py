@@ -503,7 +503,7 @@ def test_odd_16_bit_shapes_take_the_padded_dense_route(dtype, M, K, T, n, m, g, 
 
 @pytest.mark.parametrize("T", [1, 3, 16])
 @pytest.mark.parametrize("dtype,M,K,n,m,g,sd", [
-    (torch.float16, 512, 1024, 4, 8, 4, 1),       # no sparse-core operand for 4:8
+    (torch.float16, 512, 1088, 4, 8, 4, 1),       # no sparse-core operand for 4:8 (and no whole sets of 32 blocks for the streaming kernel)
     (torch.bfloat16, 760, 640, 2, 4, 16, 0),      # the reference's default orientation (reduction along the group dim) with 190 blocks: not whole groups of 4
     (torch.float16, 320, 1152, 3, 6, 12, 1),
     (torch.float32, 512, 1024, 2, 4, 16, 1),      # fp32: dense copy + fp32 GEMM
@@ -556,6 +556,49 @@ def test_few_tokens_along_the_group_dim_stream_the_compressed_lines(dtype, M, K,
     xs.copy_(x.to(DEV))
     for _ in range(3):
         assert torch.equal(sten.spmm(w, xs, reduce_dim=1), y)
+
+
+@pytest.mark.parametrize("T", [1, 5, 16])
+@pytest.mark.parametrize("dtype,M,K,n,m,g", [
+    (torch.float16, 512, 1024, 2, 8, 32),      # sixteen workgroups, four sets: some wavefronts have none
+    (torch.bfloat16, 512, 1024, 2, 8, 32),
+    (torch.float16, 200, 2560, 1, 8, 4),       # lines that are not a multiple of 32, ten sets over eight wavefronts
+    (torch.float16, 264, 768, 4, 8, 2),        # 4:8: no operand of the sparse matrix cores exists
+    (torch.bfloat16, 96, 6144, 4, 8, 1),       # 24 sets: three per wavefront, the most 4:8 takes
+    (torch.float16, 1056, 8192, 2, 8, 8),      # 32 sets: four per wavefront
+])
+def test_few_tokens_on_blocks_of_eight_stream_the_compressed_lines(dtype, M, K, n, m, g, T):
+    # 1:8, 2:8, 4:8 with the blocks along the reduction and <= 16 tokens: the rowpack operand, streamed
+    print(f"case sstream {dtype} M={M} K={K} {n}:{m}:{g} T={T}", flush=True)
+    W = seeded((M, K), dtype, seed=M + K, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, 1)
+    w = make(W, n, m, g, 1)
+    x = seeded((T, K), dtype, seed=T)
+    b = seeded((M,), dtype, seed=2)
+    ref = to_np(x).astype(np.float64) @ Wd.T
+    y = sten.spmm(w, x.to(DEV), reduce_dim=1, kernel="sstream")
+    assert rel_l2(to_np(y), ref) <= TOL[dtype]
+    yb = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)      # the automatic choice takes the same route
+    assert rel_l2(to_np(yb), ref + to_np(b).astype(np.float64)) <= TOL[dtype]
+    xs = torch.zeros((2 * T, K + 8), dtype=dtype, device=DEV)[::2, :K]
+    xs.copy_(x.to(DEV))
+    for _ in range(3):
+        assert torch.equal(sten.spmm(w, xs, reduce_dim=1), y)
+    if n < 4:
+        y2 = sten.spmm(w, x.to(DEV), reduce_dim=1, kernel="skinny")      # the operand of the sparse matrix cores
+        assert rel_l2(to_np(y2), to_np(y).astype(np.float64)) <= 2 * TOL[dtype]
+
+
+@pytest.mark.parametrize("T", [1, 16])
+def test_streamed_product_on_blocks_of_eight_at_full_size(T):
+    # 8192 x 8192 at 2:8:32 against the dense form, in fp64 on the host
+    print(f"case sstream full size T={T}", flush=True)
+    W = seeded((8192, 8192), torch.float16, seed=6, std=0.02).to(DEV)
+    w = sten.GroupedNMTensor.from_dense(W, 2, 8, sparse_dim=1, group_size=32, group_dim=0)
+    x = seeded((T, 8192), torch.float16, seed=T)
+    y = sten.spmm(w, x.to(DEV), reduce_dim=1)
+    ref = to_np(x).astype(np.float64) @ to_np(w.to_dense()).astype(np.float64).T
+    assert rel_l2(to_np(y), ref) <= TOL[torch.float16]
 
 
 @pytest.mark.parametrize("T", [1, 16])

@@ -115,3 +115,69 @@ def test_register_of_an_unused_load_reused_before_the_wait():
 \tv_accvgpr_read_b32 v5, a32
 """)
     assert ok == []
+
+
+def test_unconditional_forward_branch_is_followed():
+    # a rotated loop: its body lies behind an unconditional branch to the header and is entered only
+    # from there; falling into it after the prologue would report the refill of a set that is in
+    # flight, which never runs in that order
+    p = run("""
+\tglobal_load_dword v4, v1, s[2:3]
+\ts_branch .LBB0_2
+.LBB0_1:
+\tv_mov_b32_e32 v9, v4
+\tglobal_load_dword v4, v1, s[2:3]
+.LBB0_2:
+\ts_waitcnt vmcnt(0)
+\ts_cbranch_scc1 .LBB0_1
+""")
+    assert p == []
+    # the same body without the wait in the header is a hazard on the way round
+    p = run("""
+\tglobal_load_dword v4, v1, s[2:3]
+\ts_branch .LBB0_2
+.LBB0_1:
+\tv_mov_b32_e32 v9, v4
+\tglobal_load_dword v4, v1, s[2:3]
+.LBB0_2:
+\ts_cbranch_scc1 .LBB0_1
+\ts_waitcnt vmcnt(0)
+""")
+    assert len(p) == 1 and "v_mov_b32_e32 v9, v4" in p[0]
+
+
+def test_only_loads_of_instruction_statements_are_tracked_by_register():
+    # with the compiler's marks in the text, its own loads take their place in the queue but their
+    # registers are its own business
+    p = run("""
+\tglobal_load_dword v7, v1, s[2:3]
+\tv_mov_b32_e32 v8, v7
+\t;;#ASMSTART
+\tglobal_load_dword v4, v1, s[2:3]
+\t;;#ASMEND
+\tv_mov_b32_e32 v9, v4
+\ts_waitcnt vmcnt(0)
+""")
+    assert len(p) == 1 and "v_mov_b32_e32 v9, v4" in p[0]
+
+
+def test_scalar_register_written_by_the_vector_unit_needs_wait_states_before_a_hand_issued_load():
+    p = run("""
+\tv_readlane_b32 s2, v201, 27
+\tv_readlane_b32 s3, v201, 28
+\t;;#ASMSTART
+\tglobal_load_dwordx2 v[4:5], v1, s[2:3]
+\t;;#ASMEND
+\ts_waitcnt vmcnt(0)
+""")
+    assert len(p) == 1 and "five wait states" in p[0]
+    p = run("""
+\tv_readlane_b32 s2, v201, 27
+\tv_readlane_b32 s3, v201, 28
+\t;;#ASMSTART
+\ts_nop 4
+\tglobal_load_dwordx2 v[4:5], v1, s[2:3]
+\t;;#ASMEND
+\ts_waitcnt vmcnt(0)
+""")
+    assert p == []
