@@ -110,7 +110,7 @@ PMC_SUMMARIES = {
 # measured beside the headline workload in the default run: (workload, steps, warm-up)
 ALSO = [("c1", 50, 10), ("ref_f32", 80, 5), ("c2", 240, 10), ("c3_1_8", 40, 5), ("c3_2_8", 40, 5), ("c3_4_8", 40, 5),
         ("decode_1", 50, 10), ("decode_4", 50, 10), ("decode_8", 50, 10), ("decode_16", 50, 10),
-        ("decode_gdim_1", 50, 10), ("decode_gdim_16", 50, 10),
+        ("decode_gdim_1", 50, 10), ("decode_gdim_16", 50, 10), ("decode_2_8_1", 50, 10), ("decode_2_8_16", 50, 10),
         ("c4_b1", 50, 10), ("c4_b4", 50, 10), ("c4_b16", 50, 10),
         ("sparsify_c2", 100, 5), ("sparsify_c3_2_8", 20, 5), ("c5_step", 20, 3), ("c5_train", 20, 3)]
 
@@ -397,10 +397,10 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
     gc.disable()            # no collector pause of the host inside the timed region
     t0 = time.perf_counter()
     events[0].record(stream)
-    for g in range(len(bounds) - 1):
-        for _ in range(bounds[g], bounds[g + 1]):
+    for gi in range(len(bounds) - 1):
+        for _ in range(bounds[gi], bounds[gi + 1]):
             run_once()
-        events[g + 1].record(stream)
+        events[gi + 1].record(stream)
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / (steps * per)
     gc.enable()

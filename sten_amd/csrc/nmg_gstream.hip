@@ -133,16 +133,15 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
 #pragma unroll
         for (int tb = 0; tb < TB; tb++) acc[q][tb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // Two register sets: the loads of the next tile are in flight while a tile is multiplied.  A
-    // wavefront has few tiles (three for 4096 x 11008) and the kernel lives on the bytes it has in
-    // flight: sixteen wavefronts per CU, each with its first two tiles requested before anything
-    // else happens and the third as soon as the first has been multiplied.  The loads are
+    // NS register sets, one per tile of 32 lines: a wavefront has few tiles (three for 4096 x 11008)
+    // and the kernel lives on the bytes it has in flight, so every wavefront requests its whole
+    // range before anything else happens and multiplies the tiles as they land.  The loads are
     // instruction statements with a counted wait of their own -- left to the compiler, every wait
-    // in the loop is for *all* loads in flight, and the third tile is requested only when the
-    // second has landed.  A wavefront issues exactly OPS loads per tile and they complete in issue
-    // order, so with the next tile requested `vmcnt(OPS)` means "this tile has landed"; every
-    // register of the set passes through the wait, so the compiler orders its uses behind it (that
-    // nothing touches them earlier is checked on the compiled code, `python -m sten_amd.isa_check`).
+    // is for *all* loads in flight.  A wavefront issues exactly OPS loads per tile and they
+    // complete in issue order, so `vmcnt(j OPS)` means "all but the last j tiles have landed";
+    // every register of the set passes through the wait, so the compiler orders its uses behind it
+    // (that nothing touches them earlier is checked on the compiled code,
+    // `python -m sten_amd.isa_check`).
     typedef uint32_t gs_u32x2 __attribute__((ext_vector_type(2)));
     using VT = std::conditional_t<VB == 16, u32x4, std::conditional_t<VB == 8, gs_u32x2, uint32_t>>;
     struct Regs {
@@ -194,22 +193,14 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
             R.xmask[tb] = in_range ? x_live[tb] : 0u;
         }
     };
-    // the tile in R has landed: the next one (or its stand-in) was requested after it
-    auto landed = [&](Regs &R) __attribute__((always_inline)) {
+    // tile k has landed: the NS - 1 - k tiles requested behind it may still be on their way
+    auto landed = [&](Regs &R, auto left_tag) __attribute__((always_inline)) {
+        constexpr int LEFT = decltype(left_tag)::value;
         asm volatile("s_waitcnt vmcnt(%17)"
                      : "+v"(R.vals[0]), "+v"(R.vals[1]), "+v"(R.vals[2]), "+v"(R.vals[3]), "+v"(R.vals[4]), "+v"(R.vals[5]),
                        "+v"(R.vals[6]), "+v"(R.vals[7]), "+v"(R.pats[0]), "+v"(R.pats[1]), "+v"(R.pats[2]), "+v"(R.pats[3]),
                        "+v"(R.pats[4]), "+v"(R.pats[5]), "+v"(R.pats[6]), "+v"(R.pats[7]), "+v"(R.xf[0])
-                     : "n"((NS - 1) * OPS)
-                     : "memory");
-    };
-    // the same with nothing left in flight
-    auto drained = [&](Regs &R) __attribute__((always_inline)) {
-        asm volatile("s_waitcnt vmcnt(0)"
-                     : "+v"(R.vals[0]), "+v"(R.vals[1]), "+v"(R.vals[2]), "+v"(R.vals[3]), "+v"(R.vals[4]), "+v"(R.vals[5]),
-                       "+v"(R.vals[6]), "+v"(R.vals[7]), "+v"(R.pats[0]), "+v"(R.pats[1]), "+v"(R.pats[2]), "+v"(R.pats[3]),
-                       "+v"(R.pats[4]), "+v"(R.pats[5]), "+v"(R.pats[6]), "+v"(R.pats[7]), "+v"(R.xf[0])
-                     :
+                     : "n"(LEFT * OPS)
                      : "memory");
     };
     auto word = [](const VT &v, int w) __attribute__((always_inline)) -> uint32_t {
@@ -217,7 +208,7 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
         else return v;
     };
 
-    // The first two tiles are requested before anything else happens; the selector table is built
+    // All tiles are requested before anything else happens; the selector table is built
     // while they are on their way, from the order table in the kernel arguments (scalar loads: no
     // vector-memory operation of the compiler's own sits between the counted ones).  Entry
     // (par, p, r) = byte selectors that fetch the value kept at position r into the low half of a
@@ -284,27 +275,19 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
         }
     };
 
-    // Every turn of the loop issues the same operations whatever the range holds: beyond the last
-    // tile the loads repeat the range's first group (`GS_NONE`: cache hits, masked to zero, never
-    // multiplied into anything but zeros), so the counted wait is one constant, the loop is one
-    // block, and no register set is written on one path and left alone on another.  The scheduler fences keep a tile's last reads of a register set
-    // above the loads that refill it: the old and the new contents then share their registers, and
-    // no copy of a register with a load in flight appears at the loop's back edge.
-    for (uint32_t t = 0; t < ntiles; t += NS) {
-#pragma unroll
-        for (int k = 0; k < NS; k++) {
-            landed(rs[k]);
-            __builtin_amdgcn_sched_barrier(0);
-            multiply_tile(rs[k]);      // (an absent tile meets activations masked to zero)
-            __builtin_amdgcn_sched_barrier(0);
-            issue_tile(rs[k], t + NS + k < ntiles ? 32 * (t + NS + k) : GS_NONE);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-    // the last loads bring nothing that is read: their registers pass through the final wait, so
-    // that none is handed to the code below while a load may still land in it
-#pragma unroll
-    for (int k = 0; k < NS; k++) drained(rs[k]);
+    // One round: the host cuts the reduction so that a wavefront's range fits its register sets
+    // (32 NS lines), everything was requested above, and tile k waits for the NS - 1 - k tiles
+    // behind it at most.  The last wait leaves nothing in flight.
+    auto use = [&](Regs &R, auto k_tag) __attribute__((always_inline)) {
+        constexpr int K = decltype(k_tag)::value;
+        landed(R, std::integral_constant<int, NS - 1 - K>{});
+        __builtin_amdgcn_sched_barrier(0);
+        if ((uint32_t)K < ntiles) multiply_tile(R);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    use(rs[0], std::integral_constant<int, 0>{});
+    use(rs[1], std::integral_constant<int, 1>{});
+    if constexpr (NS == 3) use(rs[2], std::integral_constant<int, 2>{});
     __syncthreads();
 
     // Sums of the wavefronts: the upper half writes a slab each, the lower half adds theirs to the
@@ -355,6 +338,8 @@ static int gstream_plan(int64_t G, int64_t S, int m, int *spans, int *slices, in
     const int64_t quantum = 8 * GS_WAVES;
     int64_t lines = (G + sl - 1) / sl;
     lines = std::max<int64_t>((lines + quantum - 1) / quantum * quantum, 32 * GS_WAVES);
+    // a wavefront requests its whole range at once: at most as many tiles of 32 lines as it has register sets
+    lines = std::min<int64_t>(lines, 32 * GS_SETS * GS_WAVES);
     sl = (G + lines - 1) / lines;
     *spans = (int)sp;
     *slices = (int)std::max<int64_t>(sl, 1);
@@ -412,6 +397,7 @@ extern "C" int nmg_spmm_gstream(const void *d_pk_val, const void *d_pk_pat, int6
                 "workspace too small: %lld bytes given, %lld needed (nmg_spmm_gstream_plan)", (long long)ws_bytes,
                 (long long)((int64_t)slices * T * P.part_ld * 4));
     NMG_REQUIRE((int64_t)P.spans * slices <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
+    NMG_REQUIRE(P.slice_lines <= 32 * GS_SETS * GS_WAVES, NMG_ERR_UNSUPPORTED, "a slice beyond the register sets of its wavefronts");
     NMG_REQUIRE((P.slice_lines / GS_WAVES + 8) * nb * n * 2 < ((int64_t)1 << 31) && nb * n * 2 < (1 << 24) &&
                     P.slice_lines / GS_WAVES < (1 << 23),
                 NMG_ERR_UNSUPPORTED, "lines of more than 16 MiB, or the lines of one wavefront span more than 2 GiB");

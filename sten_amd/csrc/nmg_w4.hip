@@ -289,18 +289,23 @@ __global__ __launch_bounds__(64 * NW) void w4_linear_kernel(W4Params P)
 }
 
 // The same product with the activations staged through LDS: a wavefront's direct activation loads
-// touch 32 bytes of a token row per instruction; here the next group's 16 token rows x 256 bytes
-// arrive by row-contiguous DMA loads into a staging area private to the wavefront (no barrier),
-// issued before the group's weight loads so that one counted wait covers both.  One group is in
-// flight while the previous one is multiplied; 16-byte pieces of a row are XOR-swizzled with the
-// row number so that a fragment read hits distinct banks.
-template <int NW, int ND>
+// touch 32 bytes of a token row per instruction; here a group's 4 ND token rows x 256 bytes arrive
+// by row-contiguous DMA loads into a staging area private to the wavefront (no barrier), issued
+// before the group's weight loads so that one counted wait covers both; 16-byte pieces of a row
+// are XOR-swizzled with the row number so that a fragment read hits distinct banks.  A wavefront
+// keeps NS groups in flight (four up to 8 tokens: all of its range of a 4096-wide reduction is
+// requested before anything else happens; two beyond, where a group's activations take 3-4 KiB of
+// LDS).  Groups are refilled while a whole round of real ones is left; the last round waits for
+// exactly the groups behind each one and requests nothing, so no load is in flight at the end
+// that nobody reads.  A stand-in (fewer groups than sets, or the refills of the round before the
+// last) reads one cache line at the start of the operands.
+template <int NW, int ND, int NS>
 __global__ __launch_bounds__(64 * NW) void w4_linear_staged_kernel(W4Params P)
 {
     constexpr int OPS = ND + 3;
-    constexpr int BUF = 16 * 256;
+    constexpr int BUF = ND * 1024;
+    static_assert((NS - 1) * OPS < 64, "vmcnt is a 6-bit counter");
     extern __shared__ __align__(16) unsigned char w4_smem[];
-    static_assert(NW * 2 * BUF >= NW * 32 * 17 * 4, "the reduction buffer reuses the staging area");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int mb = blockIdx.x;
@@ -308,7 +313,7 @@ __global__ __launch_bounds__(64 * NW) void w4_linear_staged_kernel(W4Params P)
     const int j = lane & 31, h = lane >> 5;
     const int per = (KQ + NW - 1) / NW;
     const int kq_lo = wave * per, kq_hi = min(KQ, kq_lo + per);
-    unsigned char *stage = w4_smem + wave * (2 * BUF);
+    unsigned char *stage = w4_smem + wave * (NS * BUF);
 
     f32x16 acc;
 #pragma unroll
@@ -337,30 +342,39 @@ __global__ __launch_bounds__(64 * NW) void w4_linear_staged_kernel(W4Params P)
         uint2 ix;
         uint32_t s;
     };
-    WSet ws[2];
-    auto issue = [&](int kq, unsigned char *buf, WSet &W) {
-        const int kc = min(kq, KQ - 1);       // beyond the range: same count of operations, data unused
+    WSet ws[NS];
+    // (`s_nop 4`: a scalar base that the compiler reads back from a vector register lane needs five
+    // wait states before a memory instruction may use it, and the compiler does not look into
+    // instruction statements)
+    auto issue = [&](int kq, unsigned char *buf, WSet &W) __attribute__((always_inline)) {
+        const bool real = kq < kq_hi;
+        const int kc = real ? kq : 0;         // a stand-in: same count of operations, one cache line each
         const unsigned char *xb = (const unsigned char *)P.x + (int64_t)kc * 256;
 #pragma unroll
         for (int i = 0; i < ND; i++)
             __builtin_amdgcn_global_load_lds((glb_ptr_t)(xb + x_off[i]), (lds_ptr_t)(buf + i * 1024), 16, 0, 0);
         const unsigned char *pb = bv + (int64_t)kc * 1024, *pm = mv + (int64_t)kc * 512, *ps = sv + (int64_t)kc * 64;
-        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(W.a) : "v"(lane16), "s"(pb) : "memory");
-        asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(W.ix) : "v"(lane8), "s"(pm) : "memory");
-        asm volatile("global_load_ushort %0, %1, %2" : "=v"(W.s) : "v"(row2), "s"(ps) : "memory");
+        const uint32_t o16 = real ? lane16 : 0u, o8 = real ? lane8 : 0u, o2 = real ? row2 : 0u;
+        asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2" : "=v"(W.a) : "v"(o16), "s"(pb) : "memory");
+        asm volatile("s_nop 4\n\tglobal_load_dwordx2 %0, %1, %2" : "=v"(W.ix) : "v"(o8), "s"(pm) : "memory");
+        asm volatile("s_nop 4\n\tglobal_load_ushort %0, %1, %2" : "=v"(W.s) : "v"(o2), "s"(ps) : "memory");
     };
-    auto consume = [&](int kq, const unsigned char *buf, const WSet &W) {
+    // set k has landed: `left` groups requested behind it may still be on their way
+    auto landed = [&](WSet &W, auto left_tag) __attribute__((always_inline)) {
+        constexpr int LEFT = decltype(left_tag)::value;
+        asm volatile("s_waitcnt vmcnt(%3)" : "+v"(W.a), "+v"(W.ix), "+v"(W.s) : "n"(LEFT * OPS) : "memory");
+    };
+    auto consume = [&](const unsigned char *buf, const WSet &W) __attribute__((always_inline)) {
         u32x4 b[4][2];
 #pragma unroll
         for (int ins = 0; ins < 4; ins++)
 #pragma unroll
             for (int c = 0; c < 2; c++) b[ins][c] = *(const u32x4 *)(buf + b_off[ins][c]);
-        const bool live = kq < kq_hi;
         union {
             uint16_t u;
             _Float16 f;
         } sc;
-        sc.u = live ? (uint16_t)W.s : (uint16_t)0;      // scale 0 silences a group beyond the range
+        sc.u = (uint16_t)W.s;
         const w4_f16x2 s2 = {sc.f, sc.f};
         const uint32_t words[4] = {W.a.x, W.a.y, W.a.z, W.a.w};
 #pragma unroll
@@ -384,24 +398,33 @@ __global__ __launch_bounds__(64 * NW) void w4_linear_staged_kernel(W4Params P)
         }
     };
 
-    issue(kq_lo, stage, ws[0]);
-    for (int kq0 = kq_lo; kq0 < kq_hi; kq0 += 2) {
 #pragma unroll
-        for (int u = 0; u < 2; u++) {
-            const int kq = kq0 + u;
-            issue(kq + 1, stage + ((u + 1) & 1) * BUF, ws[(u + 1) & 1]);
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(OPS) : "memory");   // group kq has landed
+    for (int k = 0; k < NS; k++) issue(kq_lo + k, stage + k * BUF, ws[k]);
+    int kq0 = kq_lo;
+    for (; kq0 + NS < kq_hi; kq0 += NS) {
+#pragma unroll
+        for (int k = 0; k < NS; k++) {
+            landed(ws[k], std::integral_constant<int, NS - 1>{});
             __builtin_amdgcn_sched_barrier(0);
-            consume(kq, stage + u * BUF, ws[u]);
+            consume(stage + k * BUF, ws[k]);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(kq0 + NS + k, stage + k * BUF, ws[k]);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
-    // the last loads (beyond the wavefront's range) are in flight and unused: their registers pass
-    // through the final wait, so that none is reused while a load may still land in it
-    asm volatile("s_waitcnt vmcnt(0)"
-                 : "+v"(ws[0].a), "+v"(ws[0].ix), "+v"(ws[0].s), "+v"(ws[1].a), "+v"(ws[1].ix), "+v"(ws[1].s)
-                 :
-                 : "memory");
+    auto last = [&](WSet &W, auto k_tag) __attribute__((always_inline)) {
+        constexpr int K = decltype(k_tag)::value;
+        landed(W, std::integral_constant<int, NS - 1 - K>{});
+        __builtin_amdgcn_sched_barrier(0);
+        if (kq0 + K < kq_hi) consume(stage + K * BUF, W);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    last(ws[0], std::integral_constant<int, 0>{});
+    last(ws[1], std::integral_constant<int, 1>{});
+    if constexpr (NS == 4) {
+        last(ws[2], std::integral_constant<int, 2>{});
+        last(ws[3], std::integral_constant<int, 3>{});
+    }
     __syncthreads();
     float(*red)[32][17] = (float(*)[32][17])w4_smem;
     if (j < 16) {
@@ -423,7 +446,10 @@ __global__ __launch_bounds__(64 * NW) void w4_linear_staged_kernel(W4Params P)
 
 template <int NW, int ND> static void w4_launch_staged(const W4Params &P, hipStream_t s)
 {
-    hipLaunchKernelGGL((w4_linear_staged_kernel<NW, ND>), dim3((unsigned)P.MB), dim3(64 * NW), (size_t)NW * 2 * 16 * 256, s, P);
+    constexpr int NS = ND <= 2 ? 4 : 2;
+    // (the sums of the wavefronts reuse the staging area: 32 x 17 floats per wavefront)
+    constexpr size_t lds = (size_t)NW * (NS * ND * 1024 > 32 * 17 * 4 ? NS * ND * 1024 : 32 * 17 * 4);
+    hipLaunchKernelGGL((w4_linear_staged_kernel<NW, ND, NS>), dim3((unsigned)P.MB), dim3(64 * NW), lds, s, P);
 }
 template <int NW> static void w4_launch_staged_nd(const W4Params &P, hipStream_t s)
 {
