@@ -365,6 +365,8 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
     # on; the training step needs 60-80 ms to come down from 1.5-1.7 ms to 1.29 ms.  The untimed
     # steps are therefore repeated until SETTLE_S of load have passed, so that the K timed steps
     # see the clocks a workload that keeps running sees.
+    gc.collect()
+    gc.disable()            # no collector pause of the host between the settling and the timed steps, or inside them
     settle_end = time.perf_counter() + SETTLE_S
     settle_steps = 0
     est = 1.0
@@ -393,8 +395,6 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
     bounds.append(steps)
     stream = torch.cuda.current_stream()
     events = [torch.cuda.Event(enable_timing=True) for _ in bounds]
-    gc.collect()
-    gc.disable()            # no collector pause of the host inside the timed region
     t0 = time.perf_counter()
     events[0].record(stream)
     for gi in range(len(bounds) - 1):
@@ -447,7 +447,7 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="target_2_4", choices=sorted(WORKLOADS))
     ap.add_argument("--kernel", default="auto")
