@@ -71,7 +71,7 @@ template <typename T, int N>
 __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
 {
     static_assert(N == 1 || N == 2 || N == 4, "1:8, 2:8, 4:8");
-    constexpr int NS = N == 4 ? 3 : 4;       // register sets: what fits beside each other
+    constexpr int NS = N == 4 ? 2 : 4;       // register sets: what fits beside each other (a set of 4:8 takes 69 registers)
     constexpr int PB = 4 * N * 2;            // bytes of values a lane reads per half set: 8, 16, 32
     constexpr int VL = PB / 16 > 0 ? PB / 16 : 1;   // loads they take
     constexpr int NPAR = N == 1 ? 2 : 1;
@@ -80,6 +80,7 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
     using VT = std::conditional_t<PB == 8, ss_u32x2, u32x4>;
 
     __shared__ __align__(16) uint32_t tab[NPAR * MAXC * 4];
+    __shared__ uint32_t ord[(MAXC * N + 3) / 4];
     __shared__ __align__(16) float red[SS_WAVES][16][SS_LINES + 1];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -117,7 +118,7 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
     // written by the vector unit needs five wait states before a memory instruction may read it;
     // the compiler does not look into instruction statements)
     auto issue_set = [&](Regs &R, uint32_t rel) __attribute__((always_inline)) {
-        const bool in_range = rel < nsets;
+        const bool in_range = rel < nsets;      // (SS_NONE lies beyond any range)
 #pragma unroll
         for (int rb = 0; rb < 2; rb++)
 #pragma unroll
@@ -167,21 +168,27 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
     // the block from its value words (bytes 0 .. 7 of the pair {high, low}; 0x0c: zero).  The order
     // table comes with the kernel arguments (scalar loads: no vector-memory operation of the
     // compiler's own sits between the counted ones).
+    // (the order table goes to LDS first, one word per thread picked with compile-time indices: a
+    // lane-dependent index into the kernel arguments would put the table into scratch memory)
+    if (tid < (MAXC * N + 3) / 4) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int q = 0; q < (MAXC * N + 3) / 4; q++)
+            if (tid == q) word = P.order[q];
+        ord[tid] = word;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     for (int e = tid; e < NPAR * P.c * 4; e += SS_WAVES * 64) {
         const int w = e & 3, p = (e >> 2) % P.c, par = (e >> 2) / P.c;
         uint32_t sel = 0x0c0c0c0cu;
 #pragma unroll
-        for (int pp = 0; pp < MAXC; pp++)
-#pragma unroll
-            for (int j = 0; j < N; j++) {
-                const int k = pp * N + j;
-                const uint32_t pos = (P.order[k >> 2] >> (8 * (k & 3))) & 0xffu;
-                // value j of the block sits at half-word hw of the value words the perm sees
-                const uint32_t hw = N == 1 ? (uint32_t)par : (uint32_t)j;
-                const uint32_t two = (2 * hw) | ((2 * hw + 1) << 8);
-                if (pp < P.c && pp == p && (pos >> 1) == (uint32_t)w)
-                    sel = (sel & ~(0xffffu << (16 * (pos & 1)))) | (two << (16 * (pos & 1)));
-            }
+        for (int j = 0; j < N; j++) {
+            const uint32_t pos = ((const unsigned char *)ord)[p * N + j];
+            // value j of the block sits at half-word hw of the value words the perm sees
+            const uint32_t hw = N == 1 ? (uint32_t)par : (uint32_t)j;
+            const uint32_t two = (2 * hw) | ((2 * hw + 1) << 8);
+            if ((pos >> 1) == (uint32_t)w) sel = (sel & ~(0xffffu << (16 * (pos & 1)))) | (two << (16 * (pos & 1)));
+        }
         tab[e] = sel;
     }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -217,20 +224,33 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
             }
     };
 
-    // One round: the host has checked that a wavefront's range fits its register sets (reductions
-    // up to 8192 at 1:8 and 2:8, 6144 at 4:8), so everything was requested above and set k waits
-    // for the NS - 1 - k sets behind it at most.  The last wait leaves nothing in flight.
-    auto use = [&](Regs &R, auto k_tag) __attribute__((always_inline)) {
+    // A round: NS sets were requested together, set k waits for the NS - 1 - k sets behind it at
+    // most, and the last wait leaves nothing in flight.  Reductions up to 8192 (4096 at 4:8) are one
+    // round, requested above; a longer one goes on in rounds of the same shape, each requested when
+    // the one before has been multiplied (no register set then carries a load across the loop's
+    // back edge; the price is a pause of the loads between two rounds).
+    auto use = [&](Regs &R, uint32_t base, auto k_tag) __attribute__((always_inline)) {
         constexpr int K = decltype(k_tag)::value;
         landed(R, std::integral_constant<int, NS - 1 - K>{});
         __builtin_amdgcn_sched_barrier(0);
-        if ((uint32_t)K < nsets) multiply_set(R);
+        if (base + K < nsets) multiply_set(R);
         __builtin_amdgcn_sched_barrier(0);
     };
-    use(rs[0], std::integral_constant<int, 0>{});
-    use(rs[1], std::integral_constant<int, 1>{});
-    use(rs[2], std::integral_constant<int, 2>{});
-    if constexpr (NS == 4) use(rs[3], std::integral_constant<int, 3>{});
+    auto use_round = [&](uint32_t base) __attribute__((always_inline)) {
+        use(rs[0], base, std::integral_constant<int, 0>{});
+        use(rs[1], base, std::integral_constant<int, 1>{});
+        if constexpr (NS == 4) {
+            use(rs[2], base, std::integral_constant<int, 2>{});
+            use(rs[3], base, std::integral_constant<int, 3>{});
+        }
+    };
+    use_round(0);
+    for (uint32_t base = NS; base < nsets; base += NS) {
+#pragma unroll
+        for (int k = 0; k < NS; k++) issue_set(rs[k], base + k < nsets ? base + k : SS_NONE);
+        __builtin_amdgcn_sched_barrier(0);
+        use_round(base);
+    }
 #undef NMG_SS_REST
 #undef NMG_SS_V0
 #undef NMG_SS_V1
@@ -360,8 +380,7 @@ extern "C" int nmg_spmm_sstream(const void *d_lp_val, const void *d_lp_pat, int6
     P.c = (int)binom(m, n);
     const int64_t sets = nb / 32;
     P.sets_per_wave = (int)((sets + SS_WAVES - 1) / SS_WAVES);
-    NMG_REQUIRE(P.sets_per_wave <= (n == 4 ? 3 : 4), NMG_ERR_UNSUPPORTED,
-                "the streaming product takes reductions up to %d", n == 4 ? 6144 : 8192);
+    NMG_REQUIRE((int64_t)P.sets_per_wave * 4 * 64 * 8 * n < ((int64_t)1 << 31), NMG_ERR_UNSUPPORTED, "reduction too long");
     const int8_t *ord = host_order(n, m);
     NMG_REQUIRE(ord != nullptr && binom(m, n) * n <= (int64_t)sizeof(P.order), NMG_ERR_ARG, "invalid n:m = %d:%d", n, m);
     for (size_t e = 0; e < sizeof(P.order) / 4; e++) P.order[e] = 0;

@@ -551,7 +551,10 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
     if (kname in ("auto", "sstream") and reduce_sparse == 1 and T <= 16 and len(lay.dense_shape) == 2
             and x.dtype in (torch.float16, torch.bfloat16)
             and native.load().nmg_spmm_sstream_supported(lay.n, lay.m)
-            and K % 256 == 0 and K <= (6144 if lay.n == 4 else 8192)
+            and K % 256 == 0
+            # a workgroup is 32 lines: with fewer than 192 of them the operand of the sparse matrix cores
+            # (two workgroups per 32 lines) streams faster although it is larger (4:8 has none)
+            and (kname == "sstream" or lay.n == 4 or O >= 192 * 32)
             and (T == 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0
             and T * max(x.stride(0), K) * 2 < 2 ** 31 and 32 * (K // 8) * lay.n * 2 < 2 ** 31):
         lp_val, lp_pat = weight.lanepack8()
@@ -563,7 +566,7 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
         return y
     if kname == "sstream":
         raise native.NmgError("the streaming product along the sparse dim needs 16-bit data, at most 16 tokens, "
-                              "1:8, 2:8 or 4:8 and a reduction extent that is a multiple of 256, at most 8192 (4:8: 6144)")
+                              "1:8, 2:8 or 4:8 and a reduction extent that is a multiple of 256")
     packed = None
     if smf_ok and kname in ("auto", "skinny", "smfmac"):
         packed = weight.fragpack()

@@ -564,8 +564,11 @@ def test_few_tokens_along_the_group_dim_stream_the_compressed_lines(dtype, M, K,
     (torch.bfloat16, 512, 1024, 2, 8, 32),
     (torch.float16, 200, 2560, 1, 8, 4),       # lines that are not a multiple of 32, ten sets over eight wavefronts
     (torch.float16, 264, 768, 4, 8, 2),        # 4:8: no operand of the sparse matrix cores exists
-    (torch.bfloat16, 96, 6144, 4, 8, 1),       # 24 sets: three per wavefront, the most 4:8 takes
-    (torch.float16, 1056, 8192, 2, 8, 8),      # 32 sets: four per wavefront
+    (torch.bfloat16, 96, 6144, 4, 8, 1),       # 24 sets: three per wavefront, one round at 4:8
+    (torch.float16, 1056, 8192, 2, 8, 8),      # 32 sets: four per wavefront, one round
+    (torch.float16, 160, 16384, 2, 8, 4),      # 64 sets: two rounds of four per wavefront
+    (torch.bfloat16, 64, 11008 + 256, 4, 8, 2),    # 44 sets: six per wavefront (two rounds), the last wavefront with two
+    (torch.float16, 40, 9216 + 256, 1, 8, 16),     # 37 sets: five per wavefront (a second round of one set), the last wavefront with two
 ])
 def test_few_tokens_on_blocks_of_eight_stream_the_compressed_lines(dtype, M, K, n, m, g, T):
     # 1:8, 2:8, 4:8 with the blocks along the reduction and <= 16 tokens: the rowpack operand, streamed
@@ -578,12 +581,15 @@ def test_few_tokens_on_blocks_of_eight_stream_the_compressed_lines(dtype, M, K, 
     ref = to_np(x).astype(np.float64) @ Wd.T
     y = sten.spmm(w, x.to(DEV), reduce_dim=1, kernel="sstream")
     assert rel_l2(to_np(y), ref) <= TOL[dtype]
-    yb = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)      # the automatic choice takes the same route
+    yb = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1, kernel="sstream")
     assert rel_l2(to_np(yb), ref + to_np(b).astype(np.float64)) <= TOL[dtype]
+    # the automatic choice: this route for 4:8 and from 6144 lines on, the sparse matrix cores below
+    ya = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)
+    assert rel_l2(to_np(ya), ref + to_np(b).astype(np.float64)) <= TOL[dtype]
     xs = torch.zeros((2 * T, K + 8), dtype=dtype, device=DEV)[::2, :K]
     xs.copy_(x.to(DEV))
     for _ in range(3):
-        assert torch.equal(sten.spmm(w, xs, reduce_dim=1), y)
+        assert torch.equal(sten.spmm(w, xs, reduce_dim=1, kernel="sstream"), y)
     if n < 4:
         y2 = sten.spmm(w, x.to(DEV), reduce_dim=1, kernel="skinny")      # the operand of the sparse matrix cores
         assert rel_l2(to_np(y2), to_np(y).astype(np.float64)) <= 2 * TOL[dtype]

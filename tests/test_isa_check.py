@@ -181,3 +181,30 @@ def test_scalar_register_written_by_the_vector_unit_needs_wait_states_before_a_h
 \ts_waitcnt vmcnt(0)
 """)
     assert p == []
+
+
+
+def test_spill_among_outstanding_hand_issued_loads_is_reported():
+    # the compiler's wait for its scratch operation drains the loads that were meant to stay in flight
+    p = run("""
+\t;;#ASMSTART
+\tglobal_load_dwordx4 v[10:13], v2, s[4:5]
+\t;;#ASMEND
+\tscratch_load_dword v40, off, off offset:4
+\t;;#ASMSTART
+\ts_waitcnt vmcnt(0)
+\t;;#ASMEND
+\tv_add_u32_e32 v1, v10, v11
+""")
+    assert any("scratch traffic while hand-issued loads are outstanding" in q for q in p)
+    clean = run("""
+\tscratch_store_dword off, v40, off offset:4
+\t;;#ASMSTART
+\tglobal_load_dwordx4 v[10:13], v2, s[4:5]
+\t;;#ASMEND
+\t;;#ASMSTART
+\ts_waitcnt vmcnt(0)
+\t;;#ASMEND
+\tv_add_u32_e32 v1, v10, v11
+""")
+    assert clean == []
