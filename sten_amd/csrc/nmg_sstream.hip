@@ -67,11 +67,14 @@ constexpr int SS_WAVES = 8;
 constexpr int SS_LINES = 32;            // output lines per workgroup
 constexpr uint32_t SS_NONE = 0xffffff00u;
 
-template <typename T, int N>
+// RBN = 2: a workgroup takes the 32 lines of a group; RBN = 1: two workgroups share a group, 16 lines
+// each (weights of few lines: twice the workgroups pull the operand; both read the token rows).
+template <typename T, int N, int RBN>
 __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
 {
+    static_assert(RBN == 1 || RBN == 2, "one or two row blocks of 16 lines");
     static_assert(N == 1 || N == 2 || N == 4, "1:8, 2:8, 4:8");
-    constexpr int NS = N == 4 ? 2 : 4;       // register sets: what fits beside each other (a set of 4:8 takes 69 registers)
+    constexpr int NS = (N == 4 && RBN == 2) ? 2 : 4;   // register sets: what fits beside each other (a set of 4:8 takes 69 registers)
     constexpr int PB = 4 * N * 2;            // bytes of values a lane reads per half set: 8, 16, 32
     constexpr int VL = PB / 16 > 0 ? PB / 16 : 1;   // loads they take
     constexpr int NPAR = N == 1 ? 2 : 1;
@@ -81,12 +84,14 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
 
     __shared__ __align__(16) uint32_t tab[NPAR * MAXC * 4];
     __shared__ uint32_t ord[(MAXC * N + 3) / 4];
-    __shared__ __align__(16) float red[SS_WAVES][16][SS_LINES + 1];
+    __shared__ __align__(16) float red[SS_WAVES][16][16 * RBN + 1];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int i = lane & 15, kq = lane >> 4;
-    const int64_t l0 = (int64_t)blockIdx.x * SS_LINES;
+    const int64_t group = RBN == 2 ? (int64_t)blockIdx.x : (int64_t)(blockIdx.x >> 1);
+    const int rb0 = RBN == 2 ? 0 : (int)(blockIdx.x & 1);      // first row block of the workgroup
+    const int64_t l0 = group * SS_LINES + rb0 * 16;
 
     // the wavefront's sets of 32 blocks
     const uint32_t total_sets = (uint32_t)(P.nb / 32);
@@ -94,21 +99,23 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
     const uint32_t nsets = min(s_lo + P.sets_per_wave, total_sets) - s_lo;
     // a set of the operand: [rb][a][lane] shares of PB / 4 bytes
     constexpr uint32_t VSET = 4 * 64 * PB, PSET = 4 * 64 * 4;
-    const unsigned char *vwave = P.lp_val + ((int64_t)blockIdx.x * total_sets + (nsets ? s_lo : 0)) * VSET;
-    const unsigned char *pwave = P.lp_pat + ((int64_t)blockIdx.x * total_sets + (nsets ? s_lo : 0)) * PSET;
+    const unsigned char *vwave = P.lp_val + (group * total_sets + (nsets ? s_lo : 0)) * VSET + rb0 * (2 * 64 * PB);
+    const unsigned char *pwave = P.lp_pat + (group * total_sets + (nsets ? s_lo : 0)) * PSET + rb0 * (2 * 64 * 4);
     const unsigned char *xwave = P.x + (int64_t)(nsets ? s_lo : 0) * 32 * 16;
     const bool tok_live = i < P.T;
     const uint32_t x_lane = (tok_live ? (uint32_t)(i * P.ldx * 2) : 0u) + (uint32_t)kq * 16;
 
-    f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+    f32x4 acc[RBN];
+#pragma unroll
+    for (int rb = 0; rb < RBN; rb++) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     struct Regs {
-        VT vals[2][2][VL];      // [row block][half set][load]
-        uint32_t pats[2][2];
+        VT vals[RBN][2][VL];    // [row block][half set][load]
+        uint32_t pats[RBN][2];
         u32x4 xf[2][4];         // [half set][block of the lane]
         uint32_t xmask;
     } rs[NS];
-    constexpr int OPS = 4 * (VL + 1) + 8;
+    constexpr int OPS = 2 * RBN * (VL + 1) + 8;
     static_assert((NS - 1) * OPS < 64, "vmcnt is a 6-bit counter");
 
     // loads of set `rel` of the wavefront's range (SS_NONE: a stand-in beyond the range -- every
@@ -120,7 +127,7 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
     auto issue_set = [&](Regs &R, uint32_t rel) __attribute__((always_inline)) {
         const bool in_range = rel < nsets;      // (SS_NONE lies beyond any range)
 #pragma unroll
-        for (int rb = 0; rb < 2; rb++)
+        for (int rb = 0; rb < RBN; rb++)
 #pragma unroll
             for (int a = 0; a < 2; a++) {
                 const uint32_t vo = in_range ? rel * VSET + (uint32_t)((rb * 2 + a) * 64 + lane) * PB : 0u;
@@ -145,18 +152,24 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
     };
     // Every register of a set passes through the counted wait, so the compiler orders its uses
     // behind it; that nothing touches them earlier is checked on the compiled code.
-#define NMG_SS_REST(R)                                                                                             \
-    "+v"(R.pats[0][0]), "+v"(R.pats[0][1]), "+v"(R.pats[1][0]), "+v"(R.pats[1][1]), "+v"(R.xf[0][0]), "+v"(R.xf[0][1]), \
-        "+v"(R.xf[0][2]), "+v"(R.xf[0][3]), "+v"(R.xf[1][0]), "+v"(R.xf[1][1]), "+v"(R.xf[1][2]), "+v"(R.xf[1][3])
-#define NMG_SS_V0(R) "+v"(R.vals[0][0][0]), "+v"(R.vals[0][1][0]), "+v"(R.vals[1][0][0]), "+v"(R.vals[1][1][0])
-#define NMG_SS_V1(R) "+v"(R.vals[0][0][VL - 1]), "+v"(R.vals[0][1][VL - 1]), "+v"(R.vals[1][0][VL - 1]), "+v"(R.vals[1][1][VL - 1])
+#define NMG_SS_X(R)                                                                                          \
+    "+v"(R.xf[0][0]), "+v"(R.xf[0][1]), "+v"(R.xf[0][2]), "+v"(R.xf[0][3]), "+v"(R.xf[1][0]), "+v"(R.xf[1][1]), \
+        "+v"(R.xf[1][2]), "+v"(R.xf[1][3])
+#define NMG_SS_P(R, rb) "+v"(R.pats[rb][0]), "+v"(R.pats[rb][1])
+#define NMG_SS_V0(R, rb) "+v"(R.vals[rb][0][0]), "+v"(R.vals[rb][1][0])
+#define NMG_SS_V1(R, rb) "+v"(R.vals[rb][0][VL - 1]), "+v"(R.vals[rb][1][VL - 1])
     // set k of a round has landed: the NS - 1 - k sets behind it may still be on their way
+    // (every register of the set is named exactly once: a register named twice would be copied)
     auto landed = [&](Regs &R, auto left_tag) __attribute__((always_inline)) {
         constexpr int LEFT = decltype(left_tag)::value;
-        if constexpr (VL == 1)
-            asm volatile("s_waitcnt vmcnt(%16)" : NMG_SS_V0(R), NMG_SS_REST(R) : "n"(LEFT * OPS) : "memory");
+        if constexpr (RBN == 2 && VL == 1)
+            asm volatile("s_waitcnt vmcnt(%16)" : NMG_SS_V0(R, 0), NMG_SS_V0(R, 1), NMG_SS_P(R, 0), NMG_SS_P(R, 1), NMG_SS_X(R) : "n"(LEFT * OPS) : "memory");
+        else if constexpr (RBN == 2)
+            asm volatile("s_waitcnt vmcnt(%20)" : NMG_SS_V0(R, 0), NMG_SS_V0(R, 1), NMG_SS_V1(R, 0), NMG_SS_V1(R, 1), NMG_SS_P(R, 0), NMG_SS_P(R, 1), NMG_SS_X(R) : "n"(LEFT * OPS) : "memory");
+        else if constexpr (VL == 1)
+            asm volatile("s_waitcnt vmcnt(%12)" : NMG_SS_V0(R, 0), NMG_SS_P(R, 0), NMG_SS_X(R) : "n"(LEFT * OPS) : "memory");
         else
-            asm volatile("s_waitcnt vmcnt(%20)" : NMG_SS_V0(R), NMG_SS_V1(R), NMG_SS_REST(R) : "n"(LEFT * OPS) : "memory");
+            asm volatile("s_waitcnt vmcnt(%14)" : NMG_SS_V0(R, 0), NMG_SS_V1(R, 0), NMG_SS_P(R, 0), NMG_SS_X(R) : "n"(LEFT * OPS) : "memory");
     };
 
     // The wavefront's whole range is requested before anything else happens.  Every wavefront
@@ -204,7 +217,7 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
             for (int e = 0; e < 4; e++) {
                 const u32x4 xm = R.xf[a][e] & R.xmask;
 #pragma unroll
-                for (int rb = 0; rb < 2; rb++) {
+                for (int rb = 0; rb < RBN; rb++) {
                     const uint32_t p = (R.pats[rb][a] >> (8 * e)) & 0xffu;
                     const u32x4 sel = *(const u32x4 *)&tab[((N == 1 ? (e & 1) * P.c : 0) + p) * 4];
                     // the block's value words: n = 2: word e; n = 4: words 2 e, 2 e + 1; n = 1: word e / 2
@@ -251,21 +264,23 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
         __builtin_amdgcn_sched_barrier(0);
         use_round(base);
     }
-#undef NMG_SS_REST
+#undef NMG_SS_X
+#undef NMG_SS_P
 #undef NMG_SS_V0
 #undef NMG_SS_V1
 
     // sums of the wavefronts: lane (t = l % 16, rq = l / 16) holds token t, lines 16 rb + 4 rq + r
     const int rq = lane >> 4;
+    constexpr int WL = 16 * RBN;        // lines of the workgroup
     if (tok_live) {
 #pragma unroll
-        for (int rb = 0; rb < 2; rb++)
+        for (int rb = 0; rb < RBN; rb++)
 #pragma unroll
             for (int r = 0; r < 4; r++) red[wave][i][rb * 16 + 4 * rq + r] = acc[rb][r];
     }
     __syncthreads();
-    for (int e = tid; e < (int)P.T * SS_LINES; e += SS_WAVES * 64) {
-        const int tok = e / SS_LINES, ln = e % SS_LINES;
+    for (int e = tid; e < (int)P.T * WL; e += SS_WAVES * 64) {
+        const int tok = e / WL, ln = e % WL;
         const int64_t line = l0 + ln;
         if (line >= P.G) continue;
         float sum = 0.f;
@@ -386,16 +401,23 @@ extern "C" int nmg_spmm_sstream(const void *d_lp_val, const void *d_lp_pat, int6
     for (size_t e = 0; e < sizeof(P.order) / 4; e++) P.order[e] = 0;
     for (int64_t e = 0; e < binom(m, n) * n; e++) P.order[e >> 2] |= (uint32_t)(uint8_t)ord[e] << (8 * (e & 3));
     const int64_t groups = (G + SS_LINES - 1) / SS_LINES;
-    NMG_REQUIRE(groups <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
+    NMG_REQUIRE(groups <= 0x3fffffffLL, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid((unsigned)groups), block(SS_WAVES * 64);
-#define NMG_SS_N(TT)                                                                     \
-    switch (n) {                                                                           \
-    case 1: hipLaunchKernelGGL((sstream_kernel<TT, 1>), grid, block, 0, s, P); break;     \
-    case 2: hipLaunchKernelGGL((sstream_kernel<TT, 2>), grid, block, 0, s, P); break;     \
-    default: hipLaunchKernelGGL((sstream_kernel<TT, 4>), grid, block, 0, s, P); break;    \
+    // 32 lines per workgroup where that gives the chip enough workgroups, else 16 (the token rows are
+    // then read by twice the workgroups: up to 8 tokens)
+    const bool halves = groups < 192 && T <= 8;
+    const dim3 grid((unsigned)(halves ? 2 * groups : groups)), block(SS_WAVES * 64);
+#define NMG_SS_N(TT, RB)                                                                     \
+    switch (n) {                                                                               \
+    case 1: hipLaunchKernelGGL((sstream_kernel<TT, 1, RB>), grid, block, 0, s, P); break;     \
+    case 2: hipLaunchKernelGGL((sstream_kernel<TT, 2, RB>), grid, block, 0, s, P); break;     \
+    default: hipLaunchKernelGGL((sstream_kernel<TT, 4, RB>), grid, block, 0, s, P); break;    \
     }
-    if (dtype == NMG_F16) { NMG_SS_N(__half) } else { NMG_SS_N(__hip_bfloat16) }
+    if (dtype == NMG_F16) {
+        if (halves) { NMG_SS_N(__half, 1) } else { NMG_SS_N(__half, 2) }
+    } else {
+        if (halves) { NMG_SS_N(__hip_bfloat16, 1) } else { NMG_SS_N(__hip_bfloat16, 2) }
+    }
 #undef NMG_SS_N
     NMG_HIP_TRY(hipGetLastError());
     return NMG_OK;
