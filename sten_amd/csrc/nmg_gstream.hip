@@ -10,21 +10,21 @@
 //
 //  * V_MFMA_F32_16X16X32: A = 16 outputs x 32 lines, lane (i, kq) = (l % 16, l / 16) holds lines
 //    8 kq .. 8 kq + 7 of output row i.  A lane loads, for each of its 8 lines, the values and
-//    patterns of BL = 8 / m consecutive blocks (8 outputs): a quarter wavefront reads 16 * BL
-//    blocks of one line as one contiguous run (128 bytes of values at 2:4).  Output q of the lane
-//    (q = 0 .. 7) across its 8 lines is one A fragment, so a 32-line tile is 8 MFMAs, and row i of
-//    MFMA q is output 8 i + q of the wavefront's span of 128.
+//    patterns of BL = 16 / m consecutive blocks (16 outputs): a quarter wavefront reads 16 * BL
+//    blocks of one line as one contiguous run (256 bytes of values and 64 of patterns at 2:4).
+//    Output q of the lane (q = 0 .. 15) across its 8 lines is one A fragment, so a 32-line tile is
+//    16 MFMAs, and row i of MFMA q is output 16 i + q of the workgroup's span of 256.
 //  * Expansion: for a block with pattern p, position r holds value j(p, r) or nothing.  A table in
-//    LDS gives per (p, r) the byte selector pair of V_PERM_B32 that moves that value into a
-//    16-bit half (0x0c0c: zero); the selectors of lines u and u + 1 are joined by one V_PERM_B32
-//    and a second one picks the two halves out of the two lines' value words: two vector
-//    instructions per pair of dense weights.
-//  * A workgroup is 16 wavefronts on one span of 128 outputs (four per SIMD with 128 registers
-//    each: what bounds the kernel is the bytes it has in flight); they split the lines of the
-//    workgroup's slice of the reduction, add their sums in LDS one after the other (fixed order:
-//    results do not depend on timing) and write single-precision partial sums
-//    part[slice][token][output]; splitk_sum_kernel adds the slices in order, adds the bias and
-//    rounds once.
+//    LDS gives, per (pattern of line u, pattern of line u + 1, position r), the selector word with
+//    which one V_PERM_B32 builds the pair (weight of line u, weight of line u + 1) at position r
+//    from the two lines' value words (0x0c: a zero byte): one vector instruction per pair of dense
+//    weights, one 16-byte table read per four positions of a pair of lines.
+//  * A workgroup is 8 wavefronts on one span of 256 outputs and one slice of the reduction; every
+//    wavefront requests its whole range (up to three tiles of 32 lines) before anything else
+//    happens -- what bounds the kernel is the bytes it has in flight -- and multiplies the tiles
+//    as they land.  The wavefronts add their sums in LDS in a fixed order (results do not depend
+//    on timing) and write single-precision partial sums part[slice][token][output];
+//    splitk_sum_kernel adds the slices in order, adds the bias and rounds once.
 #include "nmg_common.h"
 #include "nmg_tile.h"
 
@@ -72,7 +72,7 @@ template <typename T, int N, int M, int OPL, int NW, int NS>
 __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
 {
     constexpr int TB = 1, GS_WAVES = NW, GS_OPL = OPL, GS_SPAN = 16 * OPL;
-    static_assert(NS == 2 || NS == 3, "two or three tiles in flight");
+    static_assert(NS == 2 || NS == 3, "two or three tiles per wavefront");
     static_assert((NW & (NW - 1)) == 0 && NW >= 2, "a power of two of wavefronts");
     static_assert(M == 4 || M == 8, "blocks of 4 or 8 outputs");
     static_assert(N == 1 || N == 2, "one or two kept values per block");
@@ -93,8 +93,8 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);    // wavefront-uniform: bases stay in scalar registers
     const int i = lane & 15, kq = lane >> 4;
     // Workgroup ids go to the 8 XCDs in turn; consecutive spans of a slice read neighbouring parts
-    // of the same 128-byte lines (a quarter wavefront takes 128 bytes of values and 32 of patterns
-    // per line), so every XCD gets a contiguous run of (slice, span) pairs, span fastest.
+    // of the same 128-byte lines (a quarter wavefront takes 256 bytes of values and 64 of patterns
+    // per line at 2:4), so every XCD gets a contiguous run of (slice, span) pairs, span fastest.
     int id = blockIdx.x;
     if ((gridDim.x & 7) == 0) id = (id & 7) * (gridDim.x >> 3) + (id >> 3);
     const int span = id % P.spans, slice = id / P.spans;
@@ -110,7 +110,8 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
     // Addresses: a base per wavefront and line u (scalar registers) plus one 32-bit offset per
     // lane and tile.  Nothing in the loads is conditional: a lane beyond the last block reads block 0
     // and its sums are never stored, a group of 8 lines beyond the wavefront's range reads the
-    // range's first group and meets activations masked to zero.
+    // range's first group and meets activations masked to zero, a tile beyond it reads the first
+    // bytes of the bases and is not multiplied.
     const uint32_t nlines = l1 > l0 ? (uint32_t)(l1 - l0) : 0u;
     // (a wavefront whose range is empty stands on the first lines of the slice, which exist)
     const int64_t lb = nlines ? l0 : (int64_t)slice * P.slice_lines;

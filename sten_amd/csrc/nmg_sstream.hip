@@ -21,14 +21,15 @@
 //  * Expansion: a table in LDS gives per pattern the four byte selectors (V_PERM_B32) that spread
 //    the block's value words over the four words of the fragment: one LDS read and four vector
 //    instructions per block.
-//  * A workgroup is 32 output lines (two row blocks that share the activation fragments) and 8
-//    wavefronts that split the reduction; their sums meet in LDS, fixed order, one kernel.
+//  * A workgroup is 32 output lines (two row blocks that share the activation fragments) -- 16 where
+//    the weight has too few lines to give every CU a workgroup -- and 8 wavefronts that split the
+//    reduction; their sums meet in LDS, fixed order, one kernel.
 //  * Loads are instruction statements with counted waits, up to four sets in flight per
 //    wavefront (the counter of outstanding loads holds 63): what bounds the kernel is the bytes
-//    it has in flight.  A wavefront requests its whole range before anything else happens
-//    (reductions up to 8192 at 1:8 and 2:8, 6144 at 4:8; longer ones are refused); every wavefront
-//    issues the same operations -- beyond its range every lane reads the first bytes of the
-//    operand, and those sets are never multiplied.
+//    it has in flight.  A wavefront requests a whole round of sets before anything else happens
+//    (reductions up to 8192 are one round; 4096 at 4:8 with 32 lines) and the next round when the
+//    one before has been multiplied; every wavefront issues the same operations -- beyond its
+//    range every lane reads the first bytes of the operand, and those sets are never multiplied.
 #include "nmg_common.h"
 #include "nmg_tile.h"
 
