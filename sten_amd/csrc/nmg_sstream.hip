@@ -22,14 +22,13 @@
 //    the block's value words over the four words of the fragment: one LDS read and four vector
 //    instructions per block.
 //  * A workgroup is 32 output lines (two row blocks that share the activation fragments) -- 16 where
-//    the weight has too few lines to give every CU a workgroup -- and 8 wavefronts that split the
-//    reduction; their sums meet in LDS, fixed order, one kernel.
-//  * Loads are instruction statements with counted waits, up to four sets in flight per
-//    wavefront (the counter of outstanding loads holds 63): what bounds the kernel is the bytes
-//    it has in flight.  A wavefront requests a whole round of sets before anything else happens
-//    (reductions up to 8192 are one round; 4096 at 4:8 with 32 lines) and the next round when the
-//    one before has been multiplied; every wavefront issues the same operations -- beyond its
-//    range every lane reads the first bytes of the operand, and those sets are never multiplied.
+//    the weight has too few lines to give every CU a workgroup -- and 16 wavefronts that split
+//    the reduction; their sums meet in LDS, fixed order, one kernel.
+//  * Loads are instruction statements with a wait of their own (left to the compiler, the loads
+//    of a set would be waited for one by one as they are used).  A wavefront has one set in flight;
+//    the 16 wavefronts of a workgroup keep the memory busy.  A wavefront without sets requests a
+//    stand-in (every lane reads the first bytes of the operand) so that all run the same code up
+//    to the first wait.
 #include "nmg_common.h"
 #include "nmg_tile.h"
 
@@ -64,7 +63,7 @@ struct SStream {
     uint32_t order[70];            // [c][n] kept positions per pattern, one byte each (c * n <= 280)
 };
 
-constexpr int SS_WAVES = 8;
+constexpr int SS_WAVES = 16;
 constexpr int SS_LINES = 32;            // output lines per workgroup
 constexpr uint32_t SS_NONE = 0xffffff00u;
 
@@ -75,7 +74,6 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
 {
     static_assert(RBN == 1 || RBN == 2, "one or two row blocks of 16 lines");
     static_assert(N == 1 || N == 2 || N == 4, "1:8, 2:8, 4:8");
-    constexpr int NS = (N == 4 && RBN == 2) ? 2 : 4;   // register sets: what fits beside each other (a set of 4:8 takes 69 registers)
     constexpr int PB = 4 * N * 2;            // bytes of values a lane reads per half set: 8, 16, 32
     constexpr int VL = PB / 16 > 0 ? PB / 16 : 1;   // loads they take
     constexpr int NPAR = N == 1 ? 2 : 1;
@@ -115,9 +113,7 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
         uint32_t pats[RBN][2];
         u32x4 xf[2][4];         // [half set][block of the lane]
         uint32_t xmask;
-    } rs[NS];
-    constexpr int OPS = 2 * RBN * (VL + 1) + 8;
-    static_assert((NS - 1) * OPS < 64, "vmcnt is a 6-bit counter");
+    } rs[1];
 
     // loads of set `rel` of the wavefront's range (SS_NONE: a stand-in beyond the range -- every
     // lane reads the first bytes of the wavefront's base, one cache line)
@@ -159,24 +155,22 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
 #define NMG_SS_P(R, rb) "+v"(R.pats[rb][0]), "+v"(R.pats[rb][1])
 #define NMG_SS_V0(R, rb) "+v"(R.vals[rb][0][0]), "+v"(R.vals[rb][1][0])
 #define NMG_SS_V1(R, rb) "+v"(R.vals[rb][0][VL - 1]), "+v"(R.vals[rb][1][VL - 1])
-    // set k of a round has landed: the NS - 1 - k sets behind it may still be on their way
-    // (every register of the set is named exactly once: a register named twice would be copied)
-    auto landed = [&](Regs &R, auto left_tag) __attribute__((always_inline)) {
-        constexpr int LEFT = decltype(left_tag)::value;
+    // the set has landed (every register of the set is named exactly once: a register named twice
+    // would be copied)
+    auto landed = [&](Regs &R) __attribute__((always_inline)) {
         if constexpr (RBN == 2 && VL == 1)
-            asm volatile("s_waitcnt vmcnt(%16)" : NMG_SS_V0(R, 0), NMG_SS_V0(R, 1), NMG_SS_P(R, 0), NMG_SS_P(R, 1), NMG_SS_X(R) : "n"(LEFT * OPS) : "memory");
+            asm volatile("s_waitcnt vmcnt(0)" : NMG_SS_V0(R, 0), NMG_SS_V0(R, 1), NMG_SS_P(R, 0), NMG_SS_P(R, 1), NMG_SS_X(R) : : "memory");
         else if constexpr (RBN == 2)
-            asm volatile("s_waitcnt vmcnt(%20)" : NMG_SS_V0(R, 0), NMG_SS_V0(R, 1), NMG_SS_V1(R, 0), NMG_SS_V1(R, 1), NMG_SS_P(R, 0), NMG_SS_P(R, 1), NMG_SS_X(R) : "n"(LEFT * OPS) : "memory");
+            asm volatile("s_waitcnt vmcnt(0)" : NMG_SS_V0(R, 0), NMG_SS_V0(R, 1), NMG_SS_V1(R, 0), NMG_SS_V1(R, 1), NMG_SS_P(R, 0), NMG_SS_P(R, 1), NMG_SS_X(R) : : "memory");
         else if constexpr (VL == 1)
-            asm volatile("s_waitcnt vmcnt(%12)" : NMG_SS_V0(R, 0), NMG_SS_P(R, 0), NMG_SS_X(R) : "n"(LEFT * OPS) : "memory");
+            asm volatile("s_waitcnt vmcnt(0)" : NMG_SS_V0(R, 0), NMG_SS_P(R, 0), NMG_SS_X(R) : : "memory");
         else
-            asm volatile("s_waitcnt vmcnt(%14)" : NMG_SS_V0(R, 0), NMG_SS_V1(R, 0), NMG_SS_P(R, 0), NMG_SS_X(R) : "n"(LEFT * OPS) : "memory");
+            asm volatile("s_waitcnt vmcnt(0)" : NMG_SS_V0(R, 0), NMG_SS_V1(R, 0), NMG_SS_P(R, 0), NMG_SS_X(R) : : "memory");
     };
 
-    // The wavefront's whole range is requested before anything else happens.  Every wavefront
-    // issues the same operations: a set beyond the range is a stand-in, never multiplied.
-#pragma unroll
-    for (int k = 0; k < NS; k++) issue_set(rs[k], (uint32_t)k < nsets ? (uint32_t)k : SS_NONE);
+    // The first set is requested before anything else happens (a wavefront without sets requests a
+    // stand-in, so that the code up to the first wait is the same for all).
+    issue_set(rs[0], nsets ? 0u : SS_NONE);
 
     // selector table: entry (par, p) = four selector words; word w builds positions 2 w, 2 w + 1 of
     // the block from its value words (bytes 0 .. 7 of the pair {high, low}; 0x0c: zero).  The order
@@ -238,32 +232,25 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
             }
     };
 
-    // A round: NS sets were requested together, set k waits for the NS - 1 - k sets behind it at
-    // most, and the last wait leaves nothing in flight.  Reductions up to 8192 (4096 at 4:8) are one
-    // round, requested above; a longer one goes on in rounds of the same shape, each requested when
-    // the one before has been multiplied (no register set then carries a load across the loop's
-    // back edge; the price is a pause of the loads between two rounds).
-    auto use = [&](Regs &R, uint32_t base, auto k_tag) __attribute__((always_inline)) {
-        constexpr int K = decltype(k_tag)::value;
-        landed(R, std::integral_constant<int, NS - 1 - K>{});
+    // One set in flight per wavefront: request, wait for it, multiply.  Few bytes in flight on
+    // purpose.  With a wavefront's whole range requested at once (four sets) the memory system
+    // serves the chip's requests in no particular order while a wavefront's loads complete in issue
+    // order, so every set lands near the end of the stream and every multiplication is exposed
+    // (measured on 8192 x 8192 at 2:8, one token: each of the four sets cost 0.6 us on top of a
+    // 9.8 us stream, 12.2 us; two sets in flight 11.2; one 10.6, with 16 wavefronts 10.4).  What
+    // keeps the memory busy is the other wavefronts: four per SIMD.  Nothing is in flight across
+    // the loop's back edge and no stand-in is requested behind the last set.
+    landed(rs[0]);      // (the first set, requested above -- or the stand-in of a wavefront without sets)
+    __builtin_amdgcn_sched_barrier(0);
+    if (nsets > 0) multiply_set(rs[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    for (uint32_t s1 = 1; s1 < nsets; s1++) {
+        issue_set(rs[0], s1);
         __builtin_amdgcn_sched_barrier(0);
-        if (base + K < nsets) multiply_set(R);
+        landed(rs[0]);
         __builtin_amdgcn_sched_barrier(0);
-    };
-    auto use_round = [&](uint32_t base) __attribute__((always_inline)) {
-        use(rs[0], base, std::integral_constant<int, 0>{});
-        use(rs[1], base, std::integral_constant<int, 1>{});
-        if constexpr (NS == 4) {
-            use(rs[2], base, std::integral_constant<int, 2>{});
-            use(rs[3], base, std::integral_constant<int, 3>{});
-        }
-    };
-    use_round(0);
-    for (uint32_t base = NS; base < nsets; base += NS) {
-#pragma unroll
-        for (int k = 0; k < NS; k++) issue_set(rs[k], base + k < nsets ? base + k : SS_NONE);
+        multiply_set(rs[0]);
         __builtin_amdgcn_sched_barrier(0);
-        use_round(base);
     }
 #undef NMG_SS_X
 #undef NMG_SS_P
@@ -405,8 +392,8 @@ extern "C" int nmg_spmm_sstream(const void *d_lp_val, const void *d_lp_pat, int6
     NMG_REQUIRE(groups <= 0x3fffffffLL, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
     hipStream_t s = (hipStream_t)stream;
     // 32 lines per workgroup where that gives the chip enough workgroups, else 16 (the token rows are
-    // then read by twice the workgroups: up to 8 tokens)
-    const bool halves = groups < 192 && T <= 8;
+    // then read by twice the workgroups)
+    const bool halves = groups < 192;
     const dim3 grid((unsigned)(halves ? 2 * groups : groups)), block(SS_WAVES * 64);
 #define NMG_SS_N(TT, RB)                                                                     \
     switch (n) {                                                                               \

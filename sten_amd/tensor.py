@@ -552,9 +552,9 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
             and x.dtype in (torch.float16, torch.bfloat16)
             and native.load().nmg_spmm_sstream_supported(lay.n, lay.m)
             and K % 256 == 0
-            # weights of fewer than 6144 lines with more than 8 tokens: the operand of the sparse matrix
-            # cores streams faster although it is larger (4:8 has none)
-            and (kname == "sstream" or lay.n == 4 or O >= 192 * 32 or T <= 8)
+            # weights of fewer than 3072 lines with more than 8 tokens: the operand of the sparse matrix
+            # cores streams as fast or faster although it is larger (4:8 has none)
+            and (kname == "sstream" or lay.n == 4 or O >= 96 * 32 or T <= 8)
             and (T == 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0
             and T * max(x.stride(0), K) * 2 < 2 ** 31 and 32 * (K // 8) * lay.n * 2 < 2 ** 31):
         lp_val, lp_pat = weight.lanepack8()

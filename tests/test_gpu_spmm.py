@@ -583,7 +583,7 @@ def test_few_tokens_on_blocks_of_eight_stream_the_compressed_lines(dtype, M, K, 
     assert rel_l2(to_np(y), ref) <= TOL[dtype]
     yb = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1, kernel="sstream")
     assert rel_l2(to_np(yb), ref + to_np(b).astype(np.float64)) <= TOL[dtype]
-    # the automatic choice: this route for 4:8, from 6144 lines on and up to 8 tokens, else the sparse matrix cores
+    # the automatic choice: this route for 4:8, from 3072 lines on and up to 8 tokens, else the sparse matrix cores
     ya = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)
     assert rel_l2(to_np(ya), ref + to_np(b).astype(np.float64)) <= TOL[dtype]
     xs = torch.zeros((2 * T, K + 8), dtype=dtype, device=DEV)[::2, :K]
