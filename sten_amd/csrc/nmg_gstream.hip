@@ -19,10 +19,9 @@
 //    which one V_PERM_B32 builds the pair (weight of line u, weight of line u + 1) at position r
 //    from the two lines' value words (0x0c: a zero byte): one vector instruction per pair of dense
 //    weights, one 16-byte table read per four positions of a pair of lines.
-//  * A workgroup is 8 wavefronts on one span of 256 outputs and one slice of the reduction; every
-//    wavefront requests its whole range (up to three tiles of 32 lines) before anything else
-//    happens -- what bounds the kernel is the bytes it has in flight -- and multiplies the tiles
-//    as they land.  The wavefronts add their sums in LDS in a fixed order (results do not depend
+//  * A workgroup is 8 wavefronts on one span of 256 outputs and one slice of the reduction; a
+//    wavefront walks its lines in tiles of 32, one tile in flight (the other wavefronts keep the
+//    memory busy).  The wavefronts add their sums in LDS in a fixed order (results do not depend
 //    on timing) and write single-precision partial sums part[slice][token][output];
 //    splitk_sum_kernel adds the slices in order, adds the bias and rounds once.
 #include "nmg_common.h"
@@ -66,13 +65,11 @@ __host__ __device__ constexpr int gs_table_bytes(int npar, int c, int m)
     return (npar * c * c * m * 4 + npar * c * m * 2 + 15) & ~15;
 }
 
-// OPL outputs per lane (a workgroup spans 16 * OPL outputs), NW wavefronts per workgroup, NS
-// register sets per wavefront (tiles in flight).
-template <typename T, int N, int M, int OPL, int NW, int NS>
+// OPL outputs per lane (a workgroup spans 16 * OPL outputs), NW wavefronts per workgroup.
+template <typename T, int N, int M, int OPL, int NW>
 __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
 {
     constexpr int TB = 1, GS_WAVES = NW, GS_OPL = OPL, GS_SPAN = 16 * OPL;
-    static_assert(NS == 2 || NS == 3, "two or three tiles per wavefront");
     static_assert((NW & (NW - 1)) == 0 && NW >= 2, "a power of two of wavefronts");
     static_assert(M == 4 || M == 8, "blocks of 4 or 8 outputs");
     static_assert(N == 1 || N == 2, "one or two kept values per block");
@@ -134,15 +131,11 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
 #pragma unroll
         for (int tb = 0; tb < TB; tb++) acc[q][tb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // NS register sets, one per tile of 32 lines: a wavefront has few tiles (three for 4096 x 11008)
-    // and the kernel lives on the bytes it has in flight, so every wavefront requests its whole
-    // range before anything else happens and multiplies the tiles as they land.  The loads are
-    // instruction statements with a counted wait of their own -- left to the compiler, every wait
-    // is for *all* loads in flight.  A wavefront issues exactly OPS loads per tile and they
-    // complete in issue order, so `vmcnt(j OPS)` means "all but the last j tiles have landed";
-    // every register of the set passes through the wait, so the compiler orders its uses behind it
-    // (that nothing touches them earlier is checked on the compiled code,
-    // `python -m sten_amd.isa_check`).
+    // One register set: a tile of 32 lines in flight per wavefront.  The loads are instruction
+    // statements with a wait of their own -- left to the compiler, the 17 loads of a tile are
+    // waited for one by one as they are used; every register of the set passes through the wait,
+    // so the compiler orders its uses behind it (that nothing touches them earlier is checked on
+    // the compiled code, `python -m sten_amd.isa_check`).
     typedef uint32_t gs_u32x2 __attribute__((ext_vector_type(2)));
     using VT = std::conditional_t<VB == 16, u32x4, std::conditional_t<VB == 8, gs_u32x2, uint32_t>>;
     struct Regs {
@@ -150,9 +143,7 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
         uint32_t pats[8];
         u32x4 xf[TB];
         uint32_t xmask[TB];     // all ones where the lane's token and lines exist, else zero
-    } rs[NS];
-    constexpr int OPS = 16 + TB;
-    static_assert((NS - 1) * OPS < 64, "vmcnt is a 6-bit counter");
+    } rs[1];
     static_assert(TB == 1, "the wait lists one activation fragment");
 
     // (`s_nop 4` in front of every load: the bases are scalar registers, and where the compiler
@@ -194,14 +185,14 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
             R.xmask[tb] = in_range ? x_live[tb] : 0u;
         }
     };
-    // tile k has landed: the NS - 1 - k tiles requested behind it may still be on their way
-    auto landed = [&](Regs &R, auto left_tag) __attribute__((always_inline)) {
-        constexpr int LEFT = decltype(left_tag)::value;
-        asm volatile("s_waitcnt vmcnt(%17)"
+    // the tile has landed (every register of the set passes through the wait, so the compiler
+    // orders its uses behind it)
+    auto landed = [&](Regs &R) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(0)"
                      : "+v"(R.vals[0]), "+v"(R.vals[1]), "+v"(R.vals[2]), "+v"(R.vals[3]), "+v"(R.vals[4]), "+v"(R.vals[5]),
                        "+v"(R.vals[6]), "+v"(R.vals[7]), "+v"(R.pats[0]), "+v"(R.pats[1]), "+v"(R.pats[2]), "+v"(R.pats[3]),
                        "+v"(R.pats[4]), "+v"(R.pats[5]), "+v"(R.pats[6]), "+v"(R.pats[7]), "+v"(R.xf[0])
-                     : "n"(LEFT * OPS)
+                     :
                      : "memory");
     };
     auto word = [](const VT &v, int w) __attribute__((always_inline)) -> uint32_t {
@@ -209,13 +200,12 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
         else return v;
     };
 
-    // All tiles are requested before anything else happens; the selector table is built
+    // The first tile is requested before anything else happens; the selector table is built
     // while they are on their way, from the order table in the kernel arguments (scalar loads: no
     // vector-memory operation of the compiler's own sits between the counted ones).  Entry
     // (par, p, r) = byte selectors that fetch the value kept at position r into the low half of a
     // word (from a value word that is the *low* source of V_PERM_B32).
-#pragma unroll
-    for (int k = 0; k < NS; k++) issue_tile(rs[k], (uint32_t)k < ntiles ? 32u * k : GS_NONE);
+    issue_tile(rs[0], ntiles ? 0u : GS_NONE);
     // code(par, p, r): where the value kept at position r of pattern p lies in its value word
     for (int e = tid; e < NPAR * P.c * M; e += GS_WAVES * 64) {
         const int my_p = (e / M) % P.c, my_r = e % M, my_par = e / (P.c * M);
@@ -276,19 +266,23 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
         }
     };
 
-    // One round: the host cuts the reduction so that a wavefront's range fits its register sets
-    // (32 NS lines), everything was requested above, and tile k waits for the NS - 1 - k tiles
-    // behind it at most.  The last wait leaves nothing in flight.
-    auto use = [&](Regs &R, auto k_tag) __attribute__((always_inline)) {
-        constexpr int K = decltype(k_tag)::value;
-        landed(R, std::integral_constant<int, NS - 1 - K>{});
+    // One tile in flight per wavefront: request, wait for it, multiply; the other wavefronts keep
+    // the memory busy.  (A wavefront's whole range requested at once was no faster at one token and
+    // slower at 16: the chip's requests are then served in no particular order while a wavefront's
+    // loads complete in issue order, so every tile lands near the end of the stream.)  Nothing is
+    // in flight across the loop's back edge, and no stand-in is requested behind the last tile.
+    landed(rs[0]);      // (the first tile, or the stand-in of an empty range)
+    __builtin_amdgcn_sched_barrier(0);
+    if (ntiles > 0) multiply_tile(rs[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    for (uint32_t t1 = 1; t1 < ntiles; t1++) {
+        issue_tile(rs[0], 32 * t1);
         __builtin_amdgcn_sched_barrier(0);
-        if ((uint32_t)K < ntiles) multiply_tile(R);
+        landed(rs[0]);
         __builtin_amdgcn_sched_barrier(0);
-    };
-    use(rs[0], std::integral_constant<int, 0>{});
-    use(rs[1], std::integral_constant<int, 1>{});
-    if constexpr (NS == 3) use(rs[2], std::integral_constant<int, 2>{});
+        multiply_tile(rs[0]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
     __syncthreads();
 
     // Sums of the wavefronts: the upper half writes a slab each, the lower half adds theirs to the
@@ -324,11 +318,9 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
     }
 }
 
-// The shape of the launch: outputs per lane, wavefronts per workgroup, tiles in flight per
-// wavefront.  What bounds the kernel is the bytes it has in flight: with 16 outputs per lane a tile
-// is 17 loads of up to 10.6 KiB, and three of them per wavefront (the counter of outstanding
-// loads holds 63) cover the whole range of a wavefront of a 4096 x 11008 weight.
-constexpr int GS_OPL = 16, GS_WAVES = 8, GS_SETS = 3, GS_SPAN = 16 * GS_OPL;
+// The shape of the launch: outputs per lane and wavefronts per workgroup.  With 16 outputs per lane
+// a tile is 17 loads of up to 10.6 KiB, in runs of 256 bytes per line.
+constexpr int GS_OPL = 16, GS_WAVES = 8, GS_SPAN = 16 * GS_OPL;
 
 static int gstream_plan(int64_t G, int64_t S, int m, int *spans, int *slices, int64_t *slice_lines)
 {
@@ -339,8 +331,6 @@ static int gstream_plan(int64_t G, int64_t S, int m, int *spans, int *slices, in
     const int64_t quantum = 8 * GS_WAVES;
     int64_t lines = (G + sl - 1) / sl;
     lines = std::max<int64_t>((lines + quantum - 1) / quantum * quantum, 32 * GS_WAVES);
-    // a wavefront requests its whole range at once: at most as many tiles of 32 lines as it has register sets
-    lines = std::min<int64_t>(lines, 32 * GS_SETS * GS_WAVES);
     sl = (G + lines - 1) / lines;
     *spans = (int)sp;
     *slices = (int)std::max<int64_t>(sl, 1);
@@ -398,7 +388,6 @@ extern "C" int nmg_spmm_gstream(const void *d_pk_val, const void *d_pk_pat, int6
                 "workspace too small: %lld bytes given, %lld needed (nmg_spmm_gstream_plan)", (long long)ws_bytes,
                 (long long)((int64_t)slices * T * P.part_ld * 4));
     NMG_REQUIRE((int64_t)P.spans * slices <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
-    NMG_REQUIRE(P.slice_lines <= 32 * GS_SETS * GS_WAVES, NMG_ERR_UNSUPPORTED, "a slice beyond the register sets of its wavefronts");
     NMG_REQUIRE((P.slice_lines / GS_WAVES + 8) * nb * n * 2 < ((int64_t)1 << 31) && nb * n * 2 < (1 << 24) &&
                     P.slice_lines / GS_WAVES < (1 << 23),
                 NMG_ERR_UNSUPPORTED, "lines of more than 16 MiB, or the lines of one wavefront span more than 2 GiB");
@@ -421,7 +410,7 @@ extern "C" int nmg_spmm_gstream(const void *d_pk_val, const void *d_pk_pat, int6
     NMG_REQUIRE(lds <= 160 * 1024, NMG_ERR_UNSUPPORTED, "LDS");
 #define NMG_GS_TB(TT, NN, MM)                                                                              \
     {                                                                                                        \
-        auto k = gstream_kernel<TT, NN, MM, GS_OPL, GS_WAVES, GS_SETS>;                                                            \
+        auto k = gstream_kernel<TT, NN, MM, GS_OPL, GS_WAVES>;                                                            \
         if (lds > 64 * 1024)                                                                                 \
             NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
         hipLaunchKernelGGL(k, grid, block, lds, s, P);                                                       \

@@ -535,6 +535,7 @@ def test_few_tokens_without_a_sparse_core_operand_take_the_dense_routes(dtype, M
     (torch.float16, 512, 1000, 2, 8, 4),
     (torch.bfloat16, 1040, 2056, 1, 8, 32),    # 130 blocks of 8, ragged chunks of the group dim
     (torch.float16, 4096, 2816, 2, 4, 16),     # sixteen spans, several slices of the reduction
+    (torch.bfloat16, 8192, 9000, 2, 4, 16),    # 32 spans: slices of 1152 lines, up to five tiles of 32 lines per wavefront
 ])
 def test_few_tokens_along_the_group_dim_stream_the_compressed_lines(dtype, M, K, n, m, g, T):
     # F.linear with a weight in the reference's default orientation (n:m blocks along the outputs):
