@@ -46,17 +46,16 @@ template <> struct GsMfma<__hip_bfloat16> {
 };
 
 struct GStream {
-    const unsigned char *pk_val;   // [G][nb][n] 16-bit values
-    const unsigned char *pk_pat;   // [G][nb] pattern numbers, one byte each
+    const unsigned char *gp;       // the operand in tile order ("gpack", see gpack_kernel)
     uint32_t order[14];            // [c][n] kept positions per pattern, one byte each (c * n <= 56 for m <= 8, n <= 2)
     const unsigned char *x;        // [T][ldx] 16-bit activations
     float *part;                   // [slices][T][part_ld]
-    int64_t G, nb, ldx, T, part_ld;
-    int64_t slice_lines;           // lines per slice, a multiple of 8 * GS_WAVES
+    int64_t G, ldx, T, part_ld;
+    int64_t ltiles;                // tiles of 32 lines: ceil(G / 32)
+    int wave_tiles;                // tiles per wavefront (a slice is GS_WAVES * wave_tiles tiles)
     int c, spans;
 };
 
-constexpr uint32_t GS_NONE = 0xffffff00u;   // "no tile": a line offset beyond any range
 constexpr int GS_QS = 24;          // floats between the rows of two outputs q of a token in the LDS sums
 
 // bytes of the selector tables in LDS (pair table, code table), rounded to 16
@@ -73,6 +72,7 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
     static_assert((NW & (NW - 1)) == 0 && NW >= 2, "a power of two of wavefronts");
     static_assert(M == 4 || M == 8, "blocks of 4 or 8 outputs");
     static_assert(N == 1 || N == 2, "one or two kept values per block");
+    static_assert(GS_OPL == 16, "a lane holds 16 outputs: 16, 8 or 4 bytes of values per line");
     constexpr int BL = GS_OPL / M;          // blocks per lane
     constexpr int VB = BL * N * 2;          // bytes of values per lane and line: 16, 8, 4 or 2
     constexpr int NPAR = N == 1 ? 2 : 1;    // n = 1: two blocks share a value word, the selector depends on the parity
@@ -96,27 +96,20 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
     if ((gridDim.x & 7) == 0) id = (id & 7) * (gridDim.x >> 3) + (id >> 3);
     const int span = id % P.spans, slice = id / P.spans;
 
-    const int64_t b_lane = (int64_t)span * (16 * BL) + i * BL;      // first block of the lane
-    const bool lane_ok = b_lane < P.nb;
-    const int64_t val_pitch = P.nb * N * 2, pat_pitch = P.nb;
-
-    const int64_t wave_lines = P.slice_lines / GS_WAVES;            // a multiple of 8
-    const int64_t l0 = (int64_t)slice * P.slice_lines + (int64_t)wave * wave_lines;
-    const int64_t l1 = l0 + wave_lines < P.G ? l0 + wave_lines : P.G;
-
-    // Addresses: a base per wavefront and line u (scalar registers) plus one 32-bit offset per
-    // lane and tile.  Nothing in the loads is conditional: a lane beyond the last block reads block 0
-    // and its sums are never stored, a group of 8 lines beyond the wavefront's range reads the
-    // range's first group and meets activations masked to zero, a tile beyond it reads the first
-    // bytes of the bases and is not multiplied.
-    const uint32_t nlines = l1 > l0 ? (uint32_t)(l1 - l0) : 0u;
-    // (a wavefront whose range is empty stands on the first lines of the slice, which exist)
-    const int64_t lb = nlines ? l0 : (int64_t)slice * P.slice_lines;
-    const unsigned char *vwave = P.pk_val + lb * val_pitch;
-    const unsigned char *pwave = P.pk_pat + lb * pat_pitch;
-    const unsigned char *xwave = P.x + lb * 2;
-    const uint32_t ntiles = (nlines + 31) / 32;
-    const uint32_t bl_lane = lane_ok ? (uint32_t)b_lane : 0u;
+    // The wavefront's tiles of 32 lines: consecutive in the operand (10 KiB each at 2:4), so its
+    // loads walk one contiguous run.  Lines beyond G and blocks beyond the last hold zeros there;
+    // only the activations need masking (G is a multiple of 8: a group of 8 lines is whole or absent).
+    constexpr int PBITS = (M == 4 || N == 1) ? 4 : 8;      // bits of a pattern number (c <= 16: 4)
+    constexpr int PL = 8 * BL * PBITS / 8;                 // bytes of patterns per lane and tile: 16 or 8
+    constexpr uint32_t TBYTES = 512 * VB + 64 * PL;        // bytes of a tile: values [u][lane], patterns [lane]
+    const int64_t tile0 = ((int64_t)slice * GS_WAVES + wave) * P.wave_tiles;
+    const int64_t left = P.ltiles - tile0;
+    const uint32_t ntiles = left <= 0 ? 0u : (left < P.wave_tiles ? (uint32_t)left : (uint32_t)P.wave_tiles);
+    const int64_t tb0 = ntiles ? tile0 : 0;      // (a wavefront without tiles stands on the first, which exists)
+    const int64_t lines_left = P.G - tb0 * 32;
+    const uint32_t nlines = ntiles == 0 ? 0u : (lines_left < (int64_t)ntiles * 32 ? (uint32_t)lines_left : ntiles * 32);
+    const unsigned char *twave = P.gp + ((int64_t)span * P.ltiles + tb0) * TBYTES;
+    const unsigned char *xwave = P.x + tb0 * 32 * 2;
     uint32_t x_tok[TB], x_live[TB];
 #pragma unroll
     for (int tb = 0; tb < TB; tb++) {
@@ -138,9 +131,10 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
     // the compiled code, `python -m sten_amd.isa_check`).
     typedef uint32_t gs_u32x2 __attribute__((ext_vector_type(2)));
     using VT = std::conditional_t<VB == 16, u32x4, std::conditional_t<VB == 8, gs_u32x2, uint32_t>>;
+    using PT = std::conditional_t<PL == 16, u32x4, gs_u32x2>;
     struct Regs {
-        VT vals[8];
-        uint32_t pats[8];
+        VT vals[8];             // line u of the lane's octet
+        PT pats;                // pattern (u, block bl) at bit (u BL + bl) PBITS
         u32x4 xf[TB];
         uint32_t xmask[TB];     // all ones where the lane's token and lines exist, else zero
     } rs[1];
@@ -150,37 +144,29 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
     // parks one in a lane of a vector register it reads it back with a vector instruction right
     // before the use -- a scalar register written by the vector unit needs five wait states before
     // a memory instruction may read it, and the compiler does not look into instruction statements)
-    auto issue_tile = [&](Regs &R, uint32_t rel) __attribute__((always_inline)) {
-        // ranges are multiples of 8 lines: a group of 8 is whole or absent
-        const bool in_range = rel < nlines && rel + 8 * kq < nlines;
-        const uint32_t lrel = in_range ? rel + 8 * kq : 0u;      // lines from the range's first
-        // (24-bit factors, checked by the host: one multiply-add each)
-        // (beyond the whole range every lane reads the first bytes of the base: one cache line)
-        const bool none = rel >= nlines;
-        const uint32_t v_off = none ? 0u : __umul24(lrel, (uint32_t)val_pitch) + bl_lane * (N * 2);
-        const uint32_t p_off = none ? 0u : __umul24(lrel, (uint32_t)pat_pitch) + bl_lane;
+    auto issue_tile = [&](Regs &R, uint32_t t) __attribute__((always_inline)) {
+        // (beyond the range every lane reads the first bytes of the base: one cache line)
+        const bool none = t >= ntiles;
+        const bool in_range = !none && t * 32 + 8 * kq < nlines;
+        const uint32_t v_off = none ? 0u : t * TBYTES + (uint32_t)lane * VB;
+        const uint32_t p_off = none ? 0u : t * TBYTES + 512u * VB + (uint32_t)lane * PL;
 #pragma unroll
         for (int u = 0; u < 8; u++) {
-            const unsigned char *vp = vwave + u * val_pitch;
-            const unsigned char *pp = pwave + u * pat_pitch;
+            const unsigned char *vp = twave + u * (64 * VB);
             if constexpr (VB == 16)
                 asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2" : "=v"(R.vals[u]) : "v"(v_off), "s"(vp) : "memory");
             else if constexpr (VB == 8)
                 asm volatile("s_nop 4\n\tglobal_load_dwordx2 %0, %1, %2" : "=v"(R.vals[u]) : "v"(v_off), "s"(vp) : "memory");
-            else if constexpr (VB == 4)
+            else
                 asm volatile("s_nop 4\n\tglobal_load_dword %0, %1, %2" : "=v"(R.vals[u]) : "v"(v_off), "s"(vp) : "memory");
-            else
-                asm volatile("s_nop 4\n\tglobal_load_ushort %0, %1, %2" : "=v"(R.vals[u]) : "v"(v_off), "s"(vp) : "memory");
-            if constexpr (BL == 4)
-                asm volatile("s_nop 4\n\tglobal_load_dword %0, %1, %2" : "=v"(R.pats[u]) : "v"(p_off), "s"(pp) : "memory");
-            else if constexpr (BL == 2)
-                asm volatile("s_nop 4\n\tglobal_load_ushort %0, %1, %2" : "=v"(R.pats[u]) : "v"(p_off), "s"(pp) : "memory");
-            else
-                asm volatile("s_nop 4\n\tglobal_load_ubyte %0, %1, %2" : "=v"(R.pats[u]) : "v"(p_off), "s"(pp) : "memory");
         }
+        if constexpr (PL == 16)
+            asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2" : "=v"(R.pats) : "v"(p_off), "s"(twave) : "memory");
+        else
+            asm volatile("s_nop 4\n\tglobal_load_dwordx2 %0, %1, %2" : "=v"(R.pats) : "v"(p_off), "s"(twave) : "memory");
 #pragma unroll
         for (int tb = 0; tb < TB; tb++) {
-            const uint32_t xo = none ? 0u : x_tok[tb] + lrel * 2;
+            const uint32_t xo = in_range ? x_tok[tb] + (t * 32 + 8 * kq) * 2 : 0u;
             asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2" : "=v"(R.xf[tb]) : "v"(xo), "s"(xwave) : "memory");
             R.xmask[tb] = in_range ? x_live[tb] : 0u;
         }
@@ -190,10 +176,14 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
     auto landed = [&](Regs &R) __attribute__((always_inline)) {
         asm volatile("s_waitcnt vmcnt(0)"
                      : "+v"(R.vals[0]), "+v"(R.vals[1]), "+v"(R.vals[2]), "+v"(R.vals[3]), "+v"(R.vals[4]), "+v"(R.vals[5]),
-                       "+v"(R.vals[6]), "+v"(R.vals[7]), "+v"(R.pats[0]), "+v"(R.pats[1]), "+v"(R.pats[2]), "+v"(R.pats[3]),
-                       "+v"(R.pats[4]), "+v"(R.pats[5]), "+v"(R.pats[6]), "+v"(R.pats[7]), "+v"(R.xf[0])
+                       "+v"(R.vals[6]), "+v"(R.vals[7]), "+v"(R.pats), "+v"(R.xf[0])
                      :
                      : "memory");
+    };
+    // pattern of line u, block bl
+    auto pat_of = [](const PT &v, int u, int bl) __attribute__((always_inline)) -> uint32_t {
+        const int bit = (u * BL + bl) * PBITS;
+        return (v[bit / 32] >> (bit % 32)) & ((1u << PBITS) - 1);
     };
     auto word = [](const VT &v, int w) __attribute__((always_inline)) -> uint32_t {
         if constexpr (VB >= 8) return v[w];
@@ -205,7 +195,7 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
     // vector-memory operation of the compiler's own sits between the counted ones).  Entry
     // (par, p, r) = byte selectors that fetch the value kept at position r into the low half of a
     // word (from a value word that is the *low* source of V_PERM_B32).
-    issue_tile(rs[0], ntiles ? 0u : GS_NONE);
+    issue_tile(rs[0], 0u);      // (a stand-in where the wavefront has no tile)
     // code(par, p, r): where the value kept at position r of pattern p lies in its value word
     for (int e = tid; e < NPAR * P.c * M; e += GS_WAVES * 64) {
         const int my_p = (e / M) % P.c, my_r = e % M, my_par = e / (P.c * M);
@@ -240,7 +230,7 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
             uint32_t sel[4][M];
 #pragma unroll
             for (int up = 0; up < 4; up++) {
-                const uint32_t p0 = (R.pats[2 * up] >> (8 * bl)) & 0xffu, p1 = (R.pats[2 * up + 1] >> (8 * bl)) & 0xffu;
+                const uint32_t p0 = pat_of(R.pats, 2 * up, bl), p1 = pat_of(R.pats, 2 * up + 1, bl);
                 const unsigned char *e = (const unsigned char *)pair + (N == 1 ? (bl & 1) * P.c * cM4 : 0u) +
                                          __umul24(p0, cM4) + p1 * (M * 4);
 #pragma unroll
@@ -276,7 +266,7 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
     if (ntiles > 0) multiply_tile(rs[0]);
     __builtin_amdgcn_sched_barrier(0);
     for (uint32_t t1 = 1; t1 < ntiles; t1++) {
-        issue_tile(rs[0], 32 * t1);
+        issue_tile(rs[0], t1);
         __builtin_amdgcn_sched_barrier(0);
         landed(rs[0]);
         __builtin_amdgcn_sched_barrier(0);
@@ -319,23 +309,80 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
 }
 
 // The shape of the launch: outputs per lane and wavefronts per workgroup.  With 16 outputs per lane
-// a tile is 17 loads of up to 10.6 KiB, in runs of 256 bytes per line.
+// a tile of 32 lines x 256 outputs is 10 loads of up to 9 KiB in all.
 constexpr int GS_OPL = 16, GS_WAVES = 8, GS_SPAN = 16 * GS_OPL;
 
-static int gstream_plan(int64_t G, int64_t S, int m, int *spans, int *slices, int64_t *slice_lines)
+// bytes of a tile of the operand and bits of a pattern number (as the kernel has them)
+static void gpack_shape(int n, int m, int *vb, int *pbits, int *pl, int64_t *tbytes)
 {
-    const int64_t nb = (S + m - 1) / m;
-    const int64_t sp = (nb * m + GS_SPAN - 1) / GS_SPAN;
-    // one workgroup per CU when the weight allows it; a wavefront gets at least 32 lines
-    int64_t sl = std::max<int64_t>(1, 256 / sp);
-    const int64_t quantum = 8 * GS_WAVES;
-    int64_t lines = (G + sl - 1) / sl;
-    lines = std::max<int64_t>((lines + quantum - 1) / quantum * quantum, 32 * GS_WAVES);
-    sl = (G + lines - 1) / lines;
+    const int bl = GS_OPL / m;
+    *vb = bl * n * 2;
+    *pbits = (m == 4 || n == 1) ? 4 : 8;
+    *pl = 8 * bl * *pbits / 8;
+    *tbytes = 512 * (int64_t)*vb + 64 * (int64_t)*pl;
+}
+
+// ---- the operand: rowpack in tile order.  Tile (span sp, line tile lt) = 32 lines x 256 outputs:
+//   values   [u 0..7][lane 0..63][VB bytes]   lane (i, kq) = (l % 16, l / 16): line 32 lt + 8 kq + u,
+//                                             blocks 16 BL sp + BL i .. + BL - 1 (BL = 16 / m)
+//   patterns [lane][PL bytes]                 pattern of (u, block bl) at bit (u BL + bl) PBITS
+// tiles ordered [sp][lt], so the tiles a wavefront walks are one contiguous run.  Lines beyond G and
+// blocks beyond the last are zeros with pattern 0.
+struct GPack {
+    const unsigned char *pk_val;   // [G][nb][n] 16-bit values
+    const unsigned char *pk_pat;   // [G][nb] pattern numbers, one byte each
+    unsigned char *gp;
+    int64_t G, nb, ltiles, spans;
+    int n, m;
+};
+
+__global__ __launch_bounds__(256) void gpack_kernel(GPack P)
+{
+    const int bl_n = GS_OPL / P.m, vb = bl_n * P.n * 2;
+    const int pbits = (P.m == 4 || P.n == 1) ? 4 : 8, pl = 8 * bl_n * pbits / 8;
+    const int64_t tbytes = 512 * (int64_t)vb + 64 * (int64_t)pl;
+    const int64_t tile = blockIdx.x;
+    const int64_t sp = tile / P.ltiles, lt = tile - sp * P.ltiles;
+    unsigned char *out = P.gp + tile * tbytes;
+    // values: 512 (u, lane) shares of vb bytes, as 16-bit elements
+    for (int e = threadIdx.x; e < 512 * (vb / 2); e += 256) {
+        const int h = e % (vb / 2), share = e / (vb / 2);
+        const int lane = share & 63, u = share >> 6, i = lane & 15, kq = lane >> 4;
+        const int64_t line = lt * 32 + 8 * kq + u;
+        const int64_t blk0 = sp * (16 * bl_n) + (int64_t)i * bl_n;      // the lane's first block
+        const int64_t blk = blk0 + h / P.n;
+        uint16_t v = 0;
+        if (line < P.G && blk < P.nb) v = ((const uint16_t *)P.pk_val)[(line * P.nb + blk) * P.n + h % P.n];
+        ((uint16_t *)out)[share * (vb / 2) + h] = v;
+    }
+    // patterns: one 32-bit word per thread
+    for (int e = threadIdx.x; e < 64 * (pl / 4); e += 256) {
+        const int w = e % (pl / 4), lane = e / (pl / 4), i = lane & 15, kq = lane >> 4;
+        uint32_t word = 0;
+        for (int f = 0; f < 32 / pbits; f++) {
+            const int idx = (w * 32) / pbits + f;          // = u * bl_n + bl
+            const int u = idx / bl_n, bl = idx - u * bl_n;
+            const int64_t line = lt * 32 + 8 * kq + u;
+            const int64_t blk = sp * (16 * bl_n) + (int64_t)i * bl_n + bl;
+            uint32_t p = 0;
+            if (line < P.G && blk < P.nb) p = P.pk_pat[line * P.nb + blk];
+            word |= p << (f * pbits);
+        }
+        ((uint32_t *)(out + 512 * (int64_t)vb))[lane * (pl / 4) + w] = word;
+    }
+}
+
+// slices of the reduction: one workgroup per CU when the weight allows it; a wavefront walks
+// whole tiles of 32 lines
+static void gstream_plan(int64_t G, int64_t S, int *spans, int *slices, int *wave_tiles)
+{
+    const int64_t sp = (S + GS_SPAN - 1) / GS_SPAN;
+    const int64_t ltiles = (G + 31) / 32;
+    const int64_t want = std::max<int64_t>(1, 256 / sp);                     // slices wanted
+    const int64_t per = (ltiles + want * GS_WAVES - 1) / (want * GS_WAVES);  // tiles per wavefront
+    *wave_tiles = (int)std::max<int64_t>(per, 1);
     *spans = (int)sp;
-    *slices = (int)std::max<int64_t>(sl, 1);
-    *slice_lines = lines;
-    return NMG_OK;
+    *slices = (int)((ltiles + (int64_t)*wave_tiles * GS_WAVES - 1) / ((int64_t)*wave_tiles * GS_WAVES));
 }
 
 }  // namespace nmg
@@ -347,21 +394,59 @@ extern "C" int nmg_spmm_gstream_supported(int n, int m)
     return (m == 4 || m == 8) && (n == 1 || n == 2) ? 1 : 0;
 }
 
+extern "C" int nmg_gpack_bytes(int64_t G, int64_t S, int n, int m, int64_t *bytes)
+{
+    NMG_REQUIRE(bytes, NMG_ERR_ARG, "null output pointer");
+    NMG_REQUIRE(nmg_spmm_gstream_supported(n, m), NMG_ERR_UNSUPPORTED, "the streaming product takes m = 4, 8 and n = 1, 2");
+    NMG_REQUIRE(G >= 0 && S >= 0, NMG_ERR_ARG, "negative extent");
+    int vb, pbits, pl;
+    int64_t tbytes;
+    gpack_shape(n, m, &vb, &pbits, &pl, &tbytes);
+    *bytes = ((S + GS_SPAN - 1) / GS_SPAN) * ((G + 31) / 32) * tbytes;
+    return NMG_OK;
+}
+
+extern "C" int nmg_gpack(const void *d_pk_val, const void *d_pk_pat, int64_t G, int64_t S, int n, int m, void *d_gp,
+                         int dtype, void *stream)
+{
+    NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED, "the operand holds f16/bf16");
+    NMG_REQUIRE(nmg_spmm_gstream_supported(n, m), NMG_ERR_UNSUPPORTED, "the streaming product takes m = 4, 8 and n = 1, 2");
+    NMG_REQUIRE(G >= 0 && S >= 0, NMG_ERR_ARG, "negative extent");
+    if (G == 0 || S == 0) return NMG_OK;
+    NMG_REQUIRE(d_pk_val && d_pk_pat && d_gp, NMG_ERR_ARG, "null device pointer");
+    NMG_REQUIRE(((uintptr_t)d_gp % 16) == 0 && ((uintptr_t)d_pk_val % 2) == 0, NMG_ERR_ARG, "the operand must be 16-byte aligned");
+    NMG_REQUIRE(binom(m, n) <= ((m == 4 || n == 1) ? 16 : 256), NMG_ERR_UNSUPPORTED, "pattern numbers beyond their field");
+    GPack P;
+    P.pk_val = (const unsigned char *)d_pk_val;
+    P.pk_pat = (const unsigned char *)d_pk_pat;
+    P.gp = (unsigned char *)d_gp;
+    P.G = G;
+    P.nb = (S + m - 1) / m;
+    P.ltiles = (G + 31) / 32;
+    P.spans = (S + GS_SPAN - 1) / GS_SPAN;
+    P.n = n;
+    P.m = m;
+    const int64_t tiles = P.ltiles * P.spans;
+    NMG_REQUIRE(tiles <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
+    hipLaunchKernelGGL(gpack_kernel, dim3((unsigned)tiles), dim3(256), 0, (hipStream_t)stream, P);
+    NMG_HIP_TRY(hipGetLastError());
+    return NMG_OK;
+}
+
 extern "C" int nmg_spmm_gstream_plan(int64_t G, int64_t S, int64_t T, int n, int m, int *slices, int64_t *ws_bytes)
 {
     NMG_REQUIRE(slices && ws_bytes, NMG_ERR_ARG, "null output pointer");
     NMG_REQUIRE(nmg_spmm_gstream_supported(n, m), NMG_ERR_UNSUPPORTED, "the streaming product takes m = 4, 8 and n = 1, 2");
     NMG_REQUIRE(G >= 0 && S >= 0 && T >= 0, NMG_ERR_ARG, "negative extent");
-    int spans = 1;
-    int64_t lines = 0;
-    gstream_plan(std::max<int64_t>(G, 1), std::max<int64_t>(S, 1), m, &spans, slices, &lines);
+    int spans = 1, wave_tiles = 1;
+    gstream_plan(std::max<int64_t>(G, 1), std::max<int64_t>(S, 1), &spans, slices, &wave_tiles);
     *ws_bytes = (int64_t)*slices * T * spans * GS_SPAN * 4;
     return NMG_OK;
 }
 
-extern "C" int nmg_spmm_gstream(const void *d_pk_val, const void *d_pk_pat, int64_t G, int64_t S, const void *d_x,
-                                int64_t ldx, void *d_y, int64_t ldy, const void *d_bias, int64_t T, int n, int m,
-                                int dtype, void *d_ws, int64_t ws_bytes, void *stream)
+extern "C" int nmg_spmm_gstream(const void *d_gp, int64_t G, int64_t S, const void *d_x, int64_t ldx, void *d_y,
+                                int64_t ldy, const void *d_bias, int64_t T, int n, int m, int dtype, void *d_ws,
+                                int64_t ws_bytes, void *stream)
 {
     NMG_REQUIRE(dtype == NMG_F16 || dtype == NMG_BF16, NMG_ERR_UNSUPPORTED, "the streaming product takes f16/bf16");
     NMG_REQUIRE(nmg_spmm_gstream_supported(n, m), NMG_ERR_UNSUPPORTED, "the streaming product takes m = 4, 8 and n = 1, 2");
@@ -370,29 +455,27 @@ extern "C" int nmg_spmm_gstream(const void *d_pk_val, const void *d_pk_pat, int6
     NMG_REQUIRE(ldx >= G && ldy >= S, NMG_ERR_ARG, "leading dimension smaller than row length");
     if (T == 0 || S == 0) return NMG_OK;
     NMG_REQUIRE(G > 0, NMG_ERR_UNSUPPORTED, "empty reduction: clear the output instead");
-    const int64_t nb = (S + m - 1) / m;
-    const int BL = GS_OPL / m;
     NMG_REQUIRE(G % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)d_x % 16) == 0, NMG_ERR_UNSUPPORTED,
                 "the streaming product needs a reduction extent and a row pitch of the activations that are multiples "
                 "of 8, and 16-byte aligned activations");
-    NMG_REQUIRE(nb % BL == 0 && ((uintptr_t)d_pk_val % 16) == 0 && ((uintptr_t)d_pk_pat % 4) == 0, NMG_ERR_UNSUPPORTED,
-                "the streaming product needs whole groups of %d blocks per line and aligned operands", BL);
-    NMG_REQUIRE(d_pk_val && d_pk_pat && d_x && d_y && d_ws, NMG_ERR_ARG, "null device pointer");
+    NMG_REQUIRE(d_gp && d_x && d_y && d_ws, NMG_ERR_ARG, "null device pointer");
+    NMG_REQUIRE(((uintptr_t)d_gp % 16) == 0, NMG_ERR_UNSUPPORTED, "the operand must be 16-byte aligned");
     NMG_REQUIRE(T * ldx * 2 < ((int64_t)1 << 31), NMG_ERR_UNSUPPORTED, "activations beyond 2 GiB");
 
     GStream P;
     int slices = 1;
-    gstream_plan(G, S, m, &P.spans, &slices, &P.slice_lines);
+    gstream_plan(G, S, &P.spans, &slices, &P.wave_tiles);
     P.part_ld = (int64_t)P.spans * GS_SPAN;
     NMG_REQUIRE(ws_bytes >= (int64_t)slices * T * P.part_ld * 4, NMG_ERR_ARG,
                 "workspace too small: %lld bytes given, %lld needed (nmg_spmm_gstream_plan)", (long long)ws_bytes,
                 (long long)((int64_t)slices * T * P.part_ld * 4));
     NMG_REQUIRE((int64_t)P.spans * slices <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
-    NMG_REQUIRE((P.slice_lines / GS_WAVES + 8) * nb * n * 2 < ((int64_t)1 << 31) && nb * n * 2 < (1 << 24) &&
-                    P.slice_lines / GS_WAVES < (1 << 23),
-                NMG_ERR_UNSUPPORTED, "lines of more than 16 MiB, or the lines of one wavefront span more than 2 GiB");
-    P.pk_val = (const unsigned char *)d_pk_val;
-    P.pk_pat = (const unsigned char *)d_pk_pat;
+    int vb, pbits, pl;
+    int64_t tbytes;
+    gpack_shape(n, m, &vb, &pbits, &pl, &tbytes);
+    NMG_REQUIRE(((int64_t)P.wave_tiles + 1) * tbytes < ((int64_t)1 << 31), NMG_ERR_UNSUPPORTED,
+                "the tiles of one wavefront span more than 2 GiB");
+    P.gp = (const unsigned char *)d_gp;
     const int8_t *ord = host_order(n, m);
     NMG_REQUIRE(ord != nullptr && binom(m, n) * n <= (int64_t)sizeof(P.order), NMG_ERR_ARG, "invalid n:m = %d:%d", n, m);
     for (int e = 0; e < 14; e++) P.order[e] = 0;
@@ -400,7 +483,7 @@ extern "C" int nmg_spmm_gstream(const void *d_pk_val, const void *d_pk_pat, int6
     P.x = (const unsigned char *)d_x;
     P.part = (float *)d_ws;
     P.G = G;
-    P.nb = nb;
+    P.ltiles = (G + 31) / 32;
     P.ldx = ldx;
     P.T = T;
     P.c = (int)binom(m, n);
@@ -410,7 +493,7 @@ extern "C" int nmg_spmm_gstream(const void *d_pk_val, const void *d_pk_pat, int6
     NMG_REQUIRE(lds <= 160 * 1024, NMG_ERR_UNSUPPORTED, "LDS");
 #define NMG_GS_TB(TT, NN, MM)                                                                              \
     {                                                                                                        \
-        auto k = gstream_kernel<TT, NN, MM, GS_OPL, GS_WAVES>;                                                            \
+        auto k = gstream_kernel<TT, NN, MM, GS_OPL, GS_WAVES>;                                              \
         if (lds > 64 * 1024)                                                                                 \
             NMG_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
         hipLaunchKernelGGL(k, grid, block, lds, s, P);                                                       \

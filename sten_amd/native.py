@@ -78,7 +78,9 @@ SIGNATURES = {
     "nmg_spmm_smfmac_tt": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _P]),
     "nmg_spmm_gstream_supported": (_I, [_I, _I]),
     "nmg_spmm_gstream_plan": (_I, [_I64, _I64, _I64, _I, _I, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int64)]),
-    "nmg_spmm_gstream": (_I, [_P, _P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _I, _P, _I64, _P]),
+    "nmg_gpack_bytes": (_I, [_I64, _I64, _I, _I, ctypes.POINTER(ctypes.c_int64)]),
+    "nmg_gpack": (_I, [_P, _P, _I64, _I64, _I, _I, _P, _I, _P]),
+    "nmg_spmm_gstream": (_I, [_P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _I, _P, _I64, _P]),
     "nmg_spmm_sstream_supported": (_I, [_I, _I]),
     "nmg_lanepack8_sizes": (_I, [_I64, _I64, _I, ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64)]),
     "nmg_lanepack8": (_I, [_P, _P, _I64, _I64, _I, _P, _P, _I, _P]),

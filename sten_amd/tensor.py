@@ -43,6 +43,7 @@ class GroupedNMTensor:
         self._densefrag = None
         self._dense_operand = None
         self._lanepack8 = None
+        self._gpack = None
 
     # ---- construction ----------------------------------------------------------------------
     @staticmethod
@@ -333,6 +334,26 @@ class GroupedNMTensor:
         self._lanepack8 = (self._version_key(), lp_val, lp_pat)
         return lp_val, lp_pat
 
+    def gpack(self):
+        """Operand of the streaming product along the group dim (at most 16 tokens, m = 4 or 8 with
+        n = 1 or 2): the rowpack operand in tiles of 32 lines x 256 outputs, each one contiguous
+        run in the order in which the lanes of ``nmg_spmm_gstream`` take it, pattern numbers in 4
+        bits where there are at most 16; kept until ``val`` changes."""
+        lay = self.layout
+        cached = getattr(self, "_gpack", None)
+        if cached is not None and self._key_current(cached[0]):
+            return cached[1]
+        pk_val, pk_pat = self.rowpack()
+        lib = native.load()
+        nbytes = ctypes.c_int64()
+        native.check(lib.nmg_gpack_bytes(lay.G, lay.S, lay.n, lay.m, ctypes.byref(nbytes)))
+        gp = torch.empty(max(nbytes.value, 16), dtype=torch.uint8, device=self.val.device)
+        with torch.cuda.device(gp.device):
+            native.check(lib.nmg_gpack(native.ptr(pk_val), native.ptr(pk_pat), lay.G, lay.S, lay.n, lay.m,
+                                       native.ptr(gp), native.dtype_code(self.val.dtype), native.stream_ptr(gp.device)))
+        self._gpack = (self._version_key(), gp)
+        return gp
+
     def slotmap(self):
         """int16 [num_blocks, Gpad]: for every line of the (padded) group dim and block of the
         sparse dim, the slot that holds it -- the inverse of ``idx``.  Operand of the masked
@@ -614,20 +635,19 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
     ldx = x.stride(0) if T > 1 else K      # the stride of a dim of extent 1 means nothing
     # Few tokens with the reduction along the group dim (what F.linear does with a weight in the
     # reference's default orientation): the compressed lines are streamed once and expanded in
-    # registers -- 56 MB instead of the 90 MB of the dense-core operand for 4096 x 11008 at 2:4.
+    # registers -- 51 MB instead of the 90 MB of the dense-core operand for 4096 x 11008 at 2:4.
     if (kname in ("auto", "gstream") and reduce_sparse == 0 and T <= GSTREAM_MAX_TOKENS
             and x.dtype in (torch.float16, torch.bfloat16) and len(lay.dense_shape) == 2
             and native.load().nmg_spmm_gstream_supported(lay.n, lay.m)
-            and K % 8 == 0 and ldx % 8 == 0 and x.data_ptr() % 16 == 0 and T * ldx * 2 < 2 ** 31
-            and lay.num_blocks % (16 // lay.m) == 0):
+            and K % 8 == 0 and ldx % 8 == 0 and x.data_ptr() % 16 == 0 and T * ldx * 2 < 2 ** 31):
         lib = native.load()
-        pk_val, pk_pat = weight.rowpack()
+        gp = weight.gpack()
         slices, ws_bytes = ctypes.c_int(1), ctypes.c_int64(0)
         native.check(lib.nmg_spmm_gstream_plan(K, O, T, lay.n, lay.m, ctypes.byref(slices), ctypes.byref(ws_bytes)))
         ws = torch.empty((max(ws_bytes.value, 4) // 4,), dtype=torch.float32, device=x.device)
         with torch.cuda.device(x.device):
             native.check(lib.nmg_spmm_gstream(
-                native.ptr(pk_val), native.ptr(pk_pat), K, O, native.ptr(x), ldx, native.ptr(y), O,
+                native.ptr(gp), K, O, native.ptr(x), ldx, native.ptr(y), O,
                 native.ptr(bias), T, lay.n, lay.m, native.dtype_code(x.dtype), native.ptr(ws), ws.numel() * 4,
                 native.stream_ptr(x.device)))
         return y

@@ -504,7 +504,7 @@ def test_odd_16_bit_shapes_take_the_padded_dense_route(dtype, M, K, T, n, m, g, 
 @pytest.mark.parametrize("T", [1, 3, 16])
 @pytest.mark.parametrize("dtype,M,K,n,m,g,sd", [
     (torch.float16, 512, 1088, 4, 8, 4, 1),       # no sparse-core operand for 4:8 (and no whole sets of 32 blocks for the streaming kernel)
-    (torch.bfloat16, 760, 640, 2, 4, 16, 0),      # the reference's default orientation (reduction along the group dim) with 190 blocks: not whole groups of 4
+    (torch.bfloat16, 760, 640, 3, 4, 16, 0),      # the reference's default orientation (reduction along the group dim) at 3:4, which the streaming kernel does not take
     (torch.float16, 320, 1152, 3, 6, 12, 1),
     (torch.float32, 512, 1024, 2, 4, 16, 1),      # fp32: dense copy + fp32 GEMM
 ])
@@ -532,6 +532,7 @@ def test_few_tokens_without_a_sparse_core_operand_take_the_dense_routes(dtype, M
     (torch.float16, 768, 640, 2, 4, 16),       # three spans of 256 outputs, 640 lines
     (torch.bfloat16, 768, 640, 2, 4, 16),
     (torch.float16, 272, 328, 1, 4, 8),        # 68 blocks: part of a span; 41 groups of 8 lines
+    (torch.bfloat16, 760, 640, 2, 4, 16),      # 190 blocks: the last lane of a span holds two blocks of its four
     (torch.float16, 512, 1000, 2, 8, 4),
     (torch.bfloat16, 1040, 2056, 1, 8, 32),    # 130 blocks of 8, ragged chunks of the group dim
     (torch.float16, 4096, 2816, 2, 4, 16),     # sixteen spans, several slices of the reduction
