@@ -57,6 +57,7 @@ struct GStream {
 };
 
 constexpr int GS_QS = 24;          // floats between the rows of two outputs q of a token in the LDS sums
+constexpr int GS_RPAD = 4;         // floats of padding behind a token row there
 
 // bytes of the selector tables in LDS (pair table, code table), rounded to 16
 __host__ __device__ constexpr int gs_table_bytes(int npar, int c, int m)
@@ -77,7 +78,10 @@ __global__ __launch_bounds__(NW * 64) void gstream_kernel(GStream P)
     constexpr int VB = BL * N * 2;          // bytes of values per lane and line: 16, 8, 4 or 2
     constexpr int NPAR = N == 1 ? 2 : 1;    // n = 1: two blocks share a value word, the selector depends on the parity
     constexpr int MAXC = M == 4 ? 6 : 28;
-    constexpr int RS = GS_OPL * GS_QS;      // floats per token row of the LDS sums
+    // floats per token row of the LDS sums; + 4: the 16 token rows that the lanes of a quarter
+    // wavefront write at once start 16 bytes apart in the banks (a multiple of 64 floats would put
+    // them all into the same ones: 16 tokens then cost 3 us more than one)
+    constexpr int RS = GS_OPL * GS_QS + GS_RPAD;
     using F = typename GsMfma<T>::F;
 
     // LDS: [pair table][code table][sums of the wavefronts, two wavefronts per slab]
@@ -489,7 +493,7 @@ extern "C" int nmg_spmm_gstream(const void *d_gp, int64_t G, int64_t S, const vo
     P.c = (int)binom(m, n);
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid((unsigned)(P.spans * slices)), block(GS_WAVES * 64);
-    const size_t lds = (size_t)gs_table_bytes(n == 1 ? 2 : 1, P.c, m) + (size_t)(GS_WAVES / 2) * T * (GS_OPL * GS_QS) * 4;
+    const size_t lds = (size_t)gs_table_bytes(n == 1 ? 2 : 1, P.c, m) + (size_t)(GS_WAVES / 2) * T * (GS_OPL * GS_QS + GS_RPAD) * 4;
     NMG_REQUIRE(lds <= 160 * 1024, NMG_ERR_UNSUPPORTED, "LDS");
 #define NMG_GS_TB(TT, NN, MM)                                                                              \
     {                                                                                                        \
