@@ -99,3 +99,40 @@ def test_random_tile_boundary_cases():
     rng = random.Random(21)
     for _ in range(25):
         one_case(rng, big=True)
+
+
+def test_random_streamed_few_token_cases():
+    """Random shapes, patterns, token counts, row pitches and biases through the two kernels that
+    stream the compressed operand for at most 16 tokens (blocks of 8 along the reduction; the
+    reduction along the group dim), against the fp64 product of the oracle's dense form."""
+    rng = random.Random(31)
+    for _ in range(40):
+        along_sparse = rng.random() < 0.5
+        dt = rng.choice([torch.float16, torch.bfloat16])
+        T = rng.choice([1, 2, 3, 5, 8, 9, 13, 16])
+        if along_sparse:
+            n, m, g = rng.choice([1, 2, 4]), 8, rng.choice([1, 2, 4, 8, 32])
+            M, K = rng.choice([8, 40, 96, 200, 512, 1000]), 256 * rng.choice([1, 2, 3, 5, 8, 13])
+            sd, kern = 1, "sstream"
+        else:
+            m, n, g = rng.choice([4, 8]), rng.choice([1, 2]), rng.choice([1, 4, 8, 16])
+            M, K = m * rng.choice([1, 3, 17, 64, 65, 190, 520]), 8 * rng.choice([1, 4, 5, 33, 64, 100, 333])
+            sd, kern = 0, "gstream"
+        seed = rng.randint(0, 10 ** 6)
+        print(f"case streamed {kern} {dt} M={M} K={K} {n}:{m}:{g} T={T} seed={seed}", flush=True)
+        gen = torch.Generator().manual_seed(seed)
+        W = (torch.randn((M, K), generator=gen) * 0.5).to(dt)
+        val, idx, lay = oracle_sparsify(W, n, m, sd, g, 1 - sd)
+        Wd64 = O.to_dense(val, idx, lay).astype(np.float64)
+        w = sten.GroupedNMTensor.from_dense(W.to(DEV), n, m, sparse_dim=sd, group_size=g, group_dim=1 - sd)
+        x = torch.randn((T, K), generator=gen).to(dt)
+        b = torch.randn((M,), generator=gen).to(dt) if rng.random() < 0.5 else None
+        xs = x.to(DEV)
+        if rng.random() < 0.4 and T > 1:        # rows further apart than their length
+            xs = torch.zeros((2 * T, K + 8), dtype=dt, device=DEV)[::2, :K]
+            xs.copy_(x.to(DEV))
+        y = sten.spmm(w, xs, None if b is None else b.to(DEV), reduce_dim=1, kernel=kern)
+        ref = to_np(x).astype(np.float64) @ Wd64.T
+        if b is not None:
+            ref = ref + to_np(b).astype(np.float64)
+        assert rel_l2(to_np(y), ref) <= TOL[dt], f"{kern} {M}x{K} {n}:{m}:{g} T={T}"
