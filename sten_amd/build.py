@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libnmg_hip.so")
 SOURCES = ["nmg_runtime.hip", "nmg_sparsify.hip", "nmg_spmm.hip", "nmg_smfmac.hip", "nmg_dense.hip",
-           "nmg_densefrag.hip", "nmg_w4.hip", "nmg_pack.hip", "nmg_sddmm.hip", "nmg_perfect.hip", "nmg_gstream.hip", "nmg_sstream.hip"]
+           "nmg_densefrag.hip", "nmg_w4.hip", "nmg_pack.hip", "nmg_sddmm.hip", "nmg_perfect.hip", "nmg_gstream.hip", "nmg_sstream.hip", "nmg_ostream.hip"]
 # bench.py's measurement aid: a library of its own, outside the product ABI
 PROBE_LIB = os.path.join(HERE, "libnmg_probe.so")
 PROBE_SOURCES = ["nmg_probe.hip"]

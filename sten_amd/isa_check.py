@@ -41,6 +41,7 @@ CHECKED = {
     "nmg_sddmm.hip": ["sddmm16_kernel"],
     "nmg_gstream.hip": ["gstream_kernel"],
     "nmg_sstream.hip": ["sstream_kernel"],
+    "nmg_ostream.hip": ["ostream_kernel"],
 }
 
 REG = re.compile(r"\b([va])(\d+)\b|\b([va])\[(\d+):(\d+)\]")

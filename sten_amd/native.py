@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(_HERE, "libnmg_hip.so")
 NMG_F32, NMG_F16, NMG_BF16, NMG_F64 = 0, 1, 2, 3
 KERNEL_AUTO, KERNEL_MFMA, KERNEL_SMFMAC, KERNEL_SKINNY = 0, 1, 2, 3
 KERNELS = {"auto": KERNEL_AUTO, "mfma": KERNEL_MFMA, "smfmac": KERNEL_SMFMAC, "skinny": KERNEL_SKINNY,
-           "expand": KERNEL_MFMA, "densefrag": KERNEL_MFMA, "gstream": KERNEL_SKINNY, "sstream": KERNEL_SKINNY}
+           "expand": KERNEL_MFMA, "densefrag": KERNEL_MFMA, "gstream": KERNEL_SKINNY, "sstream": KERNEL_SKINNY, "ostream": KERNEL_SKINNY}
 
 DTYPE_CODE = {
     torch.float32: NMG_F32,
@@ -81,6 +81,10 @@ SIGNATURES = {
     "nmg_gpack_bytes": (_I, [_I64, _I64, _I, _I, ctypes.POINTER(ctypes.c_int64)]),
     "nmg_gpack": (_I, [_P, _P, _I64, _I64, _I, _I, _P, _I, _P]),
     "nmg_spmm_gstream": (_I, [_P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _I, _P, _I64, _P]),
+    "nmg_spmm_ostream_supported": (_I, [_I, _I]),
+    "nmg_opack_bytes": (_I, [_I64, _I64, _I, _I, ctypes.POINTER(ctypes.c_int64)]),
+    "nmg_opack": (_I, [_P, _P, _I64, _I64, _I, _I, _P, _I, _P]),
+    "nmg_spmm_ostream": (_I, [_P, _I64, _I64, _P, _I64, _P, _I64, _P, _I64, _I, _I, _I, _P]),
     "nmg_spmm_sstream_supported": (_I, [_I, _I]),
     "nmg_lanepack8_sizes": (_I, [_I64, _I64, _I, ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64)]),
     "nmg_lanepack8": (_I, [_P, _P, _I64, _I64, _I, _P, _P, _I, _P]),

@@ -44,6 +44,7 @@ class GroupedNMTensor:
         self._dense_operand = None
         self._lanepack8 = None
         self._gpack = None
+        self._opack = None
 
     # ---- construction ----------------------------------------------------------------------
     @staticmethod
@@ -354,6 +355,25 @@ class GroupedNMTensor:
         self._gpack = (self._version_key(), gp)
         return gp
 
+    def opack(self):
+        """Operand of ``nmg_spmm_ostream`` (a handful of tokens, 2:4, reduction along the group dim):
+        the rowpack operand per span of 16 outputs and set of 256 lines in the order in which the
+        lanes fetch it, pattern numbers in 4 bits; kept until ``val`` changes."""
+        lay = self.layout
+        cached = getattr(self, "_opack", None)
+        if cached is not None and self._key_current(cached[0]):
+            return cached[1]
+        pk_val, pk_pat = self.rowpack()
+        lib = native.load()
+        nbytes = ctypes.c_int64()
+        native.check(lib.nmg_opack_bytes(lay.G, lay.S, lay.n, lay.m, ctypes.byref(nbytes)))
+        op = torch.empty(max(nbytes.value, 16), dtype=torch.uint8, device=self.val.device)
+        with torch.cuda.device(op.device):
+            native.check(lib.nmg_opack(native.ptr(pk_val), native.ptr(pk_pat), lay.G, lay.S, lay.n, lay.m,
+                                       native.ptr(op), native.dtype_code(self.val.dtype), native.stream_ptr(op.device)))
+        self._opack = (self._version_key(), op)
+        return op
+
     def slotmap(self):
         """int16 [num_blocks, Gpad]: for every line of the (padded) group dim and block of the
         sparse dim, the slot that holds it -- the inverse of ``idx``.  Operand of the masked
@@ -440,6 +460,8 @@ class GroupedNMTensor:
                 f"device={self.val.device})")
 
 
+OSTREAM_MAX_TOKENS = 4                # nmg_spmm_ostream: the token rows its lanes hold
+OSTREAM_AUTO_TOKENS = 2               # ... and up to where it is ahead of the sliced kernel (4096 x 11008: 12.4 / 13.3 / 16.2 against 15.9 / 16.0 / 16.3 us at 1 / 2 / 3 tokens)
 GSTREAM_MAX_TOKENS = 16               # nmg_spmm_gstream: tokens up to which the stream of the weight bounds the product
 F32_GEMM_MAX_TOKENS = 65535 * 32      # one launch of the fp32 GEMM: token tiles of 32 in grid.y
 
@@ -636,6 +658,22 @@ def spmm(weight, x, bias=None, *, reduce_dim, kernel=None):
     # Few tokens with the reduction along the group dim (what F.linear does with a weight in the
     # reference's default orientation): the compressed lines are streamed once and expanded in
     # registers -- 51 MB instead of the 90 MB of the dense-core operand for 4096 x 11008 at 2:4.
+    # ... and with a handful of tokens at 2:4 every workgroup owns 16 outputs over the whole
+    # reduction: one kernel, no sums through memory (the token rows are then read by every
+    # workgroup, which is why this is for few of them)
+    if (kname in ("auto", "ostream") and reduce_sparse == 0 and T <= (OSTREAM_AUTO_TOKENS if kname == "auto" else OSTREAM_MAX_TOKENS)
+            and x.dtype in (torch.float16, torch.bfloat16) and len(lay.dense_shape) == 2
+            and native.load().nmg_spmm_ostream_supported(lay.n, lay.m)
+            and K % 8 == 0 and ldx % 8 == 0 and x.data_ptr() % 16 == 0 and T * ldx * 2 < 2 ** 31):
+        op = weight.opack()
+        with torch.cuda.device(x.device):
+            native.check(native.load().nmg_spmm_ostream(
+                native.ptr(op), K, O, native.ptr(x), ldx, native.ptr(y), O, native.ptr(bias), T, lay.n, lay.m,
+                native.dtype_code(x.dtype), native.stream_ptr(x.device)))
+        return y
+    if kname == "ostream":
+        raise native.NmgError("the product with 16 outputs per workgroup needs 16-bit data, 2:4, the reduction along "
+                              f"the group dim, at most {OSTREAM_MAX_TOKENS} tokens and a reduction extent that is a multiple of 8")
     if (kname in ("auto", "gstream") and reduce_sparse == 0 and T <= GSTREAM_MAX_TOKENS
             and x.dtype in (torch.float16, torch.bfloat16) and len(lay.dense_shape) == 2
             and native.load().nmg_spmm_gstream_supported(lay.n, lay.m)

@@ -597,6 +597,39 @@ def test_few_tokens_on_blocks_of_eight_stream_the_compressed_lines(dtype, M, K, 
         assert rel_l2(to_np(y2), to_np(y).astype(np.float64)) <= 2 * TOL[dtype]
 
 
+@pytest.mark.parametrize("T", [1, 2, 3, 4])
+@pytest.mark.parametrize("dtype,M,K", [
+    (torch.float16, 768, 640),        # 48 spans of 16 outputs, three sets of 256 lines: most wavefronts have none
+    (torch.bfloat16, 760, 4136),      # 190 blocks: the last span holds two blocks; 17 sets, the last with 40 lines
+    (torch.float16, 40, 8),           # one group of 8 lines
+    (torch.float16, 4096, 2816),      # 256 workgroups, 11 sets
+])
+def test_a_handful_of_tokens_along_the_group_dim_with_16_outputs_per_workgroup(dtype, M, K, T):
+    # 2:4 in the reference's default orientation: every workgroup owns 16 outputs over the whole
+    # reduction, one kernel without matrix instructions; the automatic choice up to 2 tokens
+    print(f"case ostream {dtype} M={M} K={K} T={T}", flush=True)
+    n, m, g = 2, 4, 16
+    W = seeded((M, K), dtype, seed=M + K, std=0.5)
+    Wd, _ = dense_ref(W, n, m, g, 0)
+    w = make(W, n, m, g, 0)
+    x = seeded((T, K), dtype, seed=T)
+    b = seeded((M,), dtype, seed=2)
+    ref = to_np(x).astype(np.float64) @ Wd.T
+    y = sten.spmm(w, x.to(DEV), reduce_dim=1, kernel="ostream")
+    assert rel_l2(to_np(y), ref) <= TOL[dtype]
+    yb = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1, kernel="ostream")
+    assert rel_l2(to_np(yb), ref + to_np(b).astype(np.float64)) <= TOL[dtype]
+    ya = sten.spmm(w, x.to(DEV), b.to(DEV), reduce_dim=1)      # the automatic choice: this kernel or the sliced one
+    assert rel_l2(to_np(ya), ref + to_np(b).astype(np.float64)) <= TOL[dtype]
+    if K % 8 == 0 and T > 1:
+        xs = torch.zeros((2 * T, K + 8), dtype=dtype, device=DEV)[::2, :K]
+        xs.copy_(x.to(DEV))
+        for _ in range(3):
+            assert torch.equal(sten.spmm(w, xs, reduce_dim=1, kernel="ostream"), y)
+    y2 = sten.spmm(w, x.to(DEV), reduce_dim=1, kernel="gstream")      # the sliced kernel agrees
+    assert rel_l2(to_np(y2), to_np(y).astype(np.float64)) <= 2 * TOL[dtype]
+
+
 @pytest.mark.parametrize("T", [1, 16])
 def test_streamed_product_on_blocks_of_eight_at_full_size(T):
     # 8192 x 8192 at 2:8:32 against the dense form, in fp64 on the host
