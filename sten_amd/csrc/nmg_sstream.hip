@@ -16,7 +16,9 @@
 //  * Operand ("lanepack8", written once per weight version by nmg_lanepack8 from the rowpack
 //    operand): for a group of 32 lines and a set of 32 blocks, per row block rb and half a the 64
 //    lanes' shares in lane order -- lp_val [group][set][rb][a][lane][4 blocks][n] values,
-//    lp_pat [group][set][rb][a][lane][4] pattern bytes -- so every load of the kernel is one
+//    lp_pat [group][set][rb][a][lane][4] pattern bytes (4:8) or [group][set][lane] three words of
+//    sixteen 5-bit pattern numbers, (rb, a, e) at bit 5 (f % 6) of word f / 6 with f = 8 rb + 4 a + e
+//    (1:8, 2:8: at most 28 patterns) -- so every load of the kernel is one
 //    contiguous run of 256 bytes to 2 KiB.  Lines beyond the last hold zeros.
 //  * Expansion: a table in LDS gives per pattern the four byte selectors (V_PERM_B32) that spread
 //    the block's value words over the four words of the fragment: one LDS read and four vector
@@ -40,6 +42,7 @@ namespace nmg {
 typedef _Float16 ss_f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 ss_bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t ss_u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t ss_u32x3 __attribute__((ext_vector_type(3)));
 
 template <typename T> struct SsMfma;
 template <> struct SsMfma<__half> {
@@ -97,9 +100,10 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
     const uint32_t s_lo = min((uint32_t)wave * P.sets_per_wave, total_sets);
     const uint32_t nsets = min(s_lo + P.sets_per_wave, total_sets) - s_lo;
     // a set of the operand: [rb][a][lane] shares of PB / 4 bytes
-    constexpr uint32_t VSET = 4 * 64 * PB, PSET = 4 * 64 * 4;
+    constexpr bool PK5 = N <= 2;             // pattern numbers in 5 bits, sixteen per lane and set in three words
+    constexpr uint32_t VSET = 4 * 64 * PB, PSET = PK5 ? 64 * 12 : 4 * 64 * 4;
     const unsigned char *vwave = P.lp_val + (group * total_sets + (nsets ? s_lo : 0)) * VSET + rb0 * (2 * 64 * PB);
-    const unsigned char *pwave = P.lp_pat + (group * total_sets + (nsets ? s_lo : 0)) * PSET + rb0 * (2 * 64 * 4);
+    const unsigned char *pwave = P.lp_pat + (group * total_sets + (nsets ? s_lo : 0)) * PSET + (PK5 ? 0 : rb0 * (2 * 64 * 4));
     const unsigned char *xwave = P.x + (int64_t)(nsets ? s_lo : 0) * 32 * 16;
     const bool tok_live = i < P.T;
     const uint32_t x_lane = (tok_live ? (uint32_t)(i * P.ldx * 2) : 0u) + (uint32_t)kq * 16;
@@ -110,7 +114,8 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
 
     struct Regs {
         VT vals[RBN][2][VL];    // [row block][half set][load]
-        uint32_t pats[RBN][2];
+        uint32_t pats[RBN][2];  // (4:8) a word of four pattern bytes per (row block, half set)
+        ss_u32x3 pk;            // (1:8, 2:8) the lane's sixteen 5-bit pattern numbers of the set
         u32x4 xf[2][4];         // [half set][block of the lane]
         uint32_t xmask;
     } rs[1];
@@ -136,8 +141,13 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
                     for (int v = 0; v < VL; v++)
                         asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2" : "=v"(R.vals[rb][a][v]) : "v"(vo + 16 * v), "s"(vwave) : "memory");
                 }
-                asm volatile("s_nop 4\n\tglobal_load_dword %0, %1, %2" : "=v"(R.pats[rb][a]) : "v"(po), "s"(pwave) : "memory");
+                if constexpr (!PK5)
+                    asm volatile("s_nop 4\n\tglobal_load_dword %0, %1, %2" : "=v"(R.pats[rb][a]) : "v"(po), "s"(pwave) : "memory");
             }
+        if constexpr (PK5) {
+            const uint32_t po = in_range ? rel * PSET + (uint32_t)lane * 12 : 0u;
+            asm volatile("s_nop 4\n\tglobal_load_dwordx3 %0, %1, %2" : "=v"(R.pk) : "v"(po), "s"(pwave) : "memory");
+        }
 #pragma unroll
         for (int a = 0; a < 2; a++)
 #pragma unroll
@@ -153,20 +163,22 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
     "+v"(R.xf[0][0]), "+v"(R.xf[0][1]), "+v"(R.xf[0][2]), "+v"(R.xf[0][3]), "+v"(R.xf[1][0]), "+v"(R.xf[1][1]), \
         "+v"(R.xf[1][2]), "+v"(R.xf[1][3])
 #define NMG_SS_P(R, rb) "+v"(R.pats[rb][0]), "+v"(R.pats[rb][1])
+#define NMG_SS_K(R) "+v"(R.pk)
 #define NMG_SS_V0(R, rb) "+v"(R.vals[rb][0][0]), "+v"(R.vals[rb][1][0])
 #define NMG_SS_V1(R, rb) "+v"(R.vals[rb][0][VL - 1]), "+v"(R.vals[rb][1][VL - 1])
     // the set has landed (every register of the set is named exactly once: a register named twice
     // would be copied)
     auto landed = [&](Regs &R) __attribute__((always_inline)) {
-        if constexpr (RBN == 2 && VL == 1)
-            asm volatile("s_waitcnt vmcnt(0)" : NMG_SS_V0(R, 0), NMG_SS_V0(R, 1), NMG_SS_P(R, 0), NMG_SS_P(R, 1), NMG_SS_X(R) : : "memory");
+        if constexpr (PK5 && RBN == 2)
+            asm volatile("s_waitcnt vmcnt(0)" : NMG_SS_V0(R, 0), NMG_SS_V0(R, 1), NMG_SS_K(R), NMG_SS_X(R) : : "memory");
+        else if constexpr (PK5)
+            asm volatile("s_waitcnt vmcnt(0)" : NMG_SS_V0(R, 0), NMG_SS_K(R), NMG_SS_X(R) : : "memory");
         else if constexpr (RBN == 2)
             asm volatile("s_waitcnt vmcnt(0)" : NMG_SS_V0(R, 0), NMG_SS_V0(R, 1), NMG_SS_V1(R, 0), NMG_SS_V1(R, 1), NMG_SS_P(R, 0), NMG_SS_P(R, 1), NMG_SS_X(R) : : "memory");
-        else if constexpr (VL == 1)
-            asm volatile("s_waitcnt vmcnt(0)" : NMG_SS_V0(R, 0), NMG_SS_P(R, 0), NMG_SS_X(R) : : "memory");
         else
             asm volatile("s_waitcnt vmcnt(0)" : NMG_SS_V0(R, 0), NMG_SS_V1(R, 0), NMG_SS_P(R, 0), NMG_SS_X(R) : : "memory");
     };
+    static_assert(PK5 == (VL == 1), "the lists above: one load of values per share with 5-bit patterns, two at 4:8");
 
     // The first set is requested before anything else happens (a wavefront without sets requests a
     // stand-in, so that the code up to the first wait is the same for all).
@@ -206,6 +218,19 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
         else return v[w / 4][w % 4];
     };
     auto multiply_set = [&](const Regs &R) __attribute__((always_inline)) {
+        // the workgroup's pattern numbers from bit 0 on, six per word (a workgroup of 16 lines takes
+        // the upper eight of the lane's sixteen: fields 8 .. 15 lie from bit 10 of word 1 on)
+        uint32_t q[3] = {0u, 0u, 0u};
+        if constexpr (PK5) {
+            if (RBN == 2 || rb0 == 0) {
+                q[0] = R.pk[0];
+                q[1] = R.pk[1];
+                q[2] = R.pk[2];
+            } else {
+                q[0] = (R.pk[1] >> 10) | ((R.pk[2] & 0x3ffu) << 20);
+                q[1] = (R.pk[2] >> 10) & 0x3ffu;
+            }
+        }
 #pragma unroll
         for (int a = 0; a < 2; a++)
 #pragma unroll
@@ -213,7 +238,13 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
                 const u32x4 xm = R.xf[a][e] & R.xmask;
 #pragma unroll
                 for (int rb = 0; rb < RBN; rb++) {
-                    const uint32_t p = (R.pats[rb][a] >> (8 * e)) & 0xffu;
+                    uint32_t p;
+                    if constexpr (PK5) {
+                        const int f = 8 * rb + 4 * a + e;
+                        p = (q[f / 6] >> (5 * (f % 6))) & 31u;
+                    } else {
+                        p = (R.pats[rb][a] >> (8 * e)) & 0xffu;
+                    }
                     const u32x4 sel = *(const u32x4 *)&tab[((N == 1 ? (e & 1) * P.c : 0) + p) * 4];
                     // the block's value words: n = 2: word e; n = 4: words 2 e, 2 e + 1; n = 1: word e / 2
                     uint32_t lo, hi;
@@ -254,6 +285,7 @@ __global__ __launch_bounds__(SS_WAVES * 64) void sstream_kernel(SStream P)
     }
 #undef NMG_SS_X
 #undef NMG_SS_P
+#undef NMG_SS_K
 #undef NMG_SS_V0
 #undef NMG_SS_V1
 
@@ -305,7 +337,29 @@ __global__ __launch_bounds__(256) void lanepack8_kernel(LanePack P)
         for (int j = 0; j < P.n; j++) P.lp_val[(sh * 4 + e) * P.n + j] = live ? P.pk_val[src * P.n + j] : (uint16_t)0;
         pats |= (live ? (uint32_t)P.pk_pat[src] : 0u) << (8 * e);
     }
-    ((uint32_t *)P.lp_pat)[sh] = pats;
+    if (P.n == 4) ((uint32_t *)P.lp_pat)[sh] = pats;
+}
+
+// 1:8, 2:8: the sixteen pattern numbers of a lane and set in 5 bits each, six per word --
+// one thread per (group, set, lane)
+__global__ __launch_bounds__(256) void lanepack8_pat5_kernel(LanePack P)
+{
+    const int64_t rec = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (rec >= P.shares / 4) return;
+    const int lane = (int)(rec & 63), i = lane & 15, kq = lane >> 4;
+    const int64_t gs = rec >> 6, group = gs / P.sets, set = gs - group * P.sets;
+    uint32_t w[3] = {0u, 0u, 0u};
+    for (int f = 0; f < 16; f++) {
+        const int rb = f >> 3, a = (f >> 2) & 1, e = f & 3;
+        const int64_t line = group * SS_LINES + rb * 16 + i;
+        const int64_t blk = set * 32 + 16 * a + 4 * e + kq;
+        const uint32_t p = line < P.G ? (uint32_t)P.pk_pat[line * P.nb + blk] : 0u;
+        w[f / 6] |= p << (5 * (f % 6));
+    }
+    uint32_t *dst = (uint32_t *)P.lp_pat + rec * 3;
+    dst[0] = w[0];
+    dst[1] = w[1];
+    dst[2] = w[2];
 }
 
 }  // namespace nmg
@@ -321,7 +375,7 @@ extern "C" int nmg_lanepack8_sizes(int64_t G, int64_t S, int n, int64_t *val_ele
     NMG_REQUIRE(S % 256 == 0, NMG_ERR_UNSUPPORTED, "the operand holds whole sets of 32 blocks: S must be a multiple of 256");
     const int64_t shares = ((G + SS_LINES - 1) / SS_LINES) * (S / 256) * 4 * 64;
     *val_elems = shares * 4 * n;
-    *pat_bytes = shares * 4;
+    *pat_bytes = n == 4 ? shares * 4 : shares * 3;      // a word per share, or three words per lane and set
     return NMG_OK;
 }
 
@@ -347,6 +401,9 @@ extern "C" int nmg_lanepack8(const void *d_pk_val, const void *d_pk_pat, int64_t
     const int64_t blocks = (P.shares + 255) / 256;
     NMG_REQUIRE(blocks <= 0x7fffffffLL, NMG_ERR_UNSUPPORTED, "weight too large for one launch");
     hipLaunchKernelGGL(lanepack8_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, P);
+    if (n != 4)
+        hipLaunchKernelGGL(lanepack8_pat5_kernel, dim3((unsigned)((P.shares / 4 + 255) / 256)), dim3(256), 0,
+                           (hipStream_t)stream, P);
     NMG_HIP_TRY(hipGetLastError());
     return NMG_OK;
 }
