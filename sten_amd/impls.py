@@ -55,8 +55,9 @@ def _dense_product(form, x, a):
     """Dense product on this library's matrix-core kernels, operands as they lie in memory:
     ``"tn"``: x [K, T], a [K, O] -> x^T @ a (``nmg_gemm_tn``);  ``"nt"``: x [T, K], a [O, K] -> x @ a^T
     (``nmg_gemm_nt``).  fp32 always; 16-bit types where the kernels take the shape (extents and
-    pitches that are multiples of 8, 16-byte aligned bases; ``"nt"``: K a multiple of 64) -- what
-    they do not take goes to ``torch.mm``."""
+    pitches that are multiples of 8, 16-byte aligned bases; ``"nt"``: K a multiple of 64) -- other
+    16-bit shapes go through the fp32 kernel (operands widened, result rounded once); only what
+    that does not take either (double, more than 2 097 120 tokens) goes to ``torch.mm``."""
     dt = x.dtype
     if form == "tn":
         (K, T), O = x.shape, a.shape[1]
@@ -73,7 +74,12 @@ def _dense_product(form, x, a):
             ok = ok and T % 8 == 0
         else:
             ok = ok and K % 64 == 0 and O * a.stride(0) * 2 < 2 ** 31 and T * x.stride(0) * 2 < 2 ** 31
+    if ok and dt == torch.float32:
+        ok = (T + 31) // 32 <= 65535
     if not ok:
+        if (x.is_cuda and a.dtype == dt and dt in (torch.float16, torch.bfloat16) and T > 0 and O > 0 and K > 0
+                and (T + 31) // 32 <= 65535):
+            return _dense_product(form, x.float(), a.float()).to(dt)
         return torch.mm(x.t(), a) if form == "tn" else torch.mm(x, a.t())
     entry = native.load().nmg_gemm_tn if form == "tn" else native.load().nmg_gemm_nt
     y = torch.empty((T, O), dtype=dt, device=x.device)

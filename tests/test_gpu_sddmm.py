@@ -258,18 +258,23 @@ def test_dense_weight_gradient_in_16_bit(dtype, R, C, T, bias):
     assert bool((buf[:, C:] == 7.0).all()), "wrote beyond the rows of the result"
 
 
-def test_default_gradient_format_takes_no_library_gemm(monkeypatch):
+@pytest.mark.parametrize("fin,fout,tokens", [
+    (256, 384, 72),
+    (250, 380, 37),     # extents that the 16-bit kernels do not take: widened, through the fp32 kernel
+])
+def test_default_gradient_format_takes_no_library_gemm(monkeypatch, fin, fout, tokens):
     # F.linear backward with the default (dense) weight-gradient format in fp16: forward, grad_input and
     # the dense dY^T X all run on this library's kernels -- torch.mm must not be called
+    print(f"case default grad format {fin}->{fout} x {tokens}", flush=True)
     torch.manual_seed(0)
-    lin = torch.nn.Linear(256, 384, bias=True).half().to(DEV)
+    lin = torch.nn.Linear(fin, fout, bias=True).half().to(DEV)
     sb = sten.SparsityBuilder()
     sb.set_weight("weight", initial_sparsifier=sten.GroupedNMSparsifier(2, 4, 16, sparse_dim=1, group_dim=0),
                   out_format=sten.GroupedNMTensor)
     sp = sb.get_sparse_model(lin)
     Wd = sp.weight.wrapped_tensor.to_dense().detach().float()
-    x = torch.randn(72, 256, device=DEV).half().requires_grad_(True)
-    gy = torch.randn(72, 384, device=DEV).half()
+    x = torch.randn(tokens, fin, device=DEV).half().requires_grad_(True)
+    gy = torch.randn(tokens, fout, device=DEV).half()
 
     def no_mm(*a, **k):
         raise AssertionError("torch.mm was called in the backward of the sparse linear")
