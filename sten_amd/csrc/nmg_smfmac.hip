@@ -1167,7 +1167,7 @@ template <typename T> static int launch_smfmac(SmfParams &P, int variant, hipStr
         // vector caches and is 2-4 % faster per flop in steady state (16384 x 4096 x 4096 tokens:
         // 267 against 273 us; 8192^2 x 4096, 2:8: 250 against 260); what decides is how the tiles
         // fill the chip: rounds of 256 tiles, a 256 x 256 tile taking twice the time of a 256 x 128
-        // one (two of which share a CU when there are more than 256).
+        // one (both are one workgroup per CU: 260 and 448 registers per lane).
         const int64_t tm = (P.M + 255) / 256, t256 = tm * ((P.T + 255) / 256), t128 = tm * ((P.T + 127) / 128);
         const double cost128 = (double)((t128 + 255) / 256), cost256 = (double)((t256 + 255) / 256) * 2.0 / 1.025;
         variant = (P.ksplit <= 1 && cost256 < cost128) ? 8 : 6;
