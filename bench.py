@@ -56,6 +56,7 @@ PEAK_HBM_GBS = 8000.0
 SETTLE_S = 0.08                # untimed load before the timed steps (see measure())
 GRAPH_STEPS = 20               # steps per replayed HIP graph (decode shapes)
 FP32_WORKLOADS = ("c1", "ref_f32", "big_f32")
+BF16_WORKLOADS = ("target_2_4_bf16",)
 
 WORKLOADS = {
     # name: (kind, M, K, tokens, n, m, g, description)
@@ -65,6 +66,8 @@ WORKLOADS = {
     "c2": ("fwd", 4096, 4096, 2048, 2, 4, 16, "configs[1]: W 4096x4096 fp16 2:4:16 along K x 2048 tokens, forward"),
     "target_2_4": ("fwd", 4096, 11008, 2048, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 2048 tokens, forward"),
     "target_2_4_4k": ("fwd", 4096, 11008, 4096, 2, 4, 16, "north_star: W 4096x11008 fp16 2:4:16 x 4096 tokens, forward"),
+    # the same product in bf16: three mantissa bits fewer toggle in the multipliers, and the power limit leaves more
+    "target_2_4_bf16": ("fwd", 4096, 11008, 2048, 2, 4, 16, "W 4096x11008 bf16 2:4:16 x 2048 tokens, forward"),
     "target_2_4_64": ("fwd", 4096, 11008, 64, 2, 4, 16, "W 4096x11008 fp16 2:4:16 x 64 tokens, forward (split reduction)"),
     "target_2_4_256": ("fwd", 4096, 11008, 256, 2, 4, 16, "W 4096x11008 fp16 2:4:16 x 256 tokens, forward (split reduction)"),
     "target_2_4_512": ("fwd", 4096, 11008, 512, 2, 4, 16, "W 4096x11008 fp16 2:4:16 x 512 tokens, forward (split reduction)"),
@@ -108,7 +111,7 @@ PMC_SUMMARIES = {
 }
 
 # measured beside the headline workload in the default run: (workload, steps, warm-up)
-ALSO = [("c1", 50, 10), ("ref_f32", 80, 5), ("c2", 240, 10), ("c3_1_8", 40, 5), ("c3_2_8", 40, 5), ("c3_4_8", 40, 5),
+ALSO = [("c1", 50, 10), ("ref_f32", 80, 5), ("target_2_4_bf16", 100, 10), ("c2", 240, 10), ("c3_1_8", 40, 5), ("c3_2_8", 40, 5), ("c3_4_8", 40, 5),
         ("decode_1", 50, 10), ("decode_4", 50, 10), ("decode_8", 50, 10), ("decode_16", 50, 10),
         ("decode_gdim_1", 50, 10), ("decode_gdim_16", 50, 10), ("decode_2_8_1", 50, 10), ("decode_2_8_16", 50, 10),
         ("c4_b1", 50, 10), ("c4_b4", 50, 10), ("c4_b16", 50, 10),
@@ -258,7 +261,7 @@ def measure(workload, steps, warmup, kernel="auto", variant=-1, eager=False, gra
     # copies of it in turn, more than 512 MiB in all.
     copies, turn = 1, [0]
     torch.manual_seed(0)
-    dt = torch.float32 if workload in FP32_WORKLOADS else torch.float16
+    dt = torch.float32 if workload in FP32_WORKLOADS else (torch.bfloat16 if workload in BF16_WORKLOADS else torch.float16)
     W = (torch.randn(M, K) * 0.02).to(dt).to(dev)
 
     if kind in ("step", "train"):
@@ -482,7 +485,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": row["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32" if args.workload in FP32_WORKLOADS else "f16", "data": "synthetic",
+        "dtype": "f32" if args.workload in FP32_WORKLOADS else ("bf16" if args.workload in BF16_WORKLOADS else "f16"), "data": "synthetic",
         "config": {"workload": desc, "kernel": args.kernel, "variant": args.variant, "launch": row["launch"],
                    "settle": f"{row['settle_steps']} more untimed steps ({SETTLE_S * 1e3:.0f} ms of load) between the "
                              "warm-up and the timed steps: the clocks dip for 10-60 ms after an idle spell",
